@@ -1,0 +1,141 @@
+/* lorafusion_hip.h -- C ABI of liblorafusion_hip.so (MI355X / gfx950).
+ *
+ * Drop-in boundary for the `lorafusion.ops` LoRA-linear hot path of CentML/lorafusion.  The
+ * reference's boundary is Python (Triton wrappers); each entry point below names the
+ * reference wrapper it stands in for.  A Python layer (lorafusion_amd/ops) keeps the
+ * reference's call signatures and calls these through ctypes.
+ *
+ * Conventions
+ *  - Every tensor pointer is a DEVICE pointer owned by the caller; tensors are dense row-major.
+ *    `lf_routing` and the `*_ptrs` arrays are HOST memory, read during the call only.
+ *  - dtype: LF_BF16 or LF_F16 for all 16-bit tensors of a call; accumulation is fp32.
+ *  - Return 0 on success, a negative LF_E* code otherwise (lf_strerror gives the text).  The
+ *    library keeps no global mutable state and may be called from several host threads.
+ *  - Work is enqueued on `stream` (a hipStream_t, passed as void*); nothing synchronises.
+ *  - The library allocates nothing: scratch memory comes in through `workspace`
+ *    (size from lf_workspace_bytes), 256-byte aligned.
+ *  - Shape limits: K % 128 == 0, N % 128 == 0, R % 16 == 0, 16 <= R <= 128, rank_i % 8 == 0,
+ *    at most LF_MAX_SEG adapter segments per call, routing block size 128.
+ *
+ * Notation: X [M,K], W [N,K], A_i [r_i,K], B_i [N,r_i], S [M,R] = drop(X) A^T (1/(1-p) applied,
+ * zero beyond rank_i and in padded rows), dS [M,R] = scale dY B, mask uint8 [M,K] keep-mask
+ * (non-zero = keep), R = max rank rounded up to 16.
+ */
+#ifndef LORAFUSION_HIP_H
+#define LORAFUSION_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LF_OK 0
+#define LF_EINVAL (-1)
+#define LF_ESHAPE (-2)
+#define LF_EWORKSPACE (-3)
+#define LF_ELAUNCH (-4)
+#define LF_ELIMIT (-5)
+
+#define LF_BF16 0
+#define LF_F16 1
+
+#define LF_MAX_SEG 32
+
+/* Routing of token rows to adapters.  Single adapter: n_seg = 1, block_table = NULL, `scale`
+ * and `p` apply to all M rows.  Multi-LoRA: the per-block tables built by
+ * prepare_multi_lora_batch_info (lorafusion/ops/multi_lora.py:348-453): block_table[b] =
+ * (rank, valid_rows, first_block_of_segment); segment s owns blocks
+ * [seg_first_block[s], seg_first_block[s+1]) and M must equal n_blocks * block_size_m. */
+typedef struct lf_routing {
+  int32_t n_seg;
+  int32_t block_size_m;
+  int32_t n_blocks;
+  int32_t reserved;
+  const int32_t* block_table; /* device int32 [n_blocks,3] or NULL */
+  const float* block_scale;   /* device f32 [n_blocks] */
+  const float* block_p;       /* device f32 [n_blocks] */
+  float scale;
+  float p;
+  int32_t seg_first_block[LF_MAX_SEG];
+  int32_t seg_rank[LF_MAX_SEG];
+} lf_routing;
+
+#define LF_OP_XA 0
+#define LF_OP_DYS_DYB 1
+#define LF_OP_DA 2
+#define LF_OP_FWD 3
+#define LF_OP_BWD 4
+
+int lf_version(void);
+const char* lf_strerror(int code);
+size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* routing);
+
+/* S = drop(X) A^T.  Stands in for seeded_dropout + `masked_scaled_x @ lora_a.T`
+ * (lorafusion/ops/lora_v1.py:111-119) and fused_dropout_matmul
+ * (lorafusion/ops/triton_ops/fused_dropout_matmul.py:280-354); multi-LoRA: the `full_s` product
+ * (lorafusion/ops/multi_lora.py:481-513).  mask may be NULL (no dropout). */
+int lf_lora_xa(const void* X, const uint8_t* mask, const void* const* a_ptrs, void* S, void* workspace,
+               size_t ws_bytes, int M, int K, int R, const lf_routing* routing, int dtype, void* stream);
+
+/* Y = X W^T + scale * S B^T + bias.  Stands in for fused_lora_xw_sb / fused_lora_xw_sb_tma
+ * (lorafusion/ops/triton_ops/fused_lora_xw_sb.py:209-316, fused_lora_xw_sb_tma.py:244-392) and
+ * fused_multi_lora_xw_sb (fused_multi_lora_xw_sb.py:221-339).  bias may be NULL.  With S = NULL
+ * the LoRA term is skipped (plain GEMM). */
+int lf_lora_xw_sb(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs,
+                  void* Y, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream);
+
+/* dS = scale dY B  and  dB_i = scale dY^T S over segment i.  Stands in for fused_lora_dys_dyb
+ * (lorafusion/ops/triton_ops/fused_lora_dys_dyb.py:182-301) and fused_multi_lora_dys_dyb
+ * (fused_multi_lora_dys_dyb.py:188-321).  Sums are two-stage and deterministic. */
+int lf_lora_dys_dyb(const void* dY, const void* S, const void* const* b_ptrs, void* dS, void* const* db_ptrs,
+                    void* workspace, size_t ws_bytes, int M, int N, int R, const lf_routing* routing, int dtype,
+                    void* stream);
+
+/* dA_i = dS^T drop(X) over segment i.  Stands in for `ds.T @ masked_scaled_x`
+ * (lorafusion/ops/lora_v1.py:153, lorafusion/ops/multi_lora.py:576-581). */
+int lf_lora_da(const void* X, const uint8_t* mask, const void* dS, void* const* da_ptrs, void* workspace,
+               size_t ws_bytes, int M, int K, int R, const lf_routing* routing, int dtype, void* stream);
+
+/* dX = dY W + where(mask, (dS A)/(1-p), 0).  Stands in for fused_lora_dyw_dsa(_tma)
+ * (lorafusion/ops/triton_ops/fused_lora_dyw_dsa.py:184-297) and fused_multi_lora_dyw_dsa
+ * (fused_multi_lora_dyw_dsa.py:188-305).  mask is [M,K]; NULL or p == 0 means no dropout. */
+int lf_lora_dyw_dsa(const void* dY, const void* W, const void* dS, const void* const* a_ptrs, const uint8_t* mask,
+                    void* dX, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream);
+
+/* Whole forward: lf_lora_xa then lf_lora_xw_sb.  Stands in for _fused_linear_lora_forward
+ * (lorafusion/ops/lora_v1.py:87-129) and _fused_linear_multi_lora_forward
+ * (lorafusion/ops/multi_lora.py:456-536).  S_out [M,R] is the tensor to keep for backward. */
+int lf_lora_fwd(const void* X, const void* W, const void* bias, const uint8_t* mask, const void* const* a_ptrs,
+                const void* const* b_ptrs, void* Y, void* S_out, void* workspace, size_t ws_bytes, int M, int N,
+                int K, int R, const lf_routing* routing, int dtype, void* stream);
+
+/* Whole backward: lf_lora_dys_dyb, lf_lora_da, and (dX != NULL) lf_lora_dyw_dsa.  Stands in
+ * for _fused_linear_lora_backward (lorafusion/ops/lora_v1.py:132-166) and
+ * _fused_linear_multi_lora_backward (lorafusion/ops/multi_lora.py:539-599).  dS_out [M,R] is
+ * scratch owned by the caller. */
+int lf_lora_bwd(const void* dY, const void* X, const void* W, const uint8_t* mask, const void* S,
+                const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
+                void* const* db_ptrs, void* dS_out, void* workspace, size_t ws_bytes, int M, int N, int K, int R,
+                const lf_routing* routing, int dtype, void* stream);
+
+/* C = A op(B) (+bias): trans_b = 1: B is [N,K] (C = A B^T); trans_b = 0: B is [K,N].  The same
+ * MFMA kernel as above without the LoRA term; used to time the plain base GEMMs.  tile_cfg
+ * = -1 lets the library choose. */
+int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int N, int K, int trans_b, int dtype,
+            int tile_cfg, void* stream);
+
+/* NF4 block dequantisation.  Stands in for dequantize_nf4_triton
+ * (lorafusion/ops/triton_ops/dequantize_nf4.py:271-346).  packed: uint8 [n/2] (element 2i in the
+ * high nibble of byte i); absmax: uint8 [n/blocksize] when blocksize2 > 0 (double quantised:
+ * absmax = fma(code2[absmax[b]], absmax2[b / blocksize2], offset)), else float32
+ * [n/blocksize]; out: 16-bit [n]. */
+int lf_nf4_dequant(const uint8_t* packed, const void* absmax, const float* code2, const float* absmax2,
+                   const float* offset, void* out, int64_t n_elems, int blocksize, int blocksize2, int out_dtype,
+                   void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LORAFUSION_HIP_H */

@@ -1,0 +1,159 @@
+"""ctypes binding of liblorafusion_hip.so (the C ABI declared in include/lorafusion_hip.h).
+
+There is no fallback: if the shared library is missing, ``lib()`` raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Sequence
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblorafusion_hip.so")
+
+LF_BF16, LF_F16 = 0, 1
+LF_MAX_SEG = 32
+LF_OP_XA, LF_OP_DYS_DYB, LF_OP_DA, LF_OP_FWD, LF_OP_BWD = range(5)
+
+EXPORTS = (
+    "lf_version", "lf_strerror", "lf_workspace_bytes", "lf_lora_xa", "lf_lora_xw_sb", "lf_lora_dys_dyb",
+    "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant",
+)
+
+
+class Routing(ctypes.Structure):
+    """struct lf_routing."""
+
+    _fields_ = [
+        ("n_seg", ctypes.c_int32),
+        ("block_size_m", ctypes.c_int32),
+        ("n_blocks", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+        ("block_table", ctypes.c_void_p),
+        ("block_scale", ctypes.c_void_p),
+        ("block_p", ctypes.c_void_p),
+        ("scale", ctypes.c_float),
+        ("p", ctypes.c_float),
+        ("seg_first_block", ctypes.c_int32 * LF_MAX_SEG),
+        ("seg_rank", ctypes.c_int32 * LF_MAX_SEG),
+    ]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load the HIP library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} not found: build it with `python -m lorafusion_amd.csrc.build` "
+            "(hipcc, gfx950). There is no non-HIP fallback."
+        )
+    l = ctypes.CDLL(LIB_PATH)
+    vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    rp = ctypes.POINTER(Routing)
+    l.lf_version.restype = i
+    l.lf_strerror.restype = ctypes.c_char_p
+    l.lf_strerror.argtypes = [i]
+    l.lf_workspace_bytes.restype = sz
+    l.lf_workspace_bytes.argtypes = [i, i, i, i, i, rp]
+    l.lf_lora_xa.argtypes = [vp, vp, vp, vp, vp, sz, i, i, i, rp, i, vp]
+    l.lf_lora_xw_sb.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, rp, i, vp]
+    l.lf_lora_dys_dyb.argtypes = [vp, vp, vp, vp, vp, vp, sz, i, i, i, rp, i, vp]
+    l.lf_lora_da.argtypes = [vp, vp, vp, vp, vp, sz, i, i, i, rp, i, vp]
+    l.lf_lora_dyw_dsa.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, rp, i, vp]
+    l.lf_lora_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, rp, i, vp]
+    l.lf_lora_bwd.argtypes = [vp] * 12 + [sz, i, i, i, i, rp, i, vp]
+    l.lf_gemm.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, vp]
+    l.lf_nf4_dequant.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, i, i, i, vp]
+    for name in EXPORTS:
+        if name not in ("lf_strerror", "lf_workspace_bytes"):
+            getattr(l, name).restype = i
+    _lib = l
+    return l
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what} failed: {lib().lf_strerror(rc).decode()} (code {rc})")
+
+
+def dtype_id(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return LF_BF16
+    if dtype == torch.float16:
+        return LF_F16
+    raise ValueError(f"Unsupported dtype: {dtype}; expected torch.bfloat16 or torch.float16.")
+
+
+def ptr(t: torch.Tensor | None):
+    return None if t is None else t.data_ptr()
+
+
+def ptr_array(tensors: Sequence[torch.Tensor]):
+    arr = (ctypes.c_void_p * len(tensors))()
+    for k, t in enumerate(tensors):
+        arr[k] = t.data_ptr()
+    return arr
+
+
+def stream_of(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got device {t.device}); the HIP kernels have no CPU path.")
+
+
+def workspace(nbytes: int, device) -> torch.Tensor | None:
+    """Scratch memory for one call (torch's caching allocator keeps this cheap and stream-safe)."""
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def single_routing(rank: int, scale: float, p: float) -> Routing:
+    r = Routing()
+    r.n_seg = 1
+    r.block_size_m = 128
+    r.n_blocks = 0
+    r.block_table = None
+    r.block_scale = None
+    r.block_p = None
+    r.scale = float(scale)
+    r.p = float(p)
+    r.seg_first_block[0] = 0
+    r.seg_rank[0] = int(rank)
+    return r
+
+
+def multi_routing(padded_seq_len_list, rank_list, block_table, block_scale, block_p, block_size_m: int) -> Routing:
+    if len(padded_seq_len_list) > LF_MAX_SEG:
+        raise ValueError(f"At most {LF_MAX_SEG} adapter segments per call, got {len(padded_seq_len_list)}.")
+    r = Routing()
+    r.n_seg = len(padded_seq_len_list)
+    r.block_size_m = int(block_size_m)
+    r.n_blocks = int(block_table.shape[0])
+    r.block_table = block_table.data_ptr()
+    r.block_scale = block_scale.data_ptr()
+    r.block_p = block_p.data_ptr()
+    r.scale = 1.0
+    r.p = 0.0
+    fb = 0
+    for k, (padded, rank) in enumerate(zip(padded_seq_len_list, rank_list, strict=True)):
+        r.seg_first_block[k] = fb
+        r.seg_rank[k] = int(rank)
+        fb += int(padded) // int(block_size_m)
+    return r
+
+
+def round_rank(max_rank: int) -> int:
+    """Columns of S / dS: the largest rank rounded up to the MFMA k-step of 16."""
+    return (int(max_rank) + 15) // 16 * 16

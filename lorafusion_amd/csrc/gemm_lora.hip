@@ -1,0 +1,375 @@
+// MFMA GEMM with a LoRA term seeded into the accumulator, for gfx950 (MI355X).
+//
+//   C[M,N] = A[M,K] * op(B) + mult * (L[M,R] * Rop) (+ bias)
+//
+// NT (forward,  Y  = X W^T + scale * S B^T + bias):  B = W [N,K], Rop rows = B_lora [N,rank]
+// NN (backward, dX = dY W + mask * (dS A)/(1-p)):     B = W [K,N] (W is [N_out,K_in] and the
+//     contraction runs over N_out), Rop = A_lora [rank, N]
+//
+// This replaces the Triton kernels fused_lora_xw_sb / fused_multi_lora_xw_sb
+// (lorafusion/ops/triton_ops/fused_lora_xw_sb.py:74-206, fused_multi_lora_xw_sb.py:66-218) and
+// fused_lora_dyw_dsa / fused_multi_lora_dyw_dsa (fused_lora_dyw_dsa.py:69-181,
+// fused_multi_lora_dyw_dsa.py:60-185).  As there, the accumulator starts from the LoRA product
+// and the dense K-loop adds on top of it in fp32.
+//
+// Structure: one workgroup per BMxBN tile, 64-wide wavefronts each owning a WMxWN sub-tile of
+// 32x32x16 MFMA blocks; BK = 64.  Both operand tiles go global -> LDS with 16-byte
+// direct-to-LDS loads (no VGPR staging), double buffered, one barrier per K step.  LDS rows
+// are XOR-swizzled in 16-byte granules so that the ds_read_b128 fragment reads are bank
+// conflict free; the swizzle is applied on the global side of the direct load (each lane
+// picks the granule whose LDS slot it owns).  The NN operand is stored untransposed and read
+// with ds_read_b64_tr_b16, which hands each lane four consecutive contraction elements of
+// its column.  MFMA operands are swapped (B fragment as the "a" operand) so each lane ends
+// with four consecutive output columns of one row and stores 8 bytes at a time.
+#include "lf_common.h"
+
+namespace {
+
+constexpr int BK = 64;
+
+template <typename T> struct MfmaOp;
+template <> struct MfmaOp<__bf16> {
+  static __device__ __forceinline__ lf_f32x16 run(lf_u32x4 a, lf_u32x4 b, lf_f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(lf_bf16x8, a), __builtin_bit_cast(lf_bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t bits) { return __builtin_bit_cast(float, (uint32_t)bits << 16); }
+};
+template <> struct MfmaOp<_Float16> {
+  static __device__ __forceinline__ lf_f32x16 run(lf_u32x4 a, lf_u32x4 b, lf_f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(lf_f16x8, a), __builtin_bit_cast(lf_f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+};
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+__device__ __forceinline__ void load_g2l_16(const void* g, char* lds_wave_base) {
+  // 16 bytes per lane, global -> LDS; the LDS destination is lds_wave_base + lane*16.
+  __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_wave_base, 16, 0, 0);
+}
+
+template <typename T, int BM, int BN, int WM, int WN, bool NN>
+__global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64, 1)
+gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
+  constexpr int NWM = BM / WM, NWN = BN / WN, NTHREADS = NWM * NWN * 64;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_STAGE = BM * BK * 2, B_STAGE = BN * BK * 2;
+  constexpr int NLA = BM * 8 / NTHREADS;  // 16-byte loads per thread per A tile
+  constexpr int NLB = BN * 8 / NTHREADS;
+  static_assert(NLA >= 1 && NLB >= 1 && (NTHREADS / 8) % 8 == 0, "tile/thread shape");
+  constexpr int GPR = BN / 8;             // NN: granules per LDS row of the B tile
+  constexpr int BPITCH = BN * 2;          // NN: bytes per LDS row of the B tile
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  char* ldsA = smem;
+  char* ldsB = smem + 2 * A_STAGE;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / NWN, wn = wave % NWN;
+  const int l32 = lane & 31, q = lane >> 5;
+
+  // ---- tile mapping: XCD-aware (consecutive tiles stay on one XCD's L2) + grouped along M
+  int pid = blockIdx.x;
+  const int total = p.grid_m * p.grid_n;
+  if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+  constexpr int GROUP_M = 8;
+  const int width = GROUP_M * p.grid_n;
+  const int group = pid / width;
+  const int first_m = group * GROUP_M;
+  const int gsz = min(p.grid_m - first_m, GROUP_M);
+  const int pid_m = first_m + (pid % width) % gsz;
+  const int pid_n = (pid % width) / gsz;
+  const int m0 = pid_m * BM, n0 = pid_n * BN;
+
+  const T* __restrict__ A = (const T*)p.A;
+  const T* __restrict__ B = (const T*)p.B;
+
+  // ---- per-thread global source pointers for the direct-to-LDS loads
+  const T* aptr[NLA];
+  const T* bptr[NLB];
+  {
+    const int r8 = (tid >> 3) & 7;
+    const int srcg = (tid & 7) ^ r8;  // swizzle: LDS slot (tid&7) of row r holds granule slot^(r&7)
+#pragma unroll
+    for (int i = 0; i < NLA; i++) {
+      int row = i * (NTHREADS / 8) + (tid >> 3);
+      int gm = min(m0 + row, p.M - 1);
+      aptr[i] = A + (int64_t)gm * p.lda + srcg * 8;
+    }
+    if constexpr (!NN) {
+#pragma unroll
+      for (int i = 0; i < NLB; i++) {
+        int row = i * (NTHREADS / 8) + (tid >> 3);
+        int gn = min(n0 + row, p.N - 1);
+        bptr[i] = B + (int64_t)gn * p.ldb + srcg * 8;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NLB; i++) {
+        int gid = i * NTHREADS + tid;
+        int row = gid / GPR, g = gid % GPR;
+        int srcseg = (g >> 2) ^ (row & 3);
+        int col = min(n0 + (srcseg * 4 + (g & 3)) * 8, p.N - 8);
+        bptr[i] = B + (int64_t)row * p.ldb + col;
+      }
+    }
+  }
+
+  auto issue_loads = [&](int stage) {
+    char* la = ldsA + stage * A_STAGE + wave * 1024;
+    char* lb = ldsB + stage * B_STAGE + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < NLA; i++) {
+      load_g2l_16(aptr[i], la + i * NTHREADS * 16);
+      aptr[i] += BK;
+    }
+#pragma unroll
+    for (int i = 0; i < NLB; i++) {
+      load_g2l_16(bptr[i], lb + i * NTHREADS * 16);
+      if constexpr (!NN) bptr[i] += BK; else bptr[i] += (int64_t)BK * p.ldb;
+    }
+  };
+
+  lf_f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+  issue_loads(0);
+
+  // ---- LoRA term seeds the accumulator (overlaps with the first tile's loads)
+  const int wrow0 = m0 + wm * WM;  // first row of this wave's sub-tile
+  if (p.L != nullptr && wrow0 < p.M) {
+    const T* __restrict__ L = (const T*)p.L;
+    const T* rp = (const T*)seg.ptr[0];
+    int rank = seg.rank[0];
+    float mult = p.mult_mode == 0 ? seg.scale : (seg.p > 0.f ? 1.f / (1.f - seg.p) : 1.f);
+    bool use_mask = p.mask != nullptr && p.mult_mode == 1 && seg.p > 0.f;
+    if (seg.table != nullptr) {
+      int blk = wrow0 / seg.block_size_m;
+      blk = min(blk, seg.n_blocks - 1);
+      rank = seg.table[3 * blk + 0];
+      int fb = seg.table[3 * blk + 2];
+      int s = 0;
+      for (int i = 1; i < seg.n_seg; i++) s = (seg.first_block[i] == fb) ? i : s;
+      rp = (const T*)seg.ptr[s];
+      if (p.mult_mode == 0) {
+        mult = seg.block_scale[blk];
+      } else {
+        float pb = seg.block_p[blk];
+        mult = pb > 0.f ? 1.f / (1.f - pb) : 1.f;
+        use_mask = p.mask != nullptr && pb > 0.f;
+      }
+    }
+    for (int t = 0; t < p.R / 16; t++) {
+      const int r0 = t * 16 + q * 8;
+      lf_u32x4 lf[TM], rf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        int gm = min(wrow0 + i * 32 + l32, p.M - 1);
+        lf[i] = *(const lf_u32x4*)(L + (int64_t)gm * p.R + r0);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        int gn = min(n0 + wn * WN + j * 32 + l32, p.N - 1);
+        lf_u32x4 v = {0, 0, 0, 0};
+        if (r0 < rank) {
+          if constexpr (!NN) {
+            v = *(const lf_u32x4*)(rp + (int64_t)gn * rank + r0);
+          } else {
+            const uint16_t* r16 = (const uint16_t*)rp;
+            uint32_t e[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) e[k] = r16[(int64_t)(r0 + k) * p.N + gn];
+            v[0] = e[0] | (e[1] << 16); v[1] = e[2] | (e[3] << 16);
+            v[2] = e[4] | (e[5] << 16); v[3] = e[6] | (e[7] << 16);
+          }
+        }
+        rf[j] = v;
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(rf[j], lf[i], acc[i][j]);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        acc[i][j] *= mult;
+        if (use_mask) {
+          int gm = min(wrow0 + i * 32 + l32, p.M - 1);
+#pragma unroll
+          for (int jj = 0; jj < 4; jj++) {
+            int gn = min(n0 + wn * WN + j * 32 + jj * 8 + q * 4, p.N - 4);
+            uint32_t mk = *(const uint32_t*)(p.mask + (int64_t)gm * p.ldmask + gn);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              acc[i][j][jj * 4 + e] = ((mk >> (8 * e)) & 0xffu) ? acc[i][j][jj * 4 + e] : 0.f;
+          }
+        }
+      }
+  }
+
+  // ---- per-lane LDS fragment offsets
+  int a_off[TM], b_off[TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++) a_off[i] = (wm * WM + i * 32 + l32) * 128;
+  const int sw = l32 & 7;
+  int btr_key = 0, btr_in = 0;
+  if constexpr (!NN) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) b_off[j] = (wn * WN + j * 32 + l32) * 128;
+  } else {
+    // ds_read_b64_tr_b16: within a 16-lane group, lane 4j+c addresses row j, columns 4c..4c+3 and
+    // receives column (lane&15), rows 0..3.
+    const int grp = lane >> 4, li = lane & 15, j4 = li >> 2, c = li & 3;
+    const int row0 = (grp >> 1) * 8 + j4;
+    btr_key = row0 & 3;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      int colb = (wn * WN + j * 32 + (grp & 1) * 16 + 4 * c) * 2;  // byte offset within the row
+      b_off[j] = row0 * BPITCH + (((colb >> 6) ^ btr_key) << 6) + (colb & 63);
+    }
+    (void)btr_in;
+  }
+
+  auto compute = [&](int stage) {
+    const char* sa = ldsA + stage * A_STAGE;
+    const char* sb = ldsB + stage * B_STAGE;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      lf_u32x4 af[TM], bf[TN];
+      const int slot = ((2 * ks + q) ^ sw) << 4;
+#pragma unroll
+      for (int i = 0; i < TM; i++) af[i] = *(const lf_u32x4*)(sa + a_off[i] + slot);
+      if constexpr (!NN) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) bf[j] = *(const lf_u32x4*)(sb + b_off[j] + slot);
+      } else {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const char* base = sb + b_off[j] + ks * 16 * BPITCH;
+          lf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(base));
+          lf_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(base + 4 * BPITCH));
+          lf_u32x2 lo2 = __builtin_bit_cast(lf_u32x2, lo), hi2 = __builtin_bit_cast(lf_u32x2, hi);
+          bf[j] = lf_u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(bf[j], af[i], acc[i][j]);
+    }
+  };
+
+  const int nk = p.K / BK;
+  __builtin_amdgcn_s_waitcnt(0);  // all counters (encoding 0 = vmcnt/expcnt/lgkmcnt zero)
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt++) {
+    if (kt + 1 < nk) issue_loads((kt + 1) & 1);
+    compute(kt & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: bias, convert, 8-byte stores (4 consecutive columns of one row per lane)
+  T* __restrict__ C = (T*)p.C;
+  const uint16_t* bias16 = (const uint16_t*)p.bias;
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int gm = wrow0 + i * 32 + l32;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+      for (int jj = 0; jj < 4; jj++) {
+        const int gn = n0 + wn * WN + j * 32 + jj * 8 + q * 4;
+        if (gm < p.M && gn < p.N) {
+          float v0 = acc[i][j][jj * 4 + 0], v1 = acc[i][j][jj * 4 + 1];
+          float v2 = acc[i][j][jj * 4 + 2], v3 = acc[i][j][jj * 4 + 3];
+          if (bias16 != nullptr) {
+            v0 += MfmaOp<T>::to_float(bias16[gn + 0]); v1 += MfmaOp<T>::to_float(bias16[gn + 1]);
+            v2 += MfmaOp<T>::to_float(bias16[gn + 2]); v3 += MfmaOp<T>::to_float(bias16[gn + 3]);
+          }
+          lf_u32x2 o = {MfmaOp<T>::pack2(v0, v1), MfmaOp<T>::pack2(v2, v3)};
+          *(lf_u32x2*)(C + (int64_t)gm * p.ldc + gn) = o;
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int BM, int BN, int WM, int WN, bool NN>
+int launch_cfg(LfGemmParams p, const LfSegTable& seg, hipStream_t st) {
+  constexpr int NTHREADS = (BM / WM) * (BN / WN) * 64;
+  constexpr int SMEM = 2 * (BM + BN) * BK * 2;
+  p.grid_m = (p.M + BM - 1) / BM;
+  p.grid_n = (p.N + BN - 1) / BN;
+  auto kern = gemm_lora_kernel<T, BM, BN, WM, WN, NN>;
+  static bool attr_set = false;  // idempotent; a race only repeats the same call
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess) return LF_ELAUNCH;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(p.grid_m * p.grid_n), dim3(NTHREADS), SMEM, st, p, seg);
+  return lf_check_launch();
+}
+
+template <typename T, bool NN>
+int launch_dtype(const LfGemmParams& p, const LfSegTable& seg, int cfg, hipStream_t st) {
+  // Rows of one routing block must not straddle a wave's sub-tile: WM divides block_size_m.
+  switch (cfg) {
+    case 0: return launch_cfg<T, 256, 256, 128, 128, NN>(p, seg, st);
+    case 1: return launch_cfg<T, 256, 256, 128, 64, NN>(p, seg, st);
+    case 2: return launch_cfg<T, 128, 256, 64, 128, NN>(p, seg, st);
+    case 3: return launch_cfg<T, 128, 256, 64, 64, NN>(p, seg, st);
+    case 4: return launch_cfg<T, 128, 128, 64, 64, NN>(p, seg, st);
+    default: return LF_EINVAL;
+  }
+}
+
+}  // namespace
+
+// Tile choice: fewest "rounds" of 256 CUs weighted by tile area (bigger tiles reuse more per
+// LDS byte, but a nearly empty last round wastes the chip).
+static int choose_cfg(int M, int N) {
+  const int bm[5] = {256, 256, 128, 128, 128}, bn[5] = {256, 256, 256, 256, 128};
+  const double eff[5] = {1.00, 0.97, 0.93, 0.90, 0.80};
+  int best = 0;
+  double best_cost = 1e30;
+  for (int c = 0; c < 5; c++) {
+    if (c == 1 || c == 3) continue;  // 8-wave variants are picked only explicitly
+    long tiles = (long)((M + bm[c] - 1) / bm[c]) * ((N + bn[c] - 1) / bn[c]);
+    long rounds = (tiles + 255) / 256;
+    double cost = (double)rounds * bm[c] * bn[c] / eff[c];
+    if (cost < best_cost) { best_cost = cost; best = c; }
+  }
+  return best;
+}
+
+int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st) {
+  if (p.M <= 0 || p.N <= 0 || p.K <= 0) return LF_EINVAL;
+  if (p.K % BK != 0 || p.N % 8 != 0 || p.N < 8) return LF_ESHAPE;
+  if (p.L != nullptr && (p.R % 16 != 0 || p.R <= 0 || p.R > LF_MAX_RANK)) return LF_ESHAPE;
+  if (seg.table != nullptr && (seg.block_size_m % 64 != 0)) return LF_ESHAPE;
+  int cfg = force_cfg >= 0 ? force_cfg : choose_cfg(p.M, p.N);
+  if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1)) cfg = 2;
+  if (dtype == LF_BF16) return nn ? launch_dtype<__bf16, true>(p, seg, cfg, st) : launch_dtype<__bf16, false>(p, seg, cfg, st);
+  if (dtype == LF_F16) return nn ? launch_dtype<_Float16, true>(p, seg, cfg, st) : launch_dtype<_Float16, false>(p, seg, cfg, st);
+  return LF_EINVAL;
+}

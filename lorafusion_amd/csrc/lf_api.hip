@@ -1,0 +1,190 @@
+// extern "C" entry points of liblorafusion_hip.so: argument checks, workspace carving, launches.
+#include "lf_common.h"
+
+int lf_launch_nf4_dequant(const uint8_t*, const void*, const float*, const float*, const float*, void*, int64_t,
+                          int, int, int, hipStream_t);
+int lf_launch_xa(const void*, const uint8_t*, void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
+int lf_launch_dys_dyb(const void*, const void*, void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
+int lf_launch_da(const void*, const uint8_t*, const void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
+size_t lf_xa_workspace(int, int, int, const LfSegTable&);
+size_t lf_dys_dyb_workspace(int, int, int, const LfSegTable&);
+size_t lf_da_workspace(int, int, int, const LfSegTable&);
+
+namespace {
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// Host routing description -> kernel-argument table.
+int make_seg(const lf_routing* r, int M, const void* const* ptrs, void* const* outs, LfSegTable& t) {
+  if (!r) return LF_EINVAL;
+  if (r->n_seg < 1) return LF_EINVAL;
+  if (r->n_seg > LF_MAX_SEG) return LF_ELIMIT;
+  t = LfSegTable{};
+  t.n_seg = r->n_seg;
+  t.block_size_m = r->block_size_m;
+  t.n_blocks = r->n_blocks;
+  t.table = r->block_table;
+  t.block_scale = r->block_scale;
+  t.block_p = r->block_p;
+  t.scale = r->scale;
+  t.p = r->p;
+  if (r->block_table) {
+    if (r->block_size_m != 128) return LF_ESHAPE;
+    if (r->n_blocks < 1 || (int64_t)r->n_blocks * r->block_size_m != M) return LF_ESHAPE;
+    if (!r->block_scale || !r->block_p) return LF_EINVAL;
+  } else {
+    if (r->n_seg != 1) return LF_EINVAL;
+    if (!(r->p >= 0.f && r->p < 1.f)) return LF_EINVAL;
+  }
+  for (int s = 0; s < r->n_seg; s++) {
+    t.first_block[s] = r->seg_first_block[s];
+    t.rank[s] = r->seg_rank[s];
+    t.ptr[s] = ptrs ? ptrs[s] : nullptr;
+    t.out[s] = outs ? outs[s] : nullptr;
+    if (t.rank[s] < 8 || t.rank[s] % 8 != 0 || t.rank[s] > LF_MAX_RANK) return LF_ESHAPE;
+    if (s > 0 && t.first_block[s] <= t.first_block[s - 1]) return LF_EINVAL;
+  }
+  return LF_OK;
+}
+
+bool bad_dtype(int d) { return d != LF_BF16 && d != LF_F16; }
+
+}  // namespace
+
+extern "C" {
+
+int lf_version(void) { return 1; }
+
+const char* lf_strerror(int code) {
+  switch (code) {
+    case LF_OK: return "ok";
+    case LF_EINVAL: return "invalid argument (null pointer, non-positive size, unknown dtype or bad routing)";
+    case LF_ESHAPE: return "shape not supported (need K % 128 == 0, N % 128 == 0, R % 16 == 0, R <= 128, rank % 8 == 0, routing block 128)";
+    case LF_EWORKSPACE: return "workspace missing or too small (see lf_workspace_bytes)";
+    case LF_ELAUNCH: return "HIP reported an error at kernel launch";
+    case LF_ELIMIT: return "too many adapter segments in one call";
+    default: return "unknown error code";
+  }
+}
+
+size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* routing) {
+  LfSegTable t;
+  const void* dummy_ptrs[LF_MAX_SEG] = {};
+  if (make_seg(routing, M, dummy_ptrs, nullptr, t) != LF_OK) return 0;
+  switch (op) {
+    case LF_OP_XA: return align256(lf_xa_workspace(M, K, R, t));
+    case LF_OP_DYS_DYB: return align256(lf_dys_dyb_workspace(M, N, R, t));
+    case LF_OP_DA: return align256(lf_da_workspace(M, K, R, t));
+    case LF_OP_FWD: return align256(lf_xa_workspace(M, K, R, t));
+    case LF_OP_BWD: {
+      size_t a = lf_dys_dyb_workspace(M, N, R, t), b = lf_da_workspace(M, K, R, t);
+      return align256(a > b ? a : b);
+    }
+    default: return 0;
+  }
+}
+
+int lf_lora_xa(const void* X, const uint8_t* mask, const void* const* a_ptrs, void* S, void* workspace,
+               size_t ws_bytes, int M, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  if (bad_dtype(dtype) || !a_ptrs) return LF_EINVAL;
+  LfSegTable t;
+  int rc = make_seg(routing, M, a_ptrs, nullptr, t);
+  if (rc != LF_OK) return rc;
+  for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
+  return lf_launch_xa(X, mask, S, workspace, ws_bytes, M, K, R, t, dtype, (hipStream_t)stream);
+}
+
+int lf_lora_xw_sb(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs,
+                  void* Y, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  if (bad_dtype(dtype) || !X || !W || !Y) return LF_EINVAL;
+  LfSegTable t{};
+  if (S) {
+    if (!b_ptrs) return LF_EINVAL;
+    int rc = make_seg(routing, M, b_ptrs, nullptr, t);
+    if (rc != LF_OK) return rc;
+    for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
+  }
+  if (K % 128 != 0 || N % 128 != 0) return LF_ESHAPE;
+  LfGemmParams p{};
+  p.A = X; p.B = W; p.C = Y; p.bias = bias;
+  p.M = M; p.N = N; p.K = K; p.lda = K; p.ldb = K; p.ldc = N;
+  p.L = S; p.R = R; p.mask = nullptr; p.ldmask = 0; p.mult_mode = 0;
+  return lf_launch_gemm(p, t, /*nn=*/false, dtype, -1, (hipStream_t)stream);
+}
+
+int lf_lora_dys_dyb(const void* dY, const void* S, const void* const* b_ptrs, void* dS, void* const* db_ptrs,
+                    void* workspace, size_t ws_bytes, int M, int N, int R, const lf_routing* routing, int dtype,
+                    void* stream) {
+  if (bad_dtype(dtype) || !b_ptrs || !db_ptrs) return LF_EINVAL;
+  LfSegTable t;
+  int rc = make_seg(routing, M, b_ptrs, db_ptrs, t);
+  if (rc != LF_OK) return rc;
+  return lf_launch_dys_dyb(dY, S, dS, workspace, ws_bytes, M, N, R, t, dtype, (hipStream_t)stream);
+}
+
+int lf_lora_da(const void* X, const uint8_t* mask, const void* dS, void* const* da_ptrs, void* workspace,
+               size_t ws_bytes, int M, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  if (bad_dtype(dtype) || !da_ptrs) return LF_EINVAL;
+  LfSegTable t;
+  int rc = make_seg(routing, M, nullptr, da_ptrs, t);
+  if (rc != LF_OK) return rc;
+  return lf_launch_da(X, mask, dS, workspace, ws_bytes, M, K, R, t, dtype, (hipStream_t)stream);
+}
+
+int lf_lora_dyw_dsa(const void* dY, const void* W, const void* dS, const void* const* a_ptrs, const uint8_t* mask,
+                    void* dX, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  if (bad_dtype(dtype) || !dY || !W || !dX) return LF_EINVAL;
+  LfSegTable t{};
+  if (dS) {
+    if (!a_ptrs) return LF_EINVAL;
+    int rc = make_seg(routing, M, a_ptrs, nullptr, t);
+    if (rc != LF_OK) return rc;
+    for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
+  }
+  if (K % 128 != 0 || N % 128 != 0) return LF_ESHAPE;
+  // dX[M,K] = dY[M,N] * W[N,K]: output columns = K, contraction = N
+  LfGemmParams p{};
+  p.A = dY; p.B = W; p.C = dX; p.bias = nullptr;
+  p.M = M; p.N = K; p.K = N; p.lda = N; p.ldb = K; p.ldc = K;
+  p.L = dS; p.R = R; p.mask = mask; p.ldmask = K; p.mult_mode = 1;
+  return lf_launch_gemm(p, t, /*nn=*/true, dtype, -1, (hipStream_t)stream);
+}
+
+int lf_lora_fwd(const void* X, const void* W, const void* bias, const uint8_t* mask, const void* const* a_ptrs,
+                const void* const* b_ptrs, void* Y, void* S_out, void* workspace, size_t ws_bytes, int M, int N,
+                int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  int rc = lf_lora_xa(X, mask, a_ptrs, S_out, workspace, ws_bytes, M, K, R, routing, dtype, stream);
+  if (rc != LF_OK) return rc;
+  return lf_lora_xw_sb(X, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype, stream);
+}
+
+int lf_lora_bwd(const void* dY, const void* X, const void* W, const uint8_t* mask, const void* S,
+                const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
+                void* const* db_ptrs, void* dS_out, void* workspace, size_t ws_bytes, int M, int N, int K, int R,
+                const lf_routing* routing, int dtype, void* stream) {
+  int rc = lf_lora_dys_dyb(dY, S, b_ptrs, dS_out, db_ptrs, workspace, ws_bytes, M, N, R, routing, dtype, stream);
+  if (rc != LF_OK) return rc;
+  rc = lf_lora_da(X, mask, dS_out, da_ptrs, workspace, ws_bytes, M, K, R, routing, dtype, stream);
+  if (rc != LF_OK) return rc;
+  if (dX) rc = lf_lora_dyw_dsa(dY, W, dS_out, a_ptrs, mask, dX, M, N, K, R, routing, dtype, stream);
+  return rc;
+}
+
+int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int N, int K, int trans_b, int dtype,
+            int tile_cfg, void* stream) {
+  if (bad_dtype(dtype) || !A || !B || !C) return LF_EINVAL;
+  LfSegTable t{};
+  LfGemmParams p{};
+  p.A = A; p.B = B; p.C = C; p.bias = bias;
+  p.M = M; p.N = N; p.K = K; p.lda = K; p.ldb = trans_b ? K : N; p.ldc = N;
+  return lf_launch_gemm(p, t, /*nn=*/!trans_b, dtype, tile_cfg, (hipStream_t)stream);
+}
+
+int lf_nf4_dequant(const uint8_t* packed, const void* absmax, const float* code2, const float* absmax2,
+                   const float* offset, void* out, int64_t n_elems, int blocksize, int blocksize2, int out_dtype,
+                   void* stream) {
+  return lf_launch_nf4_dequant(packed, absmax, code2, absmax2, offset, out, n_elems, blocksize, blocksize2,
+                               out_dtype, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,59 @@
+// Shared declarations for the gfx950 LoRA-linear kernels (internal; the public C ABI is
+// include/lorafusion_hip.h).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/lorafusion_hip.h"  // error codes, dtype ids, LF_MAX_SEG
+
+#define LF_MAX_RANK 128
+
+typedef __bf16 lf_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 lf_f16x8 __attribute__((ext_vector_type(8)));
+typedef float lf_f32x16 __attribute__((ext_vector_type(16)));
+typedef float lf_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t lf_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t lf_u32x2 __attribute__((ext_vector_type(2)));
+typedef short lf_s16x4 __attribute__((ext_vector_type(4)));
+
+// Per-launch routing of token blocks to adapters.  `table` == nullptr means one adapter
+// over all rows (ptr[0], rank[0]); otherwise block b = row / block_size_m has
+// (rank, valid_rows, first_block) = table[3b..3b+2] and belongs to the segment s with
+// first_block[s] == table[3b+2].
+struct LfSegTable {
+  const void* ptr[LF_MAX_SEG];   // per-segment skinny operand (B_i, A_i, ...)
+  void* out[LF_MAX_SEG];         // per-segment output (dA_i, dB_i) where a kernel has one
+  int first_block[LF_MAX_SEG];
+  int rank[LF_MAX_SEG];
+  int n_seg;
+  int block_size_m;
+  int n_blocks;
+  const int32_t* table;          // device int32 [n_blocks,3] or nullptr
+  const float* block_scale;      // device f32 [n_blocks] or nullptr
+  const float* block_p;          // device f32 [n_blocks] or nullptr
+  float scale;                   // used when table == nullptr
+  float p;                       // used when table == nullptr
+};
+
+struct LfGemmParams {
+  const void* A;      // [M,K] row-major, lda
+  const void* B;      // NT: [N,K] row-major; NN: [K,N] row-major; ldb
+  void* C;            // [M,N], ldc
+  const void* bias;   // [N] or nullptr
+  int M, N, K;
+  int64_t lda, ldb, ldc;
+  const void* L;      // [M,R] skinny left operand of the LoRA term (S or dS), or nullptr
+  int R;              // columns of L (multiple of 16)
+  const uint8_t* mask;  // [M,N] keep-mask applied to the LoRA term (dX path) or nullptr
+  int64_t ldmask;
+  int mult_mode;      // 0: LoRA term * scale ; 1: LoRA term * 1/(1-p), masked where p > 0
+  int grid_m, grid_n;
+};
+
+// launchers (one per translation unit)
+int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st);
+
+static inline int lf_check_launch() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? LF_OK : LF_ELAUNCH;
+}

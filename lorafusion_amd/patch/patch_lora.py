@@ -1,0 +1,114 @@
+"""Route PEFT LoRA linear layers through the fused HIP ops.
+
+Same behaviour as lorafusion/patch/patch_lora.py:11-184: ``apply_lora`` replaces
+``peft.tuners.lora.Linear.forward`` with ``lora_forward``, which picks the single- or
+multi-adapter op depending on the ``MultiLoRAManager`` and falls back to the unfused torch
+expressions when ``use_fused=False``.  The layer is duck-typed (``base_layer.weight/.bias``,
+``lora_A/lora_B[name].weight``, ``lora_dropout[name].p``, ``scaling[name]``, ``training``), so
+any module with those attributes works when peft is not installed.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from lorafusion_amd.ops.lora_torch_ref import torch_ref_linear_lora, torch_ref_linear_multi_lora
+from lorafusion_amd.ops.lora_v1 import fused_linear_lora
+from lorafusion_amd.ops.multi_lora import fused_linear_multi_lora, get_multi_lora_manager
+
+try:  # peft is optional
+    from peft.tuners.lora import Linear as LoRALinear
+except Exception:  # noqa: BLE001
+    LoRALinear = None
+
+_REQUIRED_ATTRS = ("base_layer", "lora_A", "lora_B", "lora_dropout", "scaling")
+
+
+def _is_lora_linear(model) -> bool:
+    if LoRALinear is not None and isinstance(model, LoRALinear):
+        return True
+    return all(hasattr(model, a) for a in _REQUIRED_ATTRS)
+
+
+def _cast_input(model, x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    cast = getattr(model, "_cast_input_dtype", None)
+    return cast(x, dtype) if cast is not None else x.to(dtype)
+
+
+def _single(model, x, adapter_key, linear_bias, use_fused):
+    lora_a = model.lora_A[adapter_key].weight
+    lora_b = model.lora_B[adapter_key].weight
+    p = float(getattr(model.lora_dropout[adapter_key], "p", 0.0)) if model.training else 0.0
+    scaling = model.scaling[adapter_key]
+    x = _cast_input(model, x, lora_a.dtype)
+    fn = fused_linear_lora if use_fused else torch_ref_linear_lora
+    return fn(x=x, linear_w=model.base_layer.weight, lora_a=lora_a, lora_b=lora_b, alpha=scaling,
+              dropout_p=p, linear_bias=linear_bias)
+
+
+def lora_forward(model, x: torch.Tensor, *args, use_fused: bool = True, **kwargs) -> torch.Tensor:
+    """Forward of a LoRA linear layer through the fused (or unfused) op."""
+    if not _is_lora_linear(model):
+        raise TypeError(f"model must be a LoRALinear, but got {type(model)}")
+    manager = get_multi_lora_manager()
+    result_dtype = x.dtype
+    linear_bias = getattr(model.base_layer, "bias", None)
+
+    if manager is None:
+        if len(model.lora_A) > 1:
+            raise ValueError("Multi-LoRA is not enabled, but the model has multiple LoRA adapters.")
+        result = _single(model, x, next(iter(model.lora_A.keys())), linear_bias, use_fused)
+        return result.to(result_dtype)
+
+    manager.register_lora_linear(model)
+    info = manager.get_newest_batch_info() if manager.is_in_forward else manager.get_oldest_batch_info()
+    if info is None:
+        raise ValueError("no MultiLoRABatchInfo registered with the manager for this pass")
+    if info.num_active_adapters == 1:
+        result = _single(model, x, f"lora_{info.lora_idx_list[0]}", linear_bias, use_fused)
+        return result.to(result_dtype)
+
+    lora_a_list = [model.lora_A[f"lora_{i}"].weight for i in info.lora_idx_list]
+    lora_b_list = [model.lora_B[f"lora_{i}"].weight for i in info.lora_idx_list]
+    x = _cast_input(model, x, lora_a_list[0].dtype)
+    if use_fused:
+        result = fused_linear_multi_lora(
+            padded_x=x,
+            linear_w=model.base_layer.weight,
+            lora_a_list=lora_a_list,
+            lora_b_list=lora_b_list,
+            seq_len_list=info.seq_len_list,
+            padded_seq_len_list=info.padded_seq_len_list,
+            block_to_lookup_table=info.block_to_lookup_table,
+            block_to_dropout_p=info.block_to_dropout_p,
+            block_to_alpha=info.block_to_alpha,
+            enable_dropout=model.training and info.enable_dropout,
+            same_dropout_p_value=info.same_dropout_p_value,
+            max_r=info.max_r,
+            linear_bias=linear_bias,
+        )
+    else:
+        result = torch_ref_linear_multi_lora(
+            padded_x=x,
+            linear_w=model.base_layer.weight,
+            lora_a_list=lora_a_list,
+            lora_b_list=lora_b_list,
+            seq_len_list=info.seq_len_list,
+            padded_seq_len_list=info.padded_seq_len_list,
+            alpha_list=info.alpha_list,
+            dropout_p_list=[p if model.training else 0.0 for p in info.dropout_p_list],
+            linear_bias=linear_bias,
+        )
+    return result.to(result_dtype)
+
+
+def apply_lora(*, use_fused: bool = True, target_cls=None) -> None:
+    """Replace ``forward`` of peft's LoRA ``Linear`` (or of ``target_cls``) with ``lora_forward``."""
+    cls = target_cls if target_cls is not None else LoRALinear
+    if cls is None:
+        raise ImportError("peft is not installed; pass target_cls=<your LoRA linear class> to apply_lora().")
+
+    def forward_wrapper(self, x: torch.Tensor, *args, **kwargs) -> torch.Tensor:
+        return lora_forward(self, x, *args, use_fused=use_fused, **kwargs)
+
+    cls.forward = forward_wrapper
