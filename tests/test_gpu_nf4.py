@@ -1,0 +1,123 @@
+"""GPU parity: NF4 dequantisation is bit-exact against the C oracle; QLoRA linear within tolerance."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import lora_ref, nf4 as onf4
+from tests.util import single_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _to_state(st: onf4.NF4State, dtype=torch.bfloat16):
+    from lorafusion_amd.ops.nf4 import QuantState, QuantState2
+
+    dev = "cuda"
+    packed = torch.from_numpy(st.packed).to(dev)
+    if st.nested:
+        qs = QuantState(torch.Size(st.shape), dtype, st.blocksize, torch.from_numpy(st.absmax).to(dev),
+                        torch.from_numpy(st.offset).to(dev),
+                        QuantState2(torch.from_numpy(st.absmax2).to(dev), torch.from_numpy(st.code2).to(dev), st.blocksize2))
+    else:
+        qs = QuantState(torch.Size(st.shape), dtype, st.blocksize, torch.from_numpy(st.absmax).to(dev))
+    return packed, qs
+
+
+def _bits(t: torch.Tensor) -> np.ndarray:
+    return t.reshape(-1).view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("shape,bs,nested", [
+    ((64, 256), 64, True), ((128, 1024), 64, True), ((256, 4096), 64, True), ((16, 2048), 128, True),
+    ((8, 64), 64, False), ((3, 1024), 32, False), ((64, 3584), 64, True),
+    ((1, 16384), 64, True),  # one second-level block exactly
+])
+def test_dequant_bit_exact(shape, bs, nested):
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
+
+    rng = np.random.default_rng(hash(shape) % 1000)
+    w = (rng.standard_normal(shape) * 0.02).astype(np.float32)
+    st = onf4.quantize_nf4(w, blocksize=bs, nested=nested)
+    expect = onf4.dequantize(st)
+    packed, qs = _to_state(st)
+    got = dequantize_nf4_triton(packed, qs)
+    assert got.shape == tuple(shape) and got.dtype == torch.bfloat16
+    assert np.array_equal(_bits(got), expect)
+
+
+def test_dequant_all_codes_random_state():
+    """Every 4-bit code against random absmax codes / scales / offset (not from the quantiser)."""
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
+
+    rng = np.random.default_rng(1)
+    n = 256 * 64 * 4
+    st = onf4.NF4State(
+        packed=rng.integers(0, 256, n // 2, dtype=np.uint8), shape=(n,), blocksize=64,
+        absmax=rng.integers(0, 256, n // 64, dtype=np.uint8), code2=onf4.dynamic_code_table(),
+        absmax2=(rng.random(n // 64 // 256) * 0.05 + 1e-3).astype(np.float32),
+        offset=np.asarray([0.0173], dtype=np.float32))
+    packed, qs = _to_state(st)
+    assert np.array_equal(_bits(dequantize_nf4_triton(packed, qs)), onf4.dequantize(st))
+
+
+def test_dequant_fp16_output():
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
+
+    rng = np.random.default_rng(2)
+    st = onf4.quantize_nf4((rng.standard_normal((32, 512)) * 0.02).astype(np.float32))
+    _, f32 = onf4.dequantize(st, want_f32=True)
+    packed, qs = _to_state(st, torch.float16)
+    got = dequantize_nf4_triton(packed, qs)
+    assert np.array_equal(got.reshape(-1).view(torch.int16).cpu().numpy().view(np.uint16),
+                          f32.astype(np.float16).view(np.uint16))
+
+
+def test_dequant_config2_shape_and_roundtrip():
+    """BASELINE configs[2] weight: [14336, 4096], blocksize 64, double quantised.  Bit-exact vs the
+    oracle, and the size-independent property |dequant(quant(w)) - w| <= half the widest code gap * absmax."""
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
+
+    rng = np.random.default_rng(3)
+    w = (rng.standard_normal((14336, 4096)) * 0.02).astype(np.float32)
+    st = onf4.quantize_nf4(w)
+    packed, qs = _to_state(st)
+    got = dequantize_nf4_triton(packed, qs)
+    assert np.array_equal(_bits(got), onf4.dequantize(st))
+    absmax_true = np.abs(w.reshape(-1, 64)).max(axis=1)
+    err = np.abs(got.float().cpu().numpy().reshape(-1, 64) - w.reshape(-1, 64)).max(axis=1)
+    # widest gap in the code is 1.0 - 0.7229568 = 0.277; half of it, plus slack for the 8-bit absmax code and bf16
+    assert (err <= (0.1386 + 0.03) * absmax_true + 1e-6).all()
+
+
+def test_dequant_errors():
+    from lorafusion_amd.ops.nf4 import QuantState, dequantize_nf4_triton
+
+    packed = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    with pytest.raises(ValueError):
+        dequantize_nf4_triton(packed, QuantState(torch.Size([128]), torch.float32, 64, torch.ones(2, device="cuda")))
+    with pytest.raises(ValueError):
+        dequantize_nf4_triton(packed, QuantState(torch.Size([256]), torch.bfloat16, 64, torch.ones(4, device="cuda")))
+    with pytest.raises(ValueError):
+        dequantize_nf4_triton(packed.float(), QuantState(torch.Size([128]), torch.bfloat16, 64, torch.ones(2, device="cuda")))
+
+
+def test_qlora_linear_parity():
+    """NF4 base weight + LoRA fwd/bwd vs the oracle evaluated on the oracle-dequantised weight."""
+    from lorafusion_amd.ops.nf4 import fused_linear_lora_nf4
+
+    M, K, N, r, p, scale = 384, 512, 768, 16, 0.1, 2.0
+    d = single_inputs(M, K, N, r, p=p, seed=9)
+    st = onf4.quantize_nf4(d["w"].float().numpy())
+    wq = torch.from_numpy(onf4.dequantize(st).view(np.int16)).view(torch.bfloat16).reshape(N, K)
+    packed, qs = _to_state(st)
+    x = d["x"].cuda().requires_grad_(True)
+    a = d["a"].cuda().requires_grad_(True)
+    b = d["b"].cuda().requires_grad_(True)
+    y = fused_linear_lora_nf4(x, packed, qs, a, b, scale, dropout_p=p, dropout_mask=d["mask"].cuda())
+    y.backward(d["dy"].cuda())
+    ye, _ = lora_ref.linear_lora_fwd_fp32(d["x"], wq, d["a"], d["b"], scale, d["mask"], p)
+    dxe, dae, dbe, _ = lora_ref.linear_lora_bwd_fp32(d["dy"], d["x"], wq, d["a"], d["b"], scale, d["mask"], p)
+    for got, exp, name in ((y, ye, "y"), (x.grad, dxe, "dx"), (a.grad, dae, "da"), (b.grad, dbe, "db")):
+        ok, rel, excess = lora_ref.check_close(got.detach().float().cpu(), exp, rtol=1e-2)
+        assert ok, f"{name}: rel {rel:.3e} excess {excess:.3e}"
