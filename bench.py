@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused LoRA-linear hot path on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): the multi-LoRA packed batch --
+4 adapters of rank 16, scales {16,32,32,64}/16, dropout {0,.05,.1,.1}, lognormal(6.5, 0.8) token
+segments clipped to [64,4096] and packed to 8192 tokens, each adapter padded to 128 rows, shared
+base W[4096,4096] bf16, explicit seeded Bernoulli keep-mask, forward + backward (dX, dA_i, dB_i).
+One "step" = one fused forward + backward of that linear layer with all inputs resident in HBM.
+
+Prints ONE JSON line.  `value` = algorithmic TFLOP/s of the whole step, counted on the 8192 real
+tokens: 2*(2MKN) + 6*M*r*(K+N).  `roofline` describes the dominant kernel (the MFMA GEMM of the
+backward, dX = dY W + LoRA term), timed live with HIP events on the launch stream.  `cpu_baseline`
+is the unfused PyTorch expression (the oracle's bf16 op-by-op arithmetic with autograd backward) on
+a bounded sample of the same workload on the host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+import torch  # noqa: E402
+
+BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+HBM_PEAK_GBS = 8000.0
+
+K = N = 4096
+RANK = 16
+TOKENS = 8192
+SCALES = [1.0, 2.0, 2.0, 4.0]
+DROPOUT = [0.0, 0.05, 0.1, 0.1]
+BLOCK = 128
+
+
+def segments(total_tokens: int, n_adapters: int, seed: int = 0):
+    rng = np.random.default_rng(seed)
+    lens, tot = [], 0
+    while tot < total_tokens:
+        n = int(np.clip(rng.lognormal(6.5, 0.8), 64, 4096))
+        n = min(n, total_tokens - tot)
+        lens.append(n)
+        tot += n
+    per = [0] * n_adapters
+    for i, n in enumerate(lens):
+        per[i % n_adapters] += n
+    return per
+
+
+def build_inputs(device, seq, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(0)
+    padded = [((n - 1) // BLOCK + 1) * BLOCK for n in seq]
+    Mp = sum(padded)
+    x = torch.randn(Mp, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(dtype)
+    dy = torch.randn(Mp, N, generator=g).to(dtype)
+    a_list, b_list = [], []
+    for i in range(len(seq)):
+        ga = torch.Generator().manual_seed(10 + i)
+        a_list.append(((torch.rand(RANK, K, generator=ga) * 2 - 1) / K ** 0.5).to(dtype))
+        b_list.append((torch.randn(N, RANK, generator=ga) * 0.01).to(dtype))
+    gm = torch.Generator().manual_seed(1)
+    row_p = torch.cat([torch.full((pl,), p) for pl, p in zip(padded, DROPOUT)])
+    mask = torch.rand(Mp, K, generator=gm) >= row_p[:, None]
+    t = dict(x=x, w=w, dy=dy, a_list=a_list, b_list=b_list, mask=mask)
+    if device is not None:
+        t = {k: ([v.to(device) for v in val] if isinstance(val, list) else val.to(device)) for k, val in t.items()}
+    t["padded"] = padded
+    return t
+
+
+def step_flops(tokens: int) -> float:
+    return 2 * (2.0 * tokens * K * N) + 6.0 * tokens * RANK * (K + N)
+
+
+def event_time_ms(fn, reps: int) -> float:
+    """Average duration of `fn`'s launches: `reps` back-to-back calls between two HIP events
+    recorded on the stream the kernels are launched on (torch's current stream)."""
+    st = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    fn()
+    torch.cuda.synchronize()
+    e0.record(st)
+    for _ in range(reps):
+        fn()
+    e1.record(st)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def cpu_baseline(seq, budget_s: float = 20.0):
+    """Oracle (bf16 op-by-op, autograd backward) on the first `sample` tokens of every adapter."""
+    from oracle import lora_ref
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    sample = 256
+    sseq = [min(n, sample) for n in seq]
+    t = build_inputs(None, sseq)
+    padded = t["padded"]
+
+    def one():
+        x = t["x"].clone().requires_grad_(True)
+        a = [v.clone().requires_grad_(True) for v in t["a_list"]]
+        b = [v.clone().requires_grad_(True) for v in t["b_list"]]
+        y = lora_ref.linear_multi_lora_bf16_opbyop(x, t["w"], a, b, sseq, padded, SCALES, DROPOUT, t["mask"])
+        y.backward(t["dy"])
+
+    one()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (len(times) < 10 and time.perf_counter() - t_start < budget_s / 2):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_start > budget_s:
+            break
+    med = sorted(times)[len(times) // 2]
+    return {
+        "value": step_flops(sum(sseq)) / med / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{sum(sseq)} tokens ({sample} per adapter) of the same multi-LoRA batch, bf16 op-by-op + autograd, "
+                  f"median of {len(times)} runs, {med * 1e3:.1f} ms/run",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (MI355X); none is visible.")
+
+    from lorafusion_amd.ops import hip_ops
+    from lorafusion_amd.ops.multi_lora import fused_linear_multi_lora, prepare_multi_lora_batch_info
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton, quantize_nf4
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    seq = segments(TOKENS, 4)
+    t = build_inputs(dev, seq)
+    info = prepare_multi_lora_batch_info(seq, [0, 1, 2, 3], [RANK] * 4, DROPOUT, SCALES, BLOCK)
+    x = t["x"].requires_grad_(True)
+    a_list = [a.requires_grad_(True) for a in t["a_list"]]
+    b_list = [b.requires_grad_(True) for b in t["b_list"]]
+    x3, dy3 = x.unsqueeze(0), t["dy"].unsqueeze(0)
+
+    def step():
+        y = fused_linear_multi_lora(
+            x3, t["w"], lora_a_list=a_list, lora_b_list=b_list, seq_len_list=seq,
+            padded_seq_len_list=info.padded_seq_len_list, block_to_lookup_table=info.block_to_lookup_table,
+            block_to_dropout_p=info.block_to_dropout_p, block_to_alpha=info.block_to_alpha,
+            enable_dropout=True, same_dropout_p_value=None, max_r=RANK, dropout_mask=t["mask"])
+        y.backward(dy3)
+        x.grad = None
+        for p in a_list + b_list:
+            p.grad = None
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = step_flops(TOKENS) / (ms * 1e-3) / 1e12
+
+    # ---- per-kernel timings with HIP events (kernel launches only, outputs preallocated by the wrappers)
+    routing = hip_ops.MultiRouting(info.padded_seq_len_list, [RANK] * 4, info.block_to_lookup_table,
+                                   info.block_to_alpha, info.block_to_dropout_p)
+    xd, wd, dyd, mask = x.detach(), t["w"], t["dy"], t["mask"]
+    ad = [a.detach() for a in a_list]
+    bd = [b.detach() for b in b_list]
+    s = hip_ops.fused_multi_lora_xa(xd, ad, routing, mask)
+    _, ds = hip_ops.fused_multi_lora_dys_dyb(dyd, s, bd, routing)
+    Mp = xd.shape[0]
+    reps = 20
+    t_fwd = event_time_ms(lambda: hip_ops.fused_multi_lora_xw_sb(xd, wd, s, bd, routing), reps)
+    t_bwd = event_time_ms(lambda: hip_ops.fused_multi_lora_dyw_dsa(dyd, wd, ds, ad, routing, mask), reps)
+    t_plain_nt = event_time_ms(lambda: hip_ops.gemm(xd, wd, trans_b=True), reps)
+    t_plain_nn = event_time_ms(lambda: hip_ops.gemm(dyd, wd, trans_b=False), reps)
+    t_xa = event_time_ms(lambda: hip_ops.fused_multi_lora_xa(xd, ad, routing, mask), reps)
+    t_dys = event_time_ms(lambda: hip_ops.fused_multi_lora_dys_dyb(dyd, s, bd, routing), reps)
+    t_da = event_time_ms(lambda: hip_ops.fused_multi_lora_da(xd, ds, routing, mask), reps)
+    # algorithmic flops of one GEMM launch: 2*Mp*K*N dense + 2*Mp*r*N LoRA seed (Mp = rows launched)
+    gemm_flops = 2.0 * Mp * K * N + 2.0 * Mp * RANK * N
+    dom_ms, dom_name = (t_bwd, "gemm_lora_kernel<NN> (dX = dY W + mask*(dS A)/(1-p))") if t_bwd >= t_fwd else \
+                       (t_fwd, "gemm_lora_kernel<NT> (Y = X W^T + scale*S B^T)")
+    achieved = gemm_flops / (dom_ms * 1e-3) / 1e12
+
+    # ---- NF4 dequant (W[14336,4096], blocksize 64, double quantised): 2.516 B/element
+    wq = torch.randn(14336, 4096, device=dev) * 0.02
+    packed, qs = quantize_nf4(wq)
+    out = torch.empty(14336 * 4096, dtype=torch.bfloat16, device=dev)
+    t_nf4 = event_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), reps)
+    n = 14336 * 4096
+    nf4_bytes = n / 2 + n / 64 + 4 * n / 16384 + 1028 + 2 * n
+    nf4_gbs = nf4_bytes / (t_nf4 * 1e-3) / 1e9
+
+    res = {
+        "metric": "fused LoRA fwd+bwd TFLOP/s (8B layer, r=16); NF4 dequant GB/s; % roofline",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "multi-LoRA packed batch: 4 adapters r=16, 8192 tokens (lognormal segments, seed 0) "
+                        f"padded to {Mp} rows, K=N=4096, fwd+bwd, explicit dropout mask",
+            "tokens": TOKENS, "rows_launched": Mp, "K": K, "N": N, "rank": RANK, "adapters": 4,
+            "seq_len_list": seq,
+        },
+        "roofline": {
+            "bound": "mfma", "achieved": round(achieved, 2), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / BF16_PEAK_TFLOPS, 4), "traffic": None,
+            "kernel": dom_name, "launch_ms": round(dom_ms, 4), "flops_per_launch": gemm_flops,
+        },
+        "kernels_ms": {
+            "xa": round(t_xa, 4), "gemm_fwd": round(t_fwd, 4), "dys_dyb": round(t_dys, 4), "da": round(t_da, 4),
+            "gemm_bwd": round(t_bwd, 4), "plain_gemm_nt": round(t_plain_nt, 4), "plain_gemm_nn": round(t_plain_nn, 4),
+        },
+        "lora_overhead_vs_plain_gemms": round((t_xa + t_fwd + t_dys + t_da + t_bwd) / (t_plain_nt + t_plain_nn) - 1.0, 4),
+        "nf4_dequant": {
+            "GB/s": round(nf4_gbs, 1), "frac_of_hbm_peak": round(nf4_gbs / HBM_PEAK_GBS, 4),
+            "launch_ms": round(t_nf4, 4), "bytes_per_launch": nf4_bytes, "shape": [14336, 4096],
+        },
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(seq)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -15,8 +15,9 @@
 // Structure: one workgroup per BMxBN tile, 64-wide wavefronts each owning a WMxWN sub-tile of
 // 32x32x16 MFMA blocks; BK = 64.  Both operand tiles go global -> LDS with 16-byte
 // direct-to-LDS loads (no VGPR staging), double buffered, one barrier per K step.  LDS rows
-// are XOR-swizzled in 16-byte granules so that the ds_read_b128 fragment reads are bank
-// conflict free; the swizzle is applied on the global side of the direct load (each lane
+// (128 bytes = 8 granules of 16 bytes) are XOR-swizzled with key (row>>1)&7 so that any 16
+// consecutive lanes of a ds_read_b128 fragment read (16 rows, one granule each) touch all 64
+// banks exactly once; the swizzle is applied on the global side of the direct load (each lane
 // picks the granule whose LDS slot it owns).  The NN operand is stored untransposed and read
 // with ds_read_b64_tr_b16, which hands each lane four consecutive contraction elements of
 // its column.  MFMA operands are swapped (B fragment as the "a" operand) so each lane ends
@@ -97,24 +98,31 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   const T* __restrict__ A = (const T*)p.A;
   const T* __restrict__ B = (const T*)p.B;
 
+  // ---- staggered start of the K loop: workgroups that run side by side walk K from different
+  // offsets (one 128-byte step apart) so their tile loads spread over the memory channels
+  // instead of all hitting the same channel when the row pitch is a power of two.
+  const int nk = p.K / BK;
+  const int kstart = ((pid_m + pid_n) & 15) % nk;
+  const int wrap_at = nk - kstart;  // number of tiles issued before the pointers wrap to k = 0
+
   // ---- per-thread global source pointers for the direct-to-LDS loads
   const T* aptr[NLA];
   const T* bptr[NLB];
   {
-    const int r8 = (tid >> 3) & 7;
-    const int srcg = (tid & 7) ^ r8;  // swizzle: LDS slot (tid&7) of row r holds granule slot^(r&7)
+    const int r8 = (tid >> 4) & 7;
+    const int srcg = (tid & 7) ^ r8;  // swizzle: LDS slot (tid&7) of row r holds granule slot^((r>>1)&7)
 #pragma unroll
     for (int i = 0; i < NLA; i++) {
       int row = i * (NTHREADS / 8) + (tid >> 3);
       int gm = min(m0 + row, p.M - 1);
-      aptr[i] = A + (int64_t)gm * p.lda + srcg * 8;
+      aptr[i] = A + (int64_t)gm * p.lda + srcg * 8 + kstart * BK;
     }
     if constexpr (!NN) {
 #pragma unroll
       for (int i = 0; i < NLB; i++) {
         int row = i * (NTHREADS / 8) + (tid >> 3);
         int gn = min(n0 + row, p.N - 1);
-        bptr[i] = B + (int64_t)gn * p.ldb + srcg * 8;
+        bptr[i] = B + (int64_t)gn * p.ldb + srcg * 8 + kstart * BK;
       }
     } else {
 #pragma unroll
@@ -123,11 +131,12 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         int row = gid / GPR, g = gid % GPR;
         int srcseg = (g >> 2) ^ (row & 3);
         int col = min(n0 + (srcseg * 4 + (g & 3)) * 8, p.N - 8);
-        bptr[i] = B + (int64_t)row * p.ldb + col;
+        bptr[i] = B + (int64_t)(row + kstart * BK) * p.ldb + col;
       }
     }
   }
 
+  int issued = 0;
   auto issue_loads = [&](int stage) {
     char* la = ldsA + stage * A_STAGE + wave * 1024;
     char* lb = ldsB + stage * B_STAGE + wave * 1024;
@@ -140,6 +149,14 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     for (int i = 0; i < NLB; i++) {
       load_g2l_16(bptr[i], lb + i * NTHREADS * 16);
       if constexpr (!NN) bptr[i] += BK; else bptr[i] += (int64_t)BK * p.ldb;
+    }
+    if (++issued == wrap_at) {
+#pragma unroll
+      for (int i = 0; i < NLA; i++) aptr[i] -= p.K;
+#pragma unroll
+      for (int i = 0; i < NLB; i++) {
+        if constexpr (!NN) bptr[i] -= p.K; else bptr[i] -= (int64_t)p.K * p.ldb;
+      }
     }
   };
 
@@ -231,7 +248,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   int a_off[TM], b_off[TN];
 #pragma unroll
   for (int i = 0; i < TM; i++) a_off[i] = (wm * WM + i * 32 + l32) * 128;
-  const int sw = l32 & 7;
+  const int sw = (l32 >> 1) & 7;
   int btr_key = 0, btr_in = 0;
   if constexpr (!NN) {
 #pragma unroll
@@ -250,42 +267,66 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     (void)btr_in;
   }
 
-  auto compute = [&](int stage) {
+  // ---- main loop.  Fragments are double buffered in registers: the LDS reads of k-step ks+1 are
+  // issued before the MFMAs of k-step ks.  The single barrier of an iteration sits before the last
+  // k-step: by then every wave has read all of the current stage, so the next stage (whose loads
+  // were issued at the top of the iteration) can be read right after it and the current stage can
+  // be overwritten by the loads issued at the top of the next iteration.
+  lf_u32x4 fa[2][TM], fb[2][TN];
+  auto read_frags = [&](int buf, int stage, int ks) {
     const char* sa = ldsA + stage * A_STAGE;
     const char* sb = ldsB + stage * B_STAGE;
+    const int slot = ((2 * ks + q) ^ sw) << 4;
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ks++) {
-      lf_u32x4 af[TM], bf[TN];
-      const int slot = ((2 * ks + q) ^ sw) << 4;
+    for (int i = 0; i < TM; i++) fa[buf][i] = *(const lf_u32x4*)(sa + a_off[i] + slot);
+    if constexpr (!NN) {
 #pragma unroll
-      for (int i = 0; i < TM; i++) af[i] = *(const lf_u32x4*)(sa + a_off[i] + slot);
-      if constexpr (!NN) {
+      for (int j = 0; j < TN; j++) fb[buf][j] = *(const lf_u32x4*)(sb + b_off[j] + slot);
+    } else {
 #pragma unroll
-        for (int j = 0; j < TN; j++) bf[j] = *(const lf_u32x4*)(sb + b_off[j] + slot);
-      } else {
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-          const char* base = sb + b_off[j] + ks * 16 * BPITCH;
-          lf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(base));
-          lf_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(base + 4 * BPITCH));
-          lf_u32x2 lo2 = __builtin_bit_cast(lf_u32x2, lo), hi2 = __builtin_bit_cast(lf_u32x2, hi);
-          bf[j] = lf_u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
-        }
+      for (int j = 0; j < TN; j++) {
+        const char* base = sb + b_off[j] + ks * 16 * BPITCH;
+        lf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(base));
+        lf_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(base + 4 * BPITCH));
+        lf_u32x2 lo2 = __builtin_bit_cast(lf_u32x2, lo), hi2 = __builtin_bit_cast(lf_u32x2, hi);
+        fb[buf][j] = lf_u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
       }
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(bf[j], af[i], acc[i][j]);
     }
   };
+  auto mfmas = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(fb[buf][j], fa[buf][i], acc[i][j]);
+  };
+  auto interleave = [&]() {  // scheduling hint: spread one k-step's LDS reads across its MFMAs
+    constexpr int NR = NN ? TM + 2 * TN : TM + TN, NM = TM * TN;
+    constexpr int PER = NM / NR > 0 ? NM / NR : 1;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, NM > PER * NR ? NM - PER * NR : 0, 0);
+  };
 
-  const int nk = p.K / BK;
-  __builtin_amdgcn_s_waitcnt(0);  // all counters (encoding 0 = vmcnt/expcnt/lgkmcnt zero)
+  __builtin_amdgcn_s_waitcnt(0);  // all counters zero: the first tile has landed
   __syncthreads();
+  read_frags(0, 0, 0);
   for (int kt = 0; kt < nk; kt++) {
-    if (kt + 1 < nk) issue_loads((kt + 1) & 1);
-    compute(kt & 1);
-    __syncthreads();
+    const int cur = kt & 1;
+    if (kt + 1 < nk) issue_loads(cur ^ 1);
+#pragma unroll
+    for (int ks = 0; ks < 3; ks++) {
+      read_frags((ks + 1) & 1, cur, ks + 1);
+      mfmas(ks & 1);
+      interleave();
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_s_barrier();
+    if (kt + 1 < nk) read_frags(0, cur ^ 1, 0);
+    mfmas(1);
+    interleave();
   }
 
   // ---- epilogue: bias, convert, 8-byte stores (4 consecutive columns of one row per lane)
@@ -345,19 +386,25 @@ int launch_dtype(const LfGemmParams& p, const LfSegTable& seg, int cfg, hipStrea
 
 }  // namespace
 
-// Tile choice: fewest "rounds" of 256 CUs weighted by tile area (bigger tiles reuse more per
-// LDS byte, but a nearly empty last round wastes the chip).
-static int choose_cfg(int M, int N) {
-  const int bm[5] = {256, 256, 128, 128, 128}, bn[5] = {256, 256, 256, 256, 128};
-  const double eff[5] = {1.00, 0.97, 0.93, 0.90, 0.80};
-  int best = 0;
+// Tile choice from a measured cost model: a launch runs in "rounds" of resident workgroups
+// (256 CUs x workgroups per CU); a full round of each configuration costs `unit` (relative to one
+// round of 256x256 tiles), a partly filled last round costs less than a full one.
+static int choose_cfg(int M, int N, bool nn) {
+  struct Cand { int cfg, bm, bn, slots; double unit_nt, unit_nn; };
+  static const Cand cands[3] = {
+      {1, 256, 256, 256, 1.000, 1.000},   // 8 waves, 128x64 per wave
+      {3, 128, 256, 256, 0.539, 0.645},   // 8 waves, 64x64 per wave
+      {4, 128, 128, 512, 0.550, 0.620},   // 4 waves, two workgroups per CU
+  };
+  int best = 1;
   double best_cost = 1e30;
-  for (int c = 0; c < 5; c++) {
-    if (c == 1 || c == 3) continue;  // 8-wave variants are picked only explicitly
-    long tiles = (long)((M + bm[c] - 1) / bm[c]) * ((N + bn[c] - 1) / bn[c]);
-    long rounds = (tiles + 255) / 256;
-    double cost = (double)rounds * bm[c] * bn[c] / eff[c];
-    if (cost < best_cost) { best_cost = cost; best = c; }
+  for (const Cand& c : cands) {
+    const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+    const long full = tiles / c.slots;
+    const double fill = (double)(tiles % c.slots) / c.slots;
+    const double unit = nn ? c.unit_nn : c.unit_nt;
+    const double cost = unit * (full + (fill > 0 ? 0.45 + 0.55 * fill : 0.0));
+    if (cost < best_cost) { best_cost = cost; best = c.cfg; }
   }
   return best;
 }
@@ -367,7 +414,7 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
   if (p.K % BK != 0 || p.N % 8 != 0 || p.N < 8) return LF_ESHAPE;
   if (p.L != nullptr && (p.R % 16 != 0 || p.R <= 0 || p.R > LF_MAX_RANK)) return LF_ESHAPE;
   if (seg.table != nullptr && (seg.block_size_m % 64 != 0)) return LF_ESHAPE;
-  int cfg = force_cfg >= 0 ? force_cfg : choose_cfg(p.M, p.N);
+  int cfg = force_cfg >= 0 ? force_cfg : choose_cfg(p.M, p.N, nn);
   if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1)) cfg = 2;
   if (dtype == LF_BF16) return nn ? launch_dtype<__bf16, true>(p, seg, cfg, st) : launch_dtype<__bf16, false>(p, seg, cfg, st);
   if (dtype == LF_F16) return nn ? launch_dtype<_Float16, true>(p, seg, cfg, st) : launch_dtype<_Float16, false>(p, seg, cfg, st);

@@ -155,7 +155,10 @@ def dequantize_exact(st: NF4State) -> np.ndarray:
         else:
             absmax = np.float32(st.absmax[blk])
         val = _round_fraction_to_f32(Fraction(float(NF4_CODE[idx])) * Fraction(float(absmax)))
-        out[e] = _f32_to_bf16_bits_exact(val)
+        bits = _f32_to_bf16_bits_exact(val)
+        if val == 0 and (np.signbit(NF4_CODE[idx]) != np.signbit(absmax)):
+            bits |= 0x8000  # IEEE sign of a zero product: code 7 (+0.0) times a negative absmax is -0.0
+        out[e] = bits
     return out
 
 

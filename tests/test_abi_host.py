@@ -1,0 +1,145 @@
+"""CPU-side checks: the C-ABI library loads, exports every symbol the header declares, rejects bad
+arguments before touching a GPU, and the Python layer fails loudly without a GPU / without the library."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "lorafusion_hip.h")).read()
+    return sorted(set(re.findall(r"\b(lf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from lorafusion_amd import _lib
+
+    lib = _lib.lib()
+    declared = _declared_symbols()
+    assert set(declared) == set(_lib.EXPORTS), (declared, _lib.EXPORTS)
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.lf_version() >= 1
+    assert b"workspace" in lib.lf_strerror(-3)
+    assert lib.lf_strerror(0) == b"ok"
+
+
+def test_routing_struct_layout_matches_header():
+    from lorafusion_amd import _lib
+
+    # 4 int32 + 3 pointers + 2 floats + 2 x 32 int32
+    assert ctypes.sizeof(_lib.Routing) == 16 + 24 + 8 + 2 * 4 * _lib.LF_MAX_SEG
+    r = _lib.single_routing(16, 2.0, 0.1)
+    assert r.n_seg == 1 and r.seg_rank[0] == 16 and abs(r.p - 0.1) < 1e-7
+
+
+def test_argument_validation_without_gpu():
+    """Error paths return codes before any launch (null pointers / bad shapes never reach a kernel)."""
+    from lorafusion_amd import _lib
+
+    lib = _lib.lib()
+    r = _lib.single_routing(16, 1.0, 0.0)
+    ptrs = (ctypes.c_void_p * 1)()
+    # null tensors
+    assert lib.lf_lora_xw_sb(None, None, None, None, ptrs, None, 128, 128, 128, 16, r, 0, None) == -1
+    assert lib.lf_nf4_dequant(None, None, None, None, None, None, 64, 64, 0, 0, None) == -1
+    assert lib.lf_gemm(None, None, None, None, 128, 128, 128, 1, 0, -1, None) == -1
+    # unknown dtype
+    one = ctypes.c_void_p(16)
+    assert lib.lf_gemm(one, one, None, one, 128, 128, 128, 1, 7, -1, None) == -1
+    # workspace sizes are positive and grow with the problem
+    small = lib.lf_workspace_bytes(_lib.LF_OP_BWD, 256, 256, 256, 16, r)
+    big = lib.lf_workspace_bytes(_lib.LF_OP_BWD, 4096, 4096, 4096, 16, r)
+    assert 0 < small < big and small % 256 == 0
+    # bad routing: rank not a multiple of 8, too many segments
+    bad = _lib.single_routing(12, 1.0, 0.0)
+    assert lib.lf_workspace_bytes(_lib.LF_OP_FWD, 256, 256, 256, 16, bad) == 0
+    bad2 = _lib.single_routing(16, 1.0, 0.0)
+    bad2.n_seg = 64
+    assert lib.lf_lora_xa(one, None, ptrs, one, one, 1 << 20, 128, 128, 16, bad2, 0, None) == -5
+
+
+def test_python_layer_refuses_cpu_tensors():
+    from lorafusion_amd.ops.lora_v1 import fused_linear_lora
+    from lorafusion_amd.ops.nf4 import QuantState, dequantize_nf4_triton
+
+    x = torch.zeros(128, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="GPU"):
+        fused_linear_lora(x, x, x[:16], x[:, :16].contiguous(), 1.0)
+    with pytest.raises(ValueError, match="GPU"):
+        dequantize_nf4_triton(torch.zeros(64, dtype=torch.uint8),
+                              QuantState(torch.Size([128]), torch.bfloat16, 64, torch.ones(2)))
+
+
+def test_missing_library_is_fatal(monkeypatch):
+    from lorafusion_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", os.path.join(ROOT, "does_not_exist.so"))
+    with pytest.raises(RuntimeError, match="no non-HIP fallback"):
+        _lib.lib()
+
+
+def test_product_does_not_import_oracle():
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "lorafusion_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text, f
+
+
+def test_manager_and_patch_host_logic():
+    from lorafusion_amd.ops import multi_lora as ml
+    from lorafusion_amd.patch import patch_lora
+
+    ml.reset_multi_lora_manager()
+    mgr = ml.init_multi_lora_manager([object(), object()], num_pipeline_stages=2)
+    with pytest.raises(ValueError):
+        ml.init_multi_lora_manager([object()], 1)
+    info_a = ml.prepare_multi_lora_batch_info([5], [0], [16], [0.0], [1.0], 128, device="cpu", allow_empty_micro_batch_info=True)
+    info_b = ml.prepare_multi_lora_batch_info([7], [1], [16], [0.0], [1.0], 128, device="cpu", allow_empty_micro_batch_info=True)
+    mgr.add_batch_info(info_a)
+    mgr.add_batch_info(info_b)
+    with pytest.raises(ValueError):
+        mgr.add_batch_info(info_b)   # deque is full
+    assert mgr.get_newest_batch_info() is info_b and mgr.get_oldest_batch_info() is info_a
+    assert info_a.microbatch_idx == 0 and info_b.microbatch_idx == 1
+    mgr.mark_backward_pass_started()
+    assert not mgr.is_in_forward
+    assert mgr.pop_oldest_batch_info() is info_a
+    mgr.mark_forward_pass_started()
+    assert mgr.is_in_forward
+    strict = ml.prepare_multi_lora_batch_info([7], [1], [16], [0.0], [1.0], 128, device="cpu")
+    with pytest.raises(ValueError):
+        mgr.add_batch_info(strict)   # MicroBatchInfo missing and not allowed to be empty
+    ml.reset_multi_lora_manager()
+    with pytest.raises(TypeError):
+        patch_lora.lora_forward(object(), torch.zeros(1))
+    assert ml.get_lora_kernel_config("fused_multi_lora_block_size_m") == 128
+    with pytest.raises(ValueError):
+        ml.get_lora_kernel_config("fused_lora_xw_sb")
+
+
+def test_torch_ref_path_matches_oracle_on_cpu():
+    """The unfused (use_fused=False) product path is plain torch and runs on CPU."""
+    from lorafusion_amd.ops.lora_torch_ref import torch_ref_linear_lora, torch_ref_linear_multi_lora
+    from oracle import lora_ref
+    from tests.util import multi_inputs, single_inputs
+
+    d = single_inputs(32, 64, 48, 8, p=0.0, seed=0, dtype=torch.float32, bias=True)
+    y = torch_ref_linear_lora(d["x"], d["w"], d["a"], d["b"], 2.0, 0.0, d["bias"])
+    ye, _ = lora_ref.linear_lora_fwd_fp32(d["x"], d["w"], d["a"], d["b"], 2.0, None, 0.0, d["bias"])
+    assert torch.allclose(y, ye, atol=1e-5)
+    seq = [5, 9]
+    m = multi_inputs(seq, 64, 48, [8, 16], [0.0, 0.0], dtype=torch.float32, block=8)
+    ym = torch_ref_linear_multi_lora(m["x"].unsqueeze(0), m["w"], lora_a_list=m["a_list"], lora_b_list=m["b_list"],
+                                     seq_len_list=seq, padded_seq_len_list=m["padded"], alpha_list=[1.0, 2.0],
+                                     dropout_p_list=[0.0, 0.0])
+    yme, _ = lora_ref.linear_multi_lora_fwd_fp32(m["x"], m["w"], m["a_list"], m["b_list"], seq, m["padded"],
+                                                 [1.0, 2.0], [0.0, 0.0])
+    assert torch.allclose(ym[0], yme, atol=1e-5)

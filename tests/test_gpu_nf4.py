@@ -86,8 +86,8 @@ def test_dequant_config2_shape_and_roundtrip():
     assert np.array_equal(_bits(got), onf4.dequantize(st))
     absmax_true = np.abs(w.reshape(-1, 64)).max(axis=1)
     err = np.abs(got.float().cpu().numpy().reshape(-1, 64) - w.reshape(-1, 64)).max(axis=1)
-    # widest gap in the code is 1.0 - 0.7229568 = 0.277; half of it, plus slack for the 8-bit absmax code and bf16
-    assert (err <= (0.1386 + 0.03) * absmax_true + 1e-6).all()
+    # widest gap in the code is -0.6962 - (-1.0) = 0.3038; half of it, plus slack for the 8-bit absmax code and bf16
+    assert (err <= (0.1520 + 0.03) * absmax_true + 1e-6).all()
 
 
 def test_dequant_errors():
