@@ -13,6 +13,14 @@
 // order, apply scale / 1/(1-p), zero padded rows and rank columns, and cast.  Results are
 // therefore run-to-run deterministic.
 //
+// Streaming: the big operand moves as 128-row x 64-column tiles.  Global loads are coalesced
+// (8 consecutive lanes read one 128-byte row segment), the keep-mask is applied in registers,
+// and the tile is written to LDS with the same XOR swizzle as the GEMM (granule g of row r
+// at slot g ^ ((r>>1)&7)), from where both MFMA access patterns are bank-conflict free:
+// row fragments (ds_read_b128) and transposed fragments (ds_read_b64_tr_b16).  Loading MFMA
+// fragments straight from global memory would put every lane on a different row (one cache
+// line per lane) and runs at a quarter of the coalesced rate.
+//
 // MFMA 16x16x32 operand layout (64 lanes): lane l holds row/col (l & 15) and the 8
 // contraction elements of chunk (l >> 4).  Where the contraction index is the slow memory
 // dimension, tiles are staged in LDS and read with ds_read_b64_tr_b16 (16 lanes read a
@@ -86,20 +94,86 @@ __device__ __forceinline__ lf_u32x4 tr_read8(const char* p, int pitch) {
   return lf_u32x4{a[0], a[1], b[0], b[1]};
 }
 
+
+constexpr int TILE_BYTES = ROWS * 128;  // 128 rows x 64 columns of 16-bit
+
+// One thread's share of a 128x64 tile: 4 granules of 8 elements (+ their 8 mask bytes each).
+struct TileRegs {
+  lf_u32x4 x[4];
+  lf_u32x2 m[4];
+};
+
+// Coalesced load of the tile whose first element is src[row0*ld + col0]; rows are clamped to max_row-1.
+template <typename T>
+__device__ __forceinline__ void tile_load(TileRegs& r, const T* __restrict__ src, const uint8_t* __restrict__ mask,
+                                          int64_t ld, int row0, int max_row, int col0, int tid, bool use_mask) {
+  const int srcg = (tid & 7) ^ ((tid >> 4) & 7);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int row = min(row0 + i * 32 + (tid >> 3), max_row - 1);
+    const int64_t off = (int64_t)row * ld + col0 + srcg * 8;
+    r.x[i] = __builtin_nontemporal_load((const lf_u32x4*)(src + off));
+    if (use_mask) r.m[i] = __builtin_nontemporal_load((const lf_u32x2*)(mask + off));
+  }
+}
+
+__device__ __forceinline__ void tile_store(const TileRegs& r, char* tile, int tid, bool use_mask) {
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    *(lf_u32x4*)(tile + (i * 256 + tid) * 16) = use_mask ? apply_mask8(r.x[i], r.m[i]) : r.x[i];
+}
+
+// Row fragment: 8 consecutive columns (granule g) of `row`.
+__device__ __forceinline__ lf_u32x4 tile_row_frag(const char* tile, int row, int g) {
+  return *(const lf_u32x4*)(tile + row * 128 + ((g ^ ((row >> 1) & 7)) << 4));
+}
+
+// Transposed fragment: rows row..row+3 and row+4..row+7 of the lane's column; `col` is the first
+// of the 4 columns this lane addresses (multiple of 4).
+__device__ __forceinline__ lf_u32x4 tile_tr_frag(const char* tile, int row, int col) {
+  const int g = col >> 3, within = (col & 7) * 2;
+  const char* p0 = tile + row * 128 + ((g ^ ((row >> 1) & 7)) << 4) + within;
+  const char* p1 = tile + (row + 4) * 128 + ((g ^ (((row + 4) >> 1) & 7)) << 4) + within;
+  lf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(p0));
+  lf_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(p1));
+  lf_u32x2 a = __builtin_bit_cast(lf_u32x2, lo), b = __builtin_bit_cast(lf_u32x2, hi);
+  return lf_u32x4{a[0], a[1], b[0], b[1]};
+}
+
 // ------------------------------------------------------------------------------------ xa
 // grid (n_blocks, ksplit); 4 waves, wave w owns rows 32w..32w+31 of the block.
 // part[ks][row][R] (fp32) = sum over this K slice of mask*X*A^T  (unscaled).
+// LDS: two X tiles + the A slice [RT*16][kslice] (row pitch kslice*2+16 bytes: 16 rows land on
+// 16 different bank groups).
 template <typename T, int RT>
 __global__ void __launch_bounds__(256)
 lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, float* __restrict__ part,
                int M, int K, int R, int kslice, const LfSegTable seg) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* xs = lds;
+  char* as = lds + 2 * TILE_BYTES;
   const int blk = blockIdx.x, ks = blockIdx.y;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, qq = lane >> 4;
   const BlockInfo bi = block_info(seg, blk, M);
   const T* __restrict__ A = (const T*)seg.ptr[bi.seg];
   const bool use_mask = mask != nullptr && bi.p > 0.f;
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
+  const int k_begin = ks * kslice;
+  const int ntiles = kslice / 64;
+  const int apitch = kslice * 2 + 16;
+
+  TileRegs tr;
+  tile_load(tr, X, mask, K, blk * ROWS, Mrows, k_begin, tid, use_mask);
+  for (int g = tid; g < RT * 16 * (kslice / 8); g += 256) {
+    const int r = g / (kslice / 8), c = g % (kslice / 8);
+    lf_u32x4 v = {0, 0, 0, 0};
+    if (r < bi.rank) v = *(const lf_u32x4*)(A + (int64_t)r * K + k_begin + c * 8);
+    *(lf_u32x4*)(as + r * apitch + c * 16) = v;
+  }
+  tile_store(tr, xs, tid, use_mask);
+  if (ntiles > 1) tile_load(tr, X, mask, K, blk * ROWS, Mrows, k_begin + 64, tid, use_mask);
+  __syncthreads();
 
   lf_f32x4 acc[2][RT];
 #pragma unroll
@@ -107,42 +181,25 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, float*
 #pragma unroll
     for (int c = 0; c < RT; c++) acc[a][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
 
-  int64_t xrow[2];
+  for (int t = 0; t < ntiles; t++) {
+    const char* cur = xs + (t & 1) * TILE_BYTES;
 #pragma unroll
-  for (int rt = 0; rt < 2; rt++) xrow[rt] = min(blk * ROWS + wave * 32 + rt * 16 + li, Mrows - 1);
-
-  const int k_begin = ks * kslice, k_end = min(K, k_begin + kslice);
-  for (int kb = k_begin; kb < k_end; kb += 128) {
-    const int kc = kb + qq * 32;  // this lane's 32 contiguous k
-    lf_u32x4 xf[2][4];
+    for (int step = 0; step < 2; step++) {
+      lf_u32x4 xf[2];
 #pragma unroll
-    for (int rt = 0; rt < 2; rt++) {
-      const T* xp = X + xrow[rt] * K + kc;
+      for (int rt = 0; rt < 2; rt++) xf[rt] = tile_row_frag(cur, wave * 32 + rt * 16 + li, step * 4 + qq);
 #pragma unroll
-      for (int j = 0; j < 4; j++) xf[rt][j] = __builtin_nontemporal_load((const lf_u32x4*)(xp + 8 * j));
-      if (use_mask) {
-        const lf_u32x2* mp = (const lf_u32x2*)(mask + xrow[rt] * K + kc);
+      for (int c = 0; c < RT; c++) {
+        const lf_u32x4 af = *(const lf_u32x4*)(as + (c * 16 + li) * apitch + (t * 64 + step * 32 + qq * 8) * 2);
 #pragma unroll
-        for (int j = 0; j < 4; j++) xf[rt][j] = apply_mask8(xf[rt][j], __builtin_nontemporal_load(mp + j));
+        for (int rt = 0; rt < 2; rt++) acc[rt][c] = Mfma16<T>::run(xf[rt], af, acc[rt][c]);
       }
     }
-#pragma unroll
-    for (int c = 0; c < RT; c++) {
-      const int r = c * 16 + li;
-      lf_u32x4 af[4];
-      if (r < bi.rank) {
-        const T* ap = A + (int64_t)r * K + kc;
-#pragma unroll
-        for (int j = 0; j < 4; j++) af[j] = *(const lf_u32x4*)(ap + 8 * j);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; j++) af[j] = lf_u32x4{0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[rt][c] = Mfma16<T>::run(xf[rt][j], af[j], acc[rt][c]);
+    if (t + 1 < ntiles) {
+      tile_store(tr, xs + ((t + 1) & 1) * TILE_BYTES, tid, use_mask);
+      if (t + 2 < ntiles) tile_load(tr, X, mask, K, blk * ROWS, Mrows, k_begin + (t + 2) * 64, tid, use_mask);
     }
+    __syncthreads();
   }
   // C layout: lane holds column (lane & 15), rows 4*(lane >> 4) + e
   float* out = part + (int64_t)ks * Mrows * R;
@@ -157,7 +214,7 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, float*
       }
 }
 
-// S[row][col] = cast( 1/(1-p) * sum_ks part[ks][row][col] ), zero for padded rows / rank columns.
+// S[row][col] = cast( mult * sum_p part[p][row][col] ), zero for padded rows / rank columns.
 template <typename T>
 __global__ void __launch_bounds__(256)
 reduce_rows_kernel(const float* __restrict__ part, T* __restrict__ out, int nparts, int M, int R,
@@ -177,20 +234,20 @@ reduce_rows_kernel(const float* __restrict__ part, T* __restrict__ out, int npar
 }
 
 // ------------------------------------------------------------------------------- dys_dyb
-// grid (n_blocks, nsplit).  Each workgroup walks its N slice in 128-column chunks:
-//   dS partial  [128 rows, R]  += dY_chunk * B_chunk          (accumulated over the slice)
-//   dB partial  [128 cols, R]   = dY_chunk^T * S_block        (complete per chunk)
-// LDS: dY chunk [128][128] pitch 288 B, B chunk [128][R] and S block [128][R] pitch 2R+32 B
-// (pitches keep the 4-row transpose reads on distinct banks).
+// grid (n_blocks, nsplit).  Each workgroup walks its N slice in 64-column tiles of dY:
+//   dS partial  [128 rows, R]  += dY_tile * B_tile            (accumulated over the slice)
+//   dB partial  [64 cols, R]    = dY_tile^T * S_block         (complete per tile)
+// LDS: two dY tiles, the S block [128][R] and two B tiles [64][R] (pitch 2R+32 bytes keeps the
+// 4-row transpose reads on distinct banks).
 template <typename T, int RT>
 __global__ void __launch_bounds__(256)
 lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __restrict__ ds_part,
                     float* __restrict__ db_part, int M, int N, int R, int nslice, const LfSegTable seg) {
-  constexpr int DYP = 288;
   constexpr int RP = RT * 32 + 32;
-  __shared__ __attribute__((aligned(16))) char lds_dy[ROWS * DYP];
-  __shared__ __attribute__((aligned(16))) char lds_b[128 * RP];
-  __shared__ __attribute__((aligned(16))) char lds_s[ROWS * RP];
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* ys = lds;
+  char* ss = lds + 2 * TILE_BYTES;
+  char* bs = ss + ROWS * RP;
 
   const int blk = blockIdx.x, ns = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -198,14 +255,45 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
   const BlockInfo bi = block_info(seg, blk, M);
   const T* __restrict__ Bl = (const T*)seg.ptr[bi.seg];
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
+  const int n_begin = ns * nslice;
+  const int ntiles = nslice / 64;
 
+  auto load_b = [&](lf_u32x4 (&br)[(64 * RT * 2 + 255) / 256], int n0) {
+#pragma unroll
+    for (int i = 0; i < (64 * RT * 2 + 255) / 256; i++) {
+      const int g = i * 256 + tid;
+      const int row = g / (RT * 2), gc = g % (RT * 2);
+      lf_u32x4 v = {0, 0, 0, 0};
+      if (g < 64 * RT * 2 && gc * 8 < bi.rank) v = *(const lf_u32x4*)(Bl + (int64_t)(n0 + row) * bi.rank + gc * 8);
+      br[i] = v;
+    }
+  };
+  auto store_b = [&](const lf_u32x4 (&br)[(64 * RT * 2 + 255) / 256], char* dst) {
+#pragma unroll
+    for (int i = 0; i < (64 * RT * 2 + 255) / 256; i++) {
+      const int g = i * 256 + tid;
+      if (g < 64 * RT * 2) *(lf_u32x4*)(dst + (g / (RT * 2)) * RP + (g % (RT * 2)) * 16) = br[i];
+    }
+  };
+
+  TileRegs tr;
+  lf_u32x4 br[(64 * RT * 2 + 255) / 256];
+  tile_load(tr, dY, (const uint8_t*)nullptr, N, blk * ROWS, Mrows, n_begin, tid, false);
+  load_b(br, n_begin);
   // S block -> LDS (rows beyond `valid` as zeros so they add nothing to dB)
-  for (int g = tid; g < ROWS * RT * 2; g += 256) {  // 16-byte granules, RT*2 per row
+  for (int g = tid; g < ROWS * RT * 2; g += 256) {
     const int row = g / (RT * 2), gc = g % (RT * 2);
     lf_u32x4 v = {0, 0, 0, 0};
     if (row < bi.valid) v = *(const lf_u32x4*)(S + (int64_t)(blk * ROWS + row) * R + gc * 8);
-    *(lf_u32x4*)(lds_s + row * RP + gc * 16) = v;
+    *(lf_u32x4*)(ss + row * RP + gc * 16) = v;
   }
+  tile_store(tr, ys, tid, false);
+  store_b(br, bs);
+  if (ntiles > 1) {
+    tile_load(tr, dY, (const uint8_t*)nullptr, N, blk * ROWS, Mrows, n_begin + 64, tid, false);
+    load_b(br, n_begin + 64);
+  }
+  __syncthreads();
 
   lf_f32x4 acc_ds[2][RT];
 #pragma unroll
@@ -213,72 +301,51 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
 #pragma unroll
     for (int c = 0; c < RT; c++) acc_ds[a][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
 
-  int64_t yrow[2];
+  for (int t = 0; t < ntiles; t++) {
+    const char* ycur = ys + (t & 1) * TILE_BYTES;
+    const char* bcur = bs + (t & 1) * 64 * RP;
+    // dS += dY_tile * B_tile : a = dY row fragment, b = B^T through the transpose read
 #pragma unroll
-  for (int rt = 0; rt < 2; rt++) yrow[rt] = min(blk * ROWS + wave * 32 + rt * 16 + li, Mrows - 1);
-
-  const int n_begin = ns * nslice, n_end = min(N, n_begin + nslice);
-  for (int nb = n_begin; nb < n_end; nb += 128) {
-    // dY chunk: this lane's fragments (row li of each 16-row tile, 32 contiguous columns)
-    lf_u32x4 yf[2][4];
+    for (int step = 0; step < 2; step++) {
+      lf_u32x4 yf[2];
 #pragma unroll
-    for (int rt = 0; rt < 2; rt++) {
-      const T* yp = dY + yrow[rt] * N + nb + qq * 32;
+      for (int rt = 0; rt < 2; rt++) yf[rt] = tile_row_frag(ycur, wave * 32 + rt * 16 + li, step * 4 + qq);
 #pragma unroll
-      for (int j = 0; j < 4; j++) yf[rt][j] = __builtin_nontemporal_load((const lf_u32x4*)(yp + 8 * j));
-    }
-    __syncthreads();  // previous chunk's LDS reads are done
+      for (int c = 0; c < RT; c++) {
+        const lf_u32x4 bf = tr_read8(bcur + (step * 32 + qq * 8 + j4) * RP + (c * 16 + 4 * c4) * 2, RP);
 #pragma unroll
-    for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        *(lf_u32x4*)(lds_dy + (wave * 32 + rt * 16 + li) * DYP + (qq * 32 + j * 8) * 2) = yf[rt][j];
-    // B chunk rows nb..nb+127 (rank columns, zero padded to R)
-    for (int g = tid; g < 128 * RT * 2; g += 256) {
-      const int row = g / (RT * 2), gc = g % (RT * 2);
-      lf_u32x4 v = {0, 0, 0, 0};
-      if (gc * 8 < bi.rank) v = *(const lf_u32x4*)(Bl + (int64_t)(nb + row) * bi.rank + gc * 8);
-      *(lf_u32x4*)(lds_b + row * RP + gc * 16) = v;
-    }
-    __syncthreads();
-
-    // dS += dY_chunk * B_chunk : a = dY fragment (registers), b = B^T via transpose read
-#pragma unroll
-    for (int c = 0; c < RT; c++) {
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const lf_u32x4 bf = tr_read8(lds_b + (qq * 32 + j * 8 + j4) * RP + (c * 16 + 4 * c4) * 2, RP);
-#pragma unroll
-        for (int rt = 0; rt < 2; rt++) acc_ds[rt][c] = Mfma16<T>::run(yf[rt][j], bf, acc_ds[rt][c]);
+        for (int rt = 0; rt < 2; rt++) acc_ds[rt][c] = Mfma16<T>::run(yf[rt], bf, acc_ds[rt][c]);
       }
     }
-    // dB chunk: D[n][r] = sum_m dY[m][n] S[m][r]; wave w owns columns 32w..32w+31 of the chunk
-    lf_f32x4 acc_db[2][RT];
+    // dB tile: D[n][r] = sum_m dY[m][n] S[m][r]; wave w owns columns 16w..16w+15 of the tile
+    lf_f32x4 acc_db[RT];
 #pragma unroll
-    for (int a = 0; a < 2; a++)
-#pragma unroll
-      for (int c = 0; c < RT; c++) acc_db[a][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < RT; c++) acc_db[c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) {
       const int mrow = kk * 32 + qq * 8 + j4;
-      lf_u32x4 sf[RT];
+      const lf_u32x4 yt = tile_tr_frag(ycur, mrow, wave * 16 + 4 * c4);
 #pragma unroll
-      for (int c = 0; c < RT; c++) sf[c] = tr_read8(lds_s + mrow * RP + (c * 16 + 4 * c4) * 2, RP);
-#pragma unroll
-      for (int nt = 0; nt < 2; nt++) {
-        const lf_u32x4 yt = tr_read8(lds_dy + mrow * DYP + (wave * 32 + nt * 16 + 4 * c4) * 2, DYP);
-#pragma unroll
-        for (int c = 0; c < RT; c++) acc_db[nt][c] = Mfma16<T>::run(yt, sf[c], acc_db[nt][c]);
+      for (int c = 0; c < RT; c++) {
+        const lf_u32x4 sf = tr_read8(ss + mrow * RP + (c * 16 + 4 * c4) * 2, RP);
+        acc_db[c] = Mfma16<T>::run(yt, sf, acc_db[c]);
       }
     }
-    float* dbo = db_part + ((int64_t)blk * N + nb) * R;
+    float* dbo = db_part + ((int64_t)blk * N + n_begin + t * 64) * R;
 #pragma unroll
-    for (int nt = 0; nt < 2; nt++)
+    for (int c = 0; c < RT; c++)
 #pragma unroll
-      for (int c = 0; c < RT; c++)
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-          dbo[(int64_t)(wave * 32 + nt * 16 + qq * 4 + e) * R + c * 16 + li] = acc_db[nt][c][e];
+      for (int e = 0; e < 4; e++) dbo[(int64_t)(wave * 16 + qq * 4 + e) * R + c * 16 + li] = acc_db[c][e];
+
+    if (t + 1 < ntiles) {
+      tile_store(tr, ys + ((t + 1) & 1) * TILE_BYTES, tid, false);
+      store_b(br, bs + ((t + 1) & 1) * 64 * RP);
+      if (t + 2 < ntiles) {
+        tile_load(tr, dY, (const uint8_t*)nullptr, N, blk * ROWS, Mrows, n_begin + (t + 2) * 64, tid, false);
+        load_b(br, n_begin + (t + 2) * 64);
+      }
+    }
+    __syncthreads();
   }
   float* dso = ds_part + (int64_t)ns * Mrows * R;
 #pragma unroll
@@ -292,121 +359,143 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
       }
 }
 
-// out_s[n][r] (r < rank_s) = cast( mult * sum over the segment's blocks of part[b][n][r] )
-//   mult_mode 0: block scale ; 1: 1/(1-p) of the block.  part is [n_blocks][rows][R].
-// Used for dB (rows = N, out [N, rank]) and dA (transposed flag: part [b][R][K], out [rank, K]).
-template <typename T>
-__global__ void __launch_bounds__(256)
-reduce_segments_kernel(const float* __restrict__ part, int rows, int R, int transposed, int mult_mode, int M,
-                       const LfSegTable seg) {
-  const int s = blockIdx.y;
-  const int rank = seg.table ? seg.rank[s] : seg.rank[0];
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into the output [rows, rank] or [rank, rows]
-  if (idx >= (int64_t)rows * rank) return;
-  int b0 = 0, b1;
-  float mult;
+// Blocks [b0, b1) of segment s.
+__device__ __forceinline__ void segment_blocks(const LfSegTable& seg, int s, int M, int& b0, int& b1) {
   if (seg.table == nullptr) {
+    b0 = 0;
     b1 = (M + ROWS - 1) / ROWS;
-    mult = mult_mode == 0 ? seg.scale : (seg.p > 0.f ? 1.f / (1.f - seg.p) : 1.f);
   } else {
     b0 = seg.first_block[s];
     b1 = (s + 1 < seg.n_seg) ? seg.first_block[s + 1] : seg.n_blocks;
+  }
+}
+
+// out_s = cast( mult * sum over parts of part[...] ) for segment s = blockIdx.y.
+//   transposed == 0 (dB): parts are the segment's blocks, part[b][n][R] -> out [rows, rank]
+//   transposed == 1 (dA): parts are the segment's chunks, part[(s*max_chunks + ch)][R][rows] -> out [rank, rows]
+//   mult_mode 0: segment scale ; 1: 1/(1-p) of the segment.
+template <typename T>
+__global__ void __launch_bounds__(256)
+reduce_segments_kernel(const float* __restrict__ part, int rows, int R, int transposed, int mult_mode, int M,
+                       int group, int max_chunks, const LfSegTable seg) {
+  const int s = blockIdx.y;
+  const int rank = seg.rank[s];
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into the output [rows, rank] or [rank, rows]
+  if (idx >= (int64_t)rows * rank) return;
+  int b0, b1;
+  segment_blocks(seg, s, M, b0, b1);
+  float mult;
+  if (seg.table == nullptr) {
+    mult = mult_mode == 0 ? seg.scale : (seg.p > 0.f ? 1.f / (1.f - seg.p) : 1.f);
+  } else {
     mult = mult_mode == 0 ? (seg.block_scale ? seg.block_scale[b0] : 1.f)
                           : ((seg.block_p && seg.block_p[b0] > 0.f) ? 1.f / (1.f - seg.block_p[b0]) : 1.f);
   }
-  int64_t pidx;
+  float v = 0.f;
   if (!transposed) {
     const int n = (int)(idx / rank), r = (int)(idx % rank);
-    pidx = (int64_t)n * R + r;
+    const int64_t pidx = (int64_t)n * R + r;
+    for (int b = b0; b < b1; b++) v += part[(int64_t)b * rows * R + pidx];
   } else {
     const int r = (int)(idx / rows), k = (int)(idx % rows);
-    pidx = (int64_t)r * rows + k;
+    const int64_t pidx = (int64_t)r * rows + k;
+    const int nch = (b1 - b0 + group - 1) / group;
+    for (int ch = 0; ch < nch; ch++) v += part[((int64_t)s * max_chunks + ch) * R * rows + pidx];
   }
-  float v = 0.f;
-  for (int b = b0; b < b1; b++) v += part[(int64_t)b * rows * R + pidx];
   ((uint16_t*)seg.out[s])[idx] = Mfma16<T>::cvt(v * mult);
 }
 
 // ------------------------------------------------------------------------------------ da
-// grid (n_blocks, K / kslice).  part[b][r][k] = sum over the block's rows of dS[m][r] * mask*X[m][k]
-// (without 1/(1-p); the reduce applies it).  dS block and X chunk are staged in LDS and both
-// read through the transpose path since the contraction index m is the slow dimension of both.
+// grid (K/64, max_chunks, n_seg).  Workgroup (kt, ch, s) owns the 64 columns kt*64.. of dA_s and
+// the `group` consecutive 128-row blocks ch*group.. of segment s; it accumulates
+//   D[r][k] = sum_m dS[m][r] * mask*X[m][k]     (1/(1-p) is applied by the reduce)
+// over its blocks and writes one fp32 partial [R][64].  Both operands are read from LDS through
+// the transpose path since the contraction index m is the slow dimension of both.
 template <typename T, int RT>
 __global__ void __launch_bounds__(256)
 lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const T* __restrict__ dS,
-               float* __restrict__ part, int M, int K, int R, int kslice, const LfSegTable seg) {
-  constexpr int XP = 288;
+               float* __restrict__ part, int M, int K, int R, int group, int max_chunks, const LfSegTable seg) {
   constexpr int RP = RT * 32 + 32;
-  __shared__ __attribute__((aligned(16))) char lds_x[ROWS * XP];
-  __shared__ __attribute__((aligned(16))) char lds_ds[ROWS * RP];
-  const int blk = blockIdx.x;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* xs = lds;
+  char* dss = lds + 2 * TILE_BYTES;
+  const int kt = blockIdx.x, ch = blockIdx.y, s = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, qq = lane >> 4, j4 = li >> 2, c4 = li & 3;
-  const BlockInfo bi = block_info(seg, blk, M);
-  const bool use_mask = mask != nullptr && bi.p > 0.f;
+  int b0, b1;
+  segment_blocks(seg, s, M, b0, b1);
+  const int bb0 = b0 + ch * group, bb1 = min(bb0 + group, b1);
+  if (bb0 >= b1) return;  // this segment has fewer chunks (uniform for the whole workgroup)
+  const float p = seg.table ? (seg.block_p ? seg.block_p[b0] : 0.f) : seg.p;
+  const bool use_mask = mask != nullptr && p > 0.f;
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
 
-  for (int g = tid; g < ROWS * RT * 2; g += 256) {
-    const int row = g / (RT * 2), gc = g % (RT * 2);
-    lf_u32x4 v = {0, 0, 0, 0};
-    if (row < bi.valid) v = *(const lf_u32x4*)(dS + (int64_t)(blk * ROWS + row) * R + gc * 8);
-    *(lf_u32x4*)(lds_ds + row * RP + gc * 16) = v;
-  }
-  int64_t xrow[2];
+  auto valid_rows = [&](int b) { return seg.table ? seg.table[3 * b + 1] : min(ROWS, M - b * ROWS); };
+  auto load_ds = [&](lf_u32x4 (&dr)[RT], int b) {
+    const int valid = valid_rows(b);
 #pragma unroll
-  for (int rt = 0; rt < 2; rt++) xrow[rt] = min(blk * ROWS + wave * 32 + rt * 16 + li, Mrows - 1);
-
-  const int k_begin = blockIdx.y * kslice, k_end = min(K, k_begin + kslice);
-  for (int kb = k_begin; kb < k_end; kb += 128) {
-    lf_u32x4 xf[2][4];
-#pragma unroll
-    for (int rt = 0; rt < 2; rt++) {
-      const T* xp = X + xrow[rt] * K + kb + qq * 32;
-#pragma unroll
-      for (int j = 0; j < 4; j++) xf[rt][j] = __builtin_nontemporal_load((const lf_u32x4*)(xp + 8 * j));
-      if (use_mask) {
-        const lf_u32x2* mp = (const lf_u32x2*)(mask + xrow[rt] * K + kb + qq * 32);
-#pragma unroll
-        for (int j = 0; j < 4; j++) xf[rt][j] = apply_mask8(xf[rt][j], __builtin_nontemporal_load(mp + j));
-      }
+    for (int i = 0; i < RT; i++) {
+      const int g = i * 256 + tid;
+      const int row = g / (RT * 2), gc = g % (RT * 2);
+      lf_u32x4 v = {0, 0, 0, 0};
+      if (row < valid) v = *(const lf_u32x4*)(dS + (int64_t)(b * ROWS + row) * R + gc * 8);
+      dr[i] = v;
     }
-    __syncthreads();
+  };
+  auto store_ds = [&](const lf_u32x4 (&dr)[RT], char* dst) {
 #pragma unroll
-    for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        *(lf_u32x4*)(lds_x + (wave * 32 + rt * 16 + li) * XP + (qq * 32 + j * 8) * 2) = xf[rt][j];
-    __syncthreads();
+    for (int i = 0; i < RT; i++) {
+      const int g = i * 256 + tid;
+      *(lf_u32x4*)(dst + (g / (RT * 2)) * RP + (g % (RT * 2)) * 16) = dr[i];
+    }
+  };
 
-    // D[r][k] = sum_m dS[m][r] X~[m][k]; wave w owns columns 32w..32w+31 of the chunk
-    lf_f32x4 acc[RT][2];
+  TileRegs tr;
+  lf_u32x4 dr[RT];
+  tile_load(tr, X, mask, K, bb0 * ROWS, Mrows, kt * 64, tid, use_mask);
+  load_ds(dr, bb0);
+  tile_store(tr, xs, tid, use_mask);
+  store_ds(dr, dss);
+  if (bb0 + 1 < bb1) {
+    tile_load(tr, X, mask, K, (bb0 + 1) * ROWS, Mrows, kt * 64, tid, use_mask);
+    load_ds(dr, bb0 + 1);
+  }
+  __syncthreads();
+
+  lf_f32x4 acc[RT];
 #pragma unroll
-    for (int c = 0; c < RT; c++)
-#pragma unroll
-      for (int a = 0; a < 2; a++) acc[c][a] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < RT; c++) acc[c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int b = bb0; b < bb1; b++) {
+    const int t = b - bb0;
+    const char* xcur = xs + (t & 1) * TILE_BYTES;
+    const char* dcur = dss + (t & 1) * ROWS * RP;
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) {
       const int mrow = kk * 32 + qq * 8 + j4;
-      lf_u32x4 df[RT];
+      const lf_u32x4 xt = tile_tr_frag(xcur, mrow, wave * 16 + 4 * c4);
 #pragma unroll
-      for (int c = 0; c < RT; c++) df[c] = tr_read8(lds_ds + mrow * RP + (c * 16 + 4 * c4) * 2, RP);
-#pragma unroll
-      for (int kt = 0; kt < 2; kt++) {
-        const lf_u32x4 xt = tr_read8(lds_x + mrow * XP + (wave * 32 + kt * 16 + 4 * c4) * 2, XP);
-#pragma unroll
-        for (int c = 0; c < RT; c++) acc[c][kt] = Mfma16<T>::run(df[c], xt, acc[c][kt]);
+      for (int c = 0; c < RT; c++) {
+        const lf_u32x4 df = tr_read8(dcur + mrow * RP + (c * 16 + 4 * c4) * 2, RP);
+        acc[c] = Mfma16<T>::run(df, xt, acc[c]);
       }
     }
-    // C layout: column (k) = lane & 15, rows (r) = 4*(lane >> 4) + e
-    float* po = part + (int64_t)blk * R * K;
-#pragma unroll
-    for (int c = 0; c < RT; c++)
-#pragma unroll
-      for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-          po[(int64_t)(c * 16 + qq * 4 + e) * K + kb + wave * 32 + kt * 16 + li] = acc[c][kt][e];
+    if (b + 1 < bb1) {
+      tile_store(tr, xs + ((t + 1) & 1) * TILE_BYTES, tid, use_mask);
+      store_ds(dr, dss + ((t + 1) & 1) * ROWS * RP);
+      if (b + 2 < bb1) {
+        tile_load(tr, X, mask, K, (b + 2) * ROWS, Mrows, kt * 64, tid, use_mask);
+        load_ds(dr, b + 2);
+      }
+    }
+    __syncthreads();
   }
+  // C layout: column (k) = lane & 15, rows (r) = 4*(lane >> 4) + e
+  float* po = part + ((int64_t)s * max_chunks + ch) * R * K;
+#pragma unroll
+  for (int c = 0; c < RT; c++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) po[(int64_t)(c * 16 + qq * 4 + e) * K + kt * 64 + wave * 16 + li] = acc[c][e];
 }
 
 int rt_of(int R) { return R <= 16 ? 1 : R <= 32 ? 2 : R <= 64 ? 4 : 8; }
@@ -415,31 +504,50 @@ int rt_of(int R) { return R <= 16 ? 1 : R <= 32 ? 2 : R <= 64 ? 4 : 8; }
 
 static int n_row_blocks(int M, const LfSegTable& seg) { return seg.table ? seg.n_blocks : (M + ROWS - 1) / ROWS; }
 
-// Split factor so that blocks * split fills the chip; slices are multiples of 128.
-static int pick_split(int nblk, int len) {
+// Split of a length-`len` axis into slices (multiples of 64) so that blocks * split fills the
+// chip; `min_split` bounds the slice length from above.
+static int pick_split(int nblk, int len, int min_split) {
   int split = 1;
-  while (nblk * split < 512 && len / (split * 2) >= 128 && (len % (split * 2 * 128)) == 0) split *= 2;
+  while (split < min_split && (len % (split * 2 * 64)) == 0) split *= 2;
+  while (nblk * split < 512 && len / (split * 2) >= 128 && (len % (split * 2 * 64)) == 0) split *= 2;
   return split;
 }
+
+static int xa_split(int nblk, int K, int R) { return pick_split(nblk, K, (K * rt_of(R) + 2047) / 2048); }
 
 size_t lf_xa_workspace(int M, int K, int R, const LfSegTable& seg) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  return (size_t)pick_split(nblk, K) * rows * R * sizeof(float);
+  return (size_t)xa_split(nblk, K, R) * rows * R * sizeof(float);
+}
+
+template <typename T, int RT>
+static int xa_launch(const void* X, const uint8_t* mask, float* part, int M, int K, int R, int kslice, dim3 grid,
+                     const LfSegTable& seg, hipStream_t st) {
+  auto kern = lora_xa_kernel<T, RT>;
+  const int smem = 2 * TILE_BYTES + RT * 16 * (kslice * 2 + 16);
+  if (smem > 160 * 1024) return LF_ESHAPE;
+  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return LF_ELAUNCH;
+  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)X, mask, part, M, K, R, kslice, seg);
+  return lf_check_launch();
 }
 
 template <typename T>
 static int xa_impl(const void* X, const uint8_t* mask, void* S, void* ws, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  const int split = pick_split(nblk, K);
+  const int split = xa_split(nblk, K, R);
   const int kslice = K / split;
   float* part = (float*)ws;
   dim3 grid(nblk, split);
-#define LF_XA(RT) hipLaunchKernelGGL((lora_xa_kernel<T, RT>), grid, dim3(256), 0, st, (const T*)X, mask, part, M, K, R, kslice, seg)
-  switch (rt_of(R)) { case 1: LF_XA(1); break; case 2: LF_XA(2); break; case 4: LF_XA(4); break; default: LF_XA(8); break; }
-#undef LF_XA
-  if (lf_check_launch() != LF_OK) return LF_ELAUNCH;
+  int rc;
+  switch (rt_of(R)) {
+    case 1: rc = xa_launch<T, 1>(X, mask, part, M, K, R, kslice, grid, seg, st); break;
+    case 2: rc = xa_launch<T, 2>(X, mask, part, M, K, R, kslice, grid, seg, st); break;
+    case 4: rc = xa_launch<T, 4>(X, mask, part, M, K, R, kslice, grid, seg, st); break;
+    default: rc = xa_launch<T, 8>(X, mask, part, M, K, R, kslice, grid, seg, st); break;
+  }
+  if (rc != LF_OK) return rc;
   const int64_t n = rows * R;
   hipLaunchKernelGGL((reduce_rows_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float*)part, (T*)S, split, M, R, 0, seg);
   return lf_check_launch();
@@ -459,22 +567,37 @@ int lf_launch_xa(const void* X, const uint8_t* mask, void* S, void* ws, size_t w
 size_t lf_dys_dyb_workspace(int M, int N, int R, const LfSegTable& seg) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  return ((size_t)pick_split(nblk, N) * rows * R + (size_t)nblk * N * R) * sizeof(float);
+  return ((size_t)pick_split(nblk, N, 1) * rows * R + (size_t)nblk * N * R) * sizeof(float);
+}
+
+template <typename T, int RT>
+static int dys_launch(const void* dY, const void* S, float* ds_part, float* db_part, int M, int N, int R, int nslice,
+                      dim3 grid, const LfSegTable& seg, hipStream_t st) {
+  auto kern = lora_dys_dyb_kernel<T, RT>;
+  constexpr int RP = RT * 32 + 32;
+  const int smem = 2 * TILE_BYTES + ROWS * RP + 2 * 64 * RP;
+  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return LF_ELAUNCH;
+  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, nslice, seg);
+  return lf_check_launch();
 }
 
 template <typename T>
 static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M, int N, int R, const LfSegTable& seg, hipStream_t st) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  const int split = pick_split(nblk, N);
+  const int split = pick_split(nblk, N, 1);
   const int nslice = N / split;
   float* ds_part = (float*)ws;
   float* db_part = ds_part + (int64_t)split * rows * R;
   dim3 grid(nblk, split);
-#define LF_DYS(RT) hipLaunchKernelGGL((lora_dys_dyb_kernel<T, RT>), grid, dim3(256), 0, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, nslice, seg)
-  switch (rt_of(R)) { case 1: LF_DYS(1); break; case 2: LF_DYS(2); break; case 4: LF_DYS(4); break; default: LF_DYS(8); break; }
-#undef LF_DYS
-  if (lf_check_launch() != LF_OK) return LF_ELAUNCH;
+  int rc;
+  switch (rt_of(R)) {
+    case 1: rc = dys_launch<T, 1>(dY, S, ds_part, db_part, M, N, R, nslice, grid, seg, st); break;
+    case 2: rc = dys_launch<T, 2>(dY, S, ds_part, db_part, M, N, R, nslice, grid, seg, st); break;
+    case 4: rc = dys_launch<T, 4>(dY, S, ds_part, db_part, M, N, R, nslice, grid, seg, st); break;
+    default: rc = dys_launch<T, 8>(dY, S, ds_part, db_part, M, N, R, nslice, grid, seg, st); break;
+  }
+  if (rc != LF_OK) return rc;
   const int64_t n = rows * R;
   hipLaunchKernelGGL((reduce_rows_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float*)ds_part, (T*)dS, split, M, R, 1, seg);
   if (lf_check_launch() != LF_OK) return LF_ELAUNCH;
@@ -482,7 +605,7 @@ static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M
   int maxrank = 0;
   for (int s = 0; s < nseg; s++) maxrank = seg.rank[s] > maxrank ? seg.rank[s] : maxrank;
   const int64_t nout = (int64_t)N * maxrank;
-  hipLaunchKernelGGL((reduce_segments_kernel<T>), dim3((unsigned)((nout + 255) / 256), nseg), dim3(256), 0, st, (const float*)db_part, N, R, 0, 0, M, seg);
+  hipLaunchKernelGGL((reduce_segments_kernel<T>), dim3((unsigned)((nout + 255) / 256), nseg), dim3(256), 0, st, (const float*)db_part, N, R, 0, 0, M, 1, 1, seg);
   return lf_check_launch();
 }
 
@@ -499,26 +622,59 @@ int lf_launch_dys_dyb(const void* dY, const void* S, void* dS, void* ws, size_t 
   return LF_EINVAL;
 }
 
+// dA chunking: `group` consecutive blocks per workgroup, chosen so the grid has >= ~1024 workgroups.
+static void da_shape(int M, int K, const LfSegTable& seg, int& group, int& max_chunks) {
+  const int nseg = seg.table ? seg.n_seg : 1;
+  int max_blocks = 0;
+  for (int s = 0; s < nseg; s++) {
+    int b0 = seg.table ? seg.first_block[s] : 0;
+    int b1 = seg.table ? ((s + 1 < nseg) ? seg.first_block[s + 1] : seg.n_blocks) : (M + ROWS - 1) / ROWS;
+    max_blocks = (b1 - b0) > max_blocks ? (b1 - b0) : max_blocks;
+  }
+  const int nblk = n_row_blocks(M, seg);
+  group = 8;
+  while (group > 1 && (int64_t)(K / 64) * ((nblk + group - 1) / group) < 1024) group /= 2;
+  max_chunks = (max_blocks + group - 1) / group;
+  if (max_chunks < 1) max_chunks = 1;
+}
+
 size_t lf_da_workspace(int M, int K, int R, const LfSegTable& seg) {
-  return (size_t)n_row_blocks(M, seg) * R * K * sizeof(float);
+  int group, max_chunks;
+  da_shape(M, K, seg, group, max_chunks);
+  const int nseg = seg.table ? seg.n_seg : 1;
+  return (size_t)nseg * max_chunks * R * K * sizeof(float);
+}
+
+template <typename T, int RT>
+static int da_launch(const void* X, const uint8_t* mask, const void* dS, float* part, int M, int K, int R, int group,
+                     int max_chunks, dim3 grid, const LfSegTable& seg, hipStream_t st) {
+  auto kern = lora_da_kernel<T, RT>;
+  constexpr int RP = RT * 32 + 32;
+  const int smem = 2 * TILE_BYTES + 2 * ROWS * RP;
+  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return LF_ELAUNCH;
+  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)X, mask, (const T*)dS, part, M, K, R, group, max_chunks, seg);
+  return lf_check_launch();
 }
 
 template <typename T>
 static int da_impl(const void* X, const uint8_t* mask, const void* dS, void* ws, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
-  const int nblk = n_row_blocks(M, seg);
-  const int split = pick_split(nblk, K);
-  const int kslice = K / split;
-  float* part = (float*)ws;
-  dim3 grid(nblk, split);
-#define LF_DA(RT) hipLaunchKernelGGL((lora_da_kernel<T, RT>), grid, dim3(256), 0, st, (const T*)X, mask, (const T*)dS, part, M, K, R, kslice, seg)
-  switch (rt_of(R)) { case 1: LF_DA(1); break; case 2: LF_DA(2); break; case 4: LF_DA(4); break; default: LF_DA(8); break; }
-#undef LF_DA
-  if (lf_check_launch() != LF_OK) return LF_ELAUNCH;
+  int group, max_chunks;
+  da_shape(M, K, seg, group, max_chunks);
   const int nseg = seg.table ? seg.n_seg : 1;
+  float* part = (float*)ws;
+  dim3 grid(K / 64, max_chunks, nseg);
+  int rc;
+  switch (rt_of(R)) {
+    case 1: rc = da_launch<T, 1>(X, mask, dS, part, M, K, R, group, max_chunks, grid, seg, st); break;
+    case 2: rc = da_launch<T, 2>(X, mask, dS, part, M, K, R, group, max_chunks, grid, seg, st); break;
+    case 4: rc = da_launch<T, 4>(X, mask, dS, part, M, K, R, group, max_chunks, grid, seg, st); break;
+    default: rc = da_launch<T, 8>(X, mask, dS, part, M, K, R, group, max_chunks, grid, seg, st); break;
+  }
+  if (rc != LF_OK) return rc;
   int maxrank = 0;
   for (int s = 0; s < nseg; s++) maxrank = seg.rank[s] > maxrank ? seg.rank[s] : maxrank;
   const int64_t nout = (int64_t)K * maxrank;
-  hipLaunchKernelGGL((reduce_segments_kernel<T>), dim3((unsigned)((nout + 255) / 256), nseg), dim3(256), 0, st, (const float*)part, K, R, 1, 1, M, seg);
+  hipLaunchKernelGGL((reduce_segments_kernel<T>), dim3((unsigned)((nout + 255) / 256), nseg), dim3(256), 0, st, (const float*)part, K, R, 1, 1, M, group, max_chunks, seg);
   return lf_check_launch();
 }
 
