@@ -139,6 +139,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -169,6 +171,13 @@ def main():
         x.grad = None
         for p in a_list + b_list:
             p.grad = None
+
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -212,6 +221,12 @@ def main():
     nf4_bytes = n / 2 + n / 64 + 4 * n / 16384 + 1028 + 2 * n
     nf4_gbs = nf4_bytes / (t_nf4 * 1e-3) / 1e9
 
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "gemm_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("dx_gemm_bytes_per_launch")
+
     res = {
         "metric": "fused LoRA fwd+bwd TFLOP/s (8B layer, r=16); NF4 dequant GB/s; % roofline",
         "value": round(value, 2),
@@ -233,7 +248,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma", "achieved": round(achieved, 2), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(achieved / BF16_PEAK_TFLOPS, 4), "traffic": None,
+            "frac": round(achieved / BF16_PEAK_TFLOPS, 4), "traffic": traffic,
             "kernel": dom_name, "launch_ms": round(dom_ms, 4), "flops_per_launch": gemm_flops,
         },
         "kernels_ms": {

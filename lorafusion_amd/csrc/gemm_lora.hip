@@ -13,20 +13,32 @@
 // and the dense K-loop adds on top of it in fp32.
 //
 // Structure: one workgroup per BMxBN tile, 64-wide wavefronts each owning a WMxWN sub-tile of
-// 32x32x16 MFMA blocks; BK = 64.  Both operand tiles go global -> LDS with 16-byte
-// direct-to-LDS loads (no VGPR staging), double buffered, one barrier per K step.  LDS rows
-// (128 bytes = 8 granules of 16 bytes) are XOR-swizzled with key (row>>1)&7 so that any 16
-// consecutive lanes of a ds_read_b128 fragment read (16 rows, one granule each) touch all 64
-// banks exactly once; the swizzle is applied on the global side of the direct load (each lane
-// picks the granule whose LDS slot it owns).  The NN operand is stored untransposed and read
-// with ds_read_b64_tr_b16, which hands each lane four consecutive contraction elements of
-// its column.  MFMA operands are swapped (B fragment as the "a" operand) so each lane ends
-// with four consecutive output columns of one row and stores 8 bytes at a time.
+// 32x32x16 MFMA blocks.  The K loop advances in steps of BK = 32 through a ring of NSTAGE LDS
+// stages; both operand tiles go global -> LDS with 16-byte direct-to-LDS buffer loads (no VGPR
+// staging, no vector ALU address work: the per-lane row offset is loop invariant and the K
+// position is a scalar offset).  NSTAGE-1 stages of loads are in flight while one stage is
+// consumed: with a single stage in flight the tile round trip under MFMA load (about twice
+// the unloaded one) is longer than the MFMA time of a K step and every step stalls on it
+// (measured: 1.18 -> 1.5 PFLOP/s on a loads+MFMA skeleton when a second stage may stay in
+// flight).  LDS rows are 64 bytes (4 granules of 16 bytes); granule g of row r is stored at
+// slot g ^ ((r>>2)&3) so that any 16 consecutive lanes of a ds_read_b128 fragment read (16
+// rows, one granule each) touch all 64 banks exactly once; the swizzle is applied on the
+// global side of the direct load (each lane fetches the granule whose LDS slot it owns).
+// The NN operand is stored untransposed and read with ds_read_b64_tr_b16, which hands each
+// lane four consecutive contraction elements of its column.  Fragments are double buffered
+// in registers (the reads of MFMA k-step ks+1 are issued before the MFMAs of ks) and each K
+// step has one barrier, placed between its two MFMA k-steps.  MFMA operands are swapped (B
+// fragment as the "a" operand) so each lane ends with four consecutive output columns of one
+// row and stores 8 bytes at a time.
 #include "lf_common.h"
+#include <type_traits>
 
 namespace {
 
-constexpr int BK = 64;
+constexpr int BK = 32;
+#ifndef LF_NSTAGE
+#define LF_NSTAGE 5
+#endif
 
 template <typename T> struct MfmaOp;
 template <> struct MfmaOp<__bf16> {
@@ -60,21 +72,22 @@ __device__ __forceinline__ void load_g2l_16(const void* g, char* lds_wave_base) 
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_wave_base, 16, 0, 0);
 }
 
-template <typename T, int BM, int BN, int WM, int WN, bool NN>
+template <typename T, int BM, int BN, int WM, int WN, bool NN, int NSTAGE>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64, 1)
 gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
-  constexpr int NWM = BM / WM, NWN = BN / WN, NTHREADS = NWM * NWN * 64;
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (buffer-resource types are device-only)
+  constexpr int NWM = BM / WM, NWN = BN / WN, NWAVES = NWM * NWN, NTHREADS = NWAVES * 64;
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int A_STAGE = BM * BK * 2, B_STAGE = BN * BK * 2;
-  constexpr int NLA = BM * 8 / NTHREADS;  // 16-byte loads per thread per A tile
-  constexpr int NLB = BN * 8 / NTHREADS;
-  static_assert(NLA >= 1 && NLB >= 1 && (NTHREADS / 8) % 8 == 0, "tile/thread shape");
+  constexpr int NLA = BM * 4 / NTHREADS;  // 16-byte loads per thread per A tile (rows of 4 granules)
+  constexpr int NLB = BN * 4 / NTHREADS;
+  static_assert(NLA >= 1 && NLB >= 1 && (NTHREADS / 4) % 16 == 0, "tile/thread shape");
   constexpr int GPR = BN / 8;             // NN: granules per LDS row of the B tile
   constexpr int BPITCH = BN * 2;          // NN: bytes per LDS row of the B tile
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   char* ldsA = smem;
-  char* ldsB = smem + 2 * A_STAGE;
+  char* ldsB = smem + NSTAGE * A_STAGE;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -95,34 +108,32 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   const int pid_n = (pid % width) / gsz;
   const int m0 = pid_m * BM, n0 = pid_n * BN;
 
-  const T* __restrict__ A = (const T*)p.A;
-  const T* __restrict__ B = (const T*)p.B;
-
   // ---- staggered start of the K loop: workgroups that run side by side walk K from different
   // offsets (one 128-byte step apart) so their tile loads spread over the memory channels
   // instead of all hitting the same channel when the row pitch is a power of two.
   const int nk = p.K / BK;
-  const int kstart = ((pid_m + pid_n) & 15) % nk;
-  const int wrap_at = nk - kstart;  // number of tiles issued before the pointers wrap to k = 0
+  const int kstart = (2 * ((pid_m + pid_n) & 15)) % nk;
 
-  // ---- per-thread global source pointers for the direct-to-LDS loads
-  const T* aptr[NLA];
-  const T* bptr[NLB];
+  // ---- direct-to-LDS buffer loads: per thread one 32-bit byte offset per 16-byte granule (row part,
+  // clamped at the matrix edge); the K position of a tile is a scalar offset shared by the wave.
+  const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, 0x7fffffff, 0x00020000);
+  uint32_t avoff[NLA], bvoff[NLB];
   {
-    const int r8 = (tid >> 4) & 7;
-    const int srcg = (tid & 7) ^ r8;  // swizzle: LDS slot (tid&7) of row r holds granule slot^((r>>1)&7)
+    // LDS slot (tid&3) of row r holds source granule slot ^ ((r>>2)&3); r>>2 = tid>>4 (mod 4)
+    const int srcg = (tid & 3) ^ ((tid >> 4) & 3);
 #pragma unroll
     for (int i = 0; i < NLA; i++) {
-      int row = i * (NTHREADS / 8) + (tid >> 3);
+      int row = i * (NTHREADS / 4) + (tid >> 2);
       int gm = min(m0 + row, p.M - 1);
-      aptr[i] = A + (int64_t)gm * p.lda + srcg * 8 + kstart * BK;
+      avoff[i] = (uint32_t)((int64_t)gm * p.lda * 2 + srcg * 16);
     }
     if constexpr (!NN) {
 #pragma unroll
       for (int i = 0; i < NLB; i++) {
-        int row = i * (NTHREADS / 8) + (tid >> 3);
+        int row = i * (NTHREADS / 4) + (tid >> 2);
         int gn = min(n0 + row, p.N - 1);
-        bptr[i] = B + (int64_t)gn * p.ldb + srcg * 8 + kstart * BK;
+        bvoff[i] = (uint32_t)((int64_t)gn * p.ldb * 2 + srcg * 16);
       }
     } else {
 #pragma unroll
@@ -131,33 +142,32 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         int row = gid / GPR, g = gid % GPR;
         int srcseg = (g >> 2) ^ (row & 3);
         int col = min(n0 + (srcseg * 4 + (g & 3)) * 8, p.N - 8);
-        bptr[i] = B + (int64_t)(row + kstart * BK) * p.ldb + col;
+        bvoff[i] = (uint32_t)((int64_t)row * p.ldb * 2 + col * 2);
       }
     }
   }
 
-  int issued = 0;
-  auto issue_loads = [&](int stage) {
+  constexpr int NL = NLA + NLB;  // loads per thread per K step
+  auto issue_loads = [&](int stage, int tile) {
     char* la = ldsA + stage * A_STAGE + wave * 1024;
     char* lb = ldsB + stage * B_STAGE + wave * 1024;
+    int kt_pos = kstart + tile;
+    if (kt_pos >= nk) kt_pos -= nk;
+    const int a_soff = kt_pos * (BK * 2);
+    const int b_soff = NN ? kt_pos * BK * (int)p.ldb * 2 : a_soff;
 #pragma unroll
-    for (int i = 0; i < NLA; i++) {
-      load_g2l_16(aptr[i], la + i * NTHREADS * 16);
-      aptr[i] += BK;
-    }
+    for (int i = 0; i < NLA; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_ptr_t)(la + i * NTHREADS * 16), 16, avoff[i], a_soff, 0, 0);
 #pragma unroll
-    for (int i = 0; i < NLB; i++) {
-      load_g2l_16(bptr[i], lb + i * NTHREADS * 16);
-      if constexpr (!NN) bptr[i] += BK; else bptr[i] += (int64_t)BK * p.ldb;
-    }
-    if (++issued == wrap_at) {
-#pragma unroll
-      for (int i = 0; i < NLA; i++) aptr[i] -= p.K;
-#pragma unroll
-      for (int i = 0; i < NLB; i++) {
-        if constexpr (!NN) bptr[i] -= p.K; else bptr[i] -= (int64_t)p.K * p.ldb;
-      }
-    }
+    for (int i = 0; i < NLB; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_ptr_t)(lb + i * NTHREADS * 16), 16, bvoff[i], b_soff, 0, 0);
+  };
+  // s_waitcnt vmcnt(n) with the other counters untouched (vmcnt = bits 3:0 and 15:14)
+  static_assert(NSTAGE >= 2 && NSTAGE <= 5 && 2 * NL < 64, "ring depth");
+  auto wait_loads = [&](int newer_stages) {
+    if (newer_stages <= 0) __builtin_amdgcn_s_waitcnt(0x0f70);
+    else if (newer_stages == 1) __builtin_amdgcn_s_waitcnt(0x0f70 | (NL & 15) | ((NL >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0f70 | ((2 * NL) & 15) | (((2 * NL) >> 4) << 14));
   };
 
   lf_f32x16 acc[TM][TN];
@@ -168,7 +178,9 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-  issue_loads(0);
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 2; t++)
+    if (t < nk) issue_loads(t, t);
 
   // ---- LoRA term seeds the accumulator (overlaps with the first tile's loads)
   const int wrow0 = m0 + wm * WM;  // first row of this wave's sub-tile
@@ -247,31 +259,24 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // ---- per-lane LDS fragment offsets
   int a_off[TM], b_off[TN];
 #pragma unroll
-  for (int i = 0; i < TM; i++) a_off[i] = (wm * WM + i * 32 + l32) * 128;
-  const int sw = (l32 >> 1) & 7;
-  int btr_key = 0, btr_in = 0;
+  for (int i = 0; i < TM; i++) a_off[i] = (wm * WM + i * 32 + l32) * 64;
+  const int sw = (l32 >> 2) & 3;
   if constexpr (!NN) {
 #pragma unroll
-    for (int j = 0; j < TN; j++) b_off[j] = (wn * WN + j * 32 + l32) * 128;
+    for (int j = 0; j < TN; j++) b_off[j] = (wn * WN + j * 32 + l32) * 64;
   } else {
     // ds_read_b64_tr_b16: within a 16-lane group, lane 4j+c addresses row j, columns 4c..4c+3 and
     // receives column (lane&15), rows 0..3.
     const int grp = lane >> 4, li = lane & 15, j4 = li >> 2, c = li & 3;
     const int row0 = (grp >> 1) * 8 + j4;
-    btr_key = row0 & 3;
+    const int key = row0 & 3;
 #pragma unroll
     for (int j = 0; j < TN; j++) {
       int colb = (wn * WN + j * 32 + (grp & 1) * 16 + 4 * c) * 2;  // byte offset within the row
-      b_off[j] = row0 * BPITCH + (((colb >> 6) ^ btr_key) << 6) + (colb & 63);
+      b_off[j] = row0 * BPITCH + (((colb >> 6) ^ key) << 6) + (colb & 63);
     }
-    (void)btr_in;
   }
 
-  // ---- main loop.  Fragments are double buffered in registers: the LDS reads of k-step ks+1 are
-  // issued before the MFMAs of k-step ks.  The single barrier of an iteration sits before the last
-  // k-step: by then every wave has read all of the current stage, so the next stage (whose loads
-  // were issued at the top of the iteration) can be read right after it and the current stage can
-  // be overwritten by the loads issued at the top of the next iteration.
   lf_u32x4 fa[2][TM], fb[2][TN];
   auto read_frags = [&](int buf, int stage, int ks) {
     const char* sa = ldsA + stage * A_STAGE;
@@ -299,69 +304,123 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
       for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(fb[buf][j], fa[buf][i], acc[i][j]);
   };
-  auto interleave = [&]() {  // scheduling hint: spread one k-step's LDS reads across its MFMAs
-    constexpr int NR = NN ? TM + 2 * TN : TM + TN, NM = TM * TN;
-    constexpr int PER = NM / NR > 0 ? NM / NR : 1;
-#pragma unroll
-    for (int r = 0; r < NR; r++) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, NM > PER * NR ? NM - PER * NR : 0, 0);
-  };
-
-  __builtin_amdgcn_s_waitcnt(0);  // all counters zero: the first tile has landed
-  __syncthreads();
-  read_frags(0, 0, 0);
-  for (int kt = 0; kt < nk; kt++) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) issue_loads(cur ^ 1);
-#pragma unroll
-    for (int ks = 0; ks < 3; ks++) {
-      read_frags((ks + 1) & 1, cur, ks + 1);
-      mfmas(ks & 1);
-      interleave();
-    }
-    __builtin_amdgcn_s_waitcnt(0);
+  // ---- main loop, two wave groups in anti-phase.  Each K step of a wave is a memory phase (issue
+  // its share of a later tile's loads, read all fragments of the current tile into registers)
+  // followed by a compute phase (the MFMAs of the step, nothing else); every phase ends in a
+  // workgroup barrier.  The second half of the waves runs one phase behind the first, so on every
+  // SIMD one wave feeds the MFMA pipe while its neighbour moves data: LDS latency never sits
+  // between two MFMAs of a wave, and the phases are long enough (16 MFMAs) that the schedule does
+  // not depend on instruction-level interleaving.
+  //   phase 2k   : group 0 reads tile k        | group 1 computes tile k-1
+  //   phase 2k+1 : group 0 computes tile k     | group 1 reads tile k
+  // Tile k is read in phases 2k and 2k+1.  Every wave waits for its own share of tile k at the end
+  // of its memory phase k-1 (phases 2k-2 / 2k-1), so the barrier closing phase 2k-1 publishes the
+  // whole tile.  The stage of tile k-1 is last read in phase 2k-1 and refilled (tile k+NSTAGE-1)
+  // from phase 2k on.  A load is in flight for 2*NSTAGE-4 phases.
+  const int grp = wave >= NWAVES / 2 ? 1 : 0;
+  auto phase_barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
-    if (kt + 1 < nk) read_frags(0, cur ^ 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // One K step of a wave.  The loads of step kt+NSTAGE-1 (into the stage of step kt-1, last read
+  // in phase 2kt-1) are issued from the compute phase, spread between the MFMAs: the texture
+  // addresser takes 16 cycles per 64-lane 16-byte load, and a burst of loads at the head of a
+  // memory phase (four waves of a CU at once) would hold those waves' LDS reads back behind it.
+  // LOAD: step kt+NSTAGE-1 exists.  NEWER: steps after kt+1 whose loads may still be in flight
+  // when the memory phase ends (step kt+1 itself must have landed).
+  using std::integral_constant;
+  int stage = 0, kt = 0;
+  auto k_step = [&](auto LOAD, auto NEWER) {
+    read_frags(0, stage, 0);
+    read_frags(1, stage, 1);
+    wait_loads(NEWER.value);
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): fragments are in registers
+    phase_barrier();
+    __builtin_amdgcn_s_setprio(1);
+    if constexpr (LOAD.value) issue_loads(stage == 0 ? NSTAGE - 1 : stage - 1, kt + NSTAGE - 1);
+    mfmas(0);
     mfmas(1);
-    interleave();
-  }
+    if constexpr (LOAD.value) {
+      constexpr int NM = 2 * TM * TN, PER = NM / NL;
+#pragma unroll
+      for (int r = 0; r < NL; r++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * NL, 0);
+    }
+    __builtin_amdgcn_s_setprio(0);
+    phase_barrier();
+    stage = stage + 1 == NSTAGE ? 0 : stage + 1;
+    kt++;
+  };
+  // steps 0..NSTAGE-3 were issued before the accumulator was seeded; step NSTAGE-2 is issued by
+  // the compute phase of step -1, which does not exist: issue it here.
+  if (NSTAGE - 2 < nk) issue_loads(NSTAGE - 2, NSTAGE - 2);
+  wait_loads(nk >= NSTAGE - 1 ? NSTAGE - 2 : nk - 1);
+  __syncthreads();
+  if (grp == 1) phase_barrier();
+  // at the end of memory phase kt the loads of steps kt+1 .. kt+NSTAGE-2 are outstanding
+  while (kt + NSTAGE - 1 < nk) k_step(integral_constant<bool, true>{}, integral_constant<int, NSTAGE - 3>{});
+  // tail: no more loads to issue; wait for everything that is still in flight
+  while (kt < nk) k_step(integral_constant<bool, false>{}, integral_constant<int, 0>{});
+  if (grp == 0) phase_barrier();
 
-  // ---- epilogue: bias, convert, 8-byte stores (4 consecutive columns of one row per lane)
+  // ---- epilogue: bias, convert, then one 32-row band of the wave's sub-tile at a time through the
+  // wave's own LDS region so that global stores are 16 bytes per lane and cover whole rows of
+  // the sub-tile (WN*2 contiguous bytes) instead of 8-byte pieces scattered over 32 rows.
+  // Granule g (16 bytes) of band row r sits at slot g ^ (r & 7).
   T* __restrict__ C = (T*)p.C;
   const uint16_t* bias16 = (const uint16_t*)p.bias;
+  constexpr int EP_PITCH = WN * 2;              // bytes per band row
+  constexpr int EP_BAND = 32 * EP_PITCH;        // bytes per band
+  constexpr int LPR = EP_PITCH / 16;            // lanes per row on the way out
+  constexpr int RPI = 64 / LPR;                 // rows per store instruction
+  static_assert(2 * NWAVES * EP_BAND <= NSTAGE * (A_STAGE + B_STAGE), "epilogue staging fits the ring");
+  __syncthreads();  // every wave is done with the ring
+  char* ep = smem + wave * (2 * EP_BAND);
+  float bv[TN][4][4];
+#pragma unroll
+  for (int j = 0; j < TN; j++)
+#pragma unroll
+    for (int jj = 0; jj < 4; jj++) {
+      const int gn = min(n0 + wn * WN + j * 32 + jj * 8 + q * 4, p.N - 4);
+#pragma unroll
+      for (int e = 0; e < 4; e++) bv[j][jj][e] = bias16 != nullptr ? MfmaOp<T>::to_float(bias16[gn + e]) : 0.f;
+    }
+  const int out_col = n0 + wn * WN + (lane % LPR) * 8;
 #pragma unroll
   for (int i = 0; i < TM; i++) {
-    const int gm = wrow0 + i * 32 + l32;
+    char* band = ep + (i & 1) * EP_BAND;
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
+    for (int j = 0; j < TN; j++)
 #pragma unroll
       for (int jj = 0; jj < 4; jj++) {
-        const int gn = n0 + wn * WN + j * 32 + jj * 8 + q * 4;
-        if (gm < p.M && gn < p.N) {
-          float v0 = acc[i][j][jj * 4 + 0], v1 = acc[i][j][jj * 4 + 1];
-          float v2 = acc[i][j][jj * 4 + 2], v3 = acc[i][j][jj * 4 + 3];
-          if (bias16 != nullptr) {
-            v0 += MfmaOp<T>::to_float(bias16[gn + 0]); v1 += MfmaOp<T>::to_float(bias16[gn + 1]);
-            v2 += MfmaOp<T>::to_float(bias16[gn + 2]); v3 += MfmaOp<T>::to_float(bias16[gn + 3]);
-          }
-          lf_u32x2 o = {MfmaOp<T>::pack2(v0, v1), MfmaOp<T>::pack2(v2, v3)};
-          *(lf_u32x2*)(C + (int64_t)gm * p.ldc + gn) = o;
-        }
+        lf_u32x2 o = {MfmaOp<T>::pack2(acc[i][j][jj * 4 + 0] + bv[j][jj][0], acc[i][j][jj * 4 + 1] + bv[j][jj][1]),
+                      MfmaOp<T>::pack2(acc[i][j][jj * 4 + 2] + bv[j][jj][2], acc[i][j][jj * 4 + 3] + bv[j][jj][3])};
+        const int g = j * 4 + jj;  // granule index within the band row; q selects its half
+        *(lf_u32x2*)(band + l32 * EP_PITCH + ((g ^ (l32 & 7)) << 4) + q * 8) = o;
       }
+#pragma unroll
+    for (int r = 0; r < 32 / RPI; r++) {
+      const int row = r * RPI + lane / LPR;
+      const int g = lane % LPR;
+      lf_u32x4 v = *(const lf_u32x4*)(band + row * EP_PITCH + ((g ^ (row & 7)) << 4));
+      const int gm = wrow0 + i * 32 + row;
+      if (gm < p.M && out_col < p.N) *(lf_u32x4*)(C + (int64_t)gm * p.ldc + out_col) = v;
     }
   }
+#endif
 }
 
-template <typename T, int BM, int BN, int WM, int WN, bool NN>
+template <typename T, int BM, int BN, int WM, int WN, bool NN, int NSTAGE>
 int launch_cfg(LfGemmParams p, const LfSegTable& seg, hipStream_t st) {
   constexpr int NTHREADS = (BM / WM) * (BN / WN) * 64;
-  constexpr int SMEM = 2 * (BM + BN) * BK * 2;
+  constexpr int SMEM = NSTAGE * (BM + BN) * BK * 2;
   p.grid_m = (p.M + BM - 1) / BM;
   p.grid_n = (p.N + BN - 1) / BN;
-  auto kern = gemm_lora_kernel<T, BM, BN, WM, WN, NN>;
+  auto kern = gemm_lora_kernel<T, BM, BN, WM, WN, NN, NSTAGE>;
   static bool attr_set = false;  // idempotent; a race only repeats the same call
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess) return LF_ELAUNCH;
@@ -375,11 +434,11 @@ template <typename T, bool NN>
 int launch_dtype(const LfGemmParams& p, const LfSegTable& seg, int cfg, hipStream_t st) {
   // Rows of one routing block must not straddle a wave's sub-tile: WM divides block_size_m.
   switch (cfg) {
-    case 0: return launch_cfg<T, 256, 256, 128, 128, NN>(p, seg, st);
-    case 1: return launch_cfg<T, 256, 256, 128, 64, NN>(p, seg, st);
-    case 2: return launch_cfg<T, 128, 256, 64, 128, NN>(p, seg, st);
-    case 3: return launch_cfg<T, 128, 256, 64, 64, NN>(p, seg, st);
-    case 4: return launch_cfg<T, 128, 128, 64, 64, NN>(p, seg, st);
+    case 0: return launch_cfg<T, 256, 256, 128, 128, NN, LF_NSTAGE>(p, seg, st);
+    case 1: return launch_cfg<T, 256, 256, 128, 64, NN, LF_NSTAGE>(p, seg, st);
+    case 2: return launch_cfg<T, 128, 256, 64, 128, NN, LF_NSTAGE>(p, seg, st);
+    case 3: return launch_cfg<T, 128, 256, 64, 64, NN, LF_NSTAGE>(p, seg, st);
+    case 4: return launch_cfg<T, 128, 128, 64, 64, NN, LF_NSTAGE>(p, seg, st);
     default: return LF_EINVAL;
   }
 }
@@ -411,8 +470,12 @@ static int choose_cfg(int M, int N, bool nn) {
 
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st) {
   if (p.M <= 0 || p.N <= 0 || p.K <= 0) return LF_EINVAL;
-  if (p.K % BK != 0 || p.N % 8 != 0 || p.N < 8) return LF_ESHAPE;
+  if (p.K % 64 != 0 || p.N % 8 != 0 || p.N < 8) return LF_ESHAPE;
+  // 16-byte output stores
+  if (p.ldc % 8 != 0 || ((uintptr_t)p.C & 15) != 0) return LF_ESHAPE;
   if (p.L != nullptr && (p.R % 16 != 0 || p.R <= 0 || p.R > LF_MAX_RANK)) return LF_ESHAPE;
+  // tile loads address the operands with 32-bit byte offsets
+  if ((int64_t)p.M * p.lda * 2 >= 0x7fffffffLL || (int64_t)(nn ? p.K : p.N) * p.ldb * 2 >= 0x7fffffffLL) return LF_ESHAPE;
   if (seg.table != nullptr && (seg.block_size_m % 64 != 0)) return LF_ESHAPE;
   int cfg = force_cfg >= 0 ? force_cfg : choose_cfg(p.M, p.N, nn);
   if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1)) cfg = 2;
