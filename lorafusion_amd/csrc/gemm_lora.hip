@@ -84,6 +84,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   static_assert(NLA >= 1 && NLB >= 1 && (NTHREADS / 4) % 16 == 0, "tile/thread shape");
   constexpr int GPR = BN / 8;             // NN: granules per LDS row of the B tile
   constexpr int BPITCH = BN * 2;          // NN: bytes per LDS row of the B tile
+  constexpr int BKEY = BPITCH / 64 >= 4 ? 3 : BPITCH / 64 - 1;  // NN: swizzle key mask over 64-byte segments
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   char* ldsA = smem;
@@ -140,7 +141,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
       for (int i = 0; i < NLB; i++) {
         int gid = i * NTHREADS + tid;
         int row = gid / GPR, g = gid % GPR;
-        int srcseg = (g >> 2) ^ (row & 3);
+        int srcseg = (g >> 2) ^ (row & BKEY);
         int col = min(n0 + (srcseg * 4 + (g & 3)) * 8, p.N - 8);
         bvoff[i] = (uint32_t)((int64_t)row * p.ldb * 2 + col * 2);
       }
@@ -191,7 +192,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     float mult = p.mult_mode == 0 ? seg.scale : (seg.p > 0.f ? 1.f / (1.f - seg.p) : 1.f);
     bool use_mask = p.mask != nullptr && p.mult_mode == 1 && seg.p > 0.f;
     if (seg.table != nullptr) {
-      int blk = wrow0 / seg.block_size_m;
+      int blk = (p.row0 + wrow0) / seg.block_size_m;
       blk = min(blk, seg.n_blocks - 1);
       rank = seg.table[3 * blk + 0];
       int fb = seg.table[3 * blk + 2];
@@ -269,7 +270,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     // receives column (lane&15), rows 0..3.
     const int grp = lane >> 4, li = lane & 15, j4 = li >> 2, c = li & 3;
     const int row0 = (grp >> 1) * 8 + j4;
-    const int key = row0 & 3;
+    const int key = row0 & BKEY;
 #pragma unroll
     for (int j = 0; j < TN; j++) {
       int colb = (wn * WN + j * 32 + (grp & 1) * 16 + 4 * c) * 2;  // byte offset within the row
@@ -370,13 +371,14 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // ---- epilogue: bias, convert, then one 32-row band of the wave's sub-tile at a time through the
   // wave's own LDS region so that global stores are 16 bytes per lane and cover whole rows of
   // the sub-tile (WN*2 contiguous bytes) instead of 8-byte pieces scattered over 32 rows.
-  // Granule g (16 bytes) of band row r sits at slot g ^ (r & 7).
+  // Granule g (16 bytes) of band row r sits at slot g ^ (r & EP_KEY).
   T* __restrict__ C = (T*)p.C;
   const uint16_t* bias16 = (const uint16_t*)p.bias;
   constexpr int EP_PITCH = WN * 2;              // bytes per band row
   constexpr int EP_BAND = 32 * EP_PITCH;        // bytes per band
   constexpr int LPR = EP_PITCH / 16;            // lanes per row on the way out
   constexpr int RPI = 64 / LPR;                 // rows per store instruction
+  constexpr int EP_KEY = LPR < 8 ? LPR - 1 : 7;
   static_assert(2 * NWAVES * EP_BAND <= NSTAGE * (A_STAGE + B_STAGE), "epilogue staging fits the ring");
   __syncthreads();  // every wave is done with the ring
   char* ep = smem + wave * (2 * EP_BAND);
@@ -400,13 +402,13 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         lf_u32x2 o = {MfmaOp<T>::pack2(acc[i][j][jj * 4 + 0] + bv[j][jj][0], acc[i][j][jj * 4 + 1] + bv[j][jj][1]),
                       MfmaOp<T>::pack2(acc[i][j][jj * 4 + 2] + bv[j][jj][2], acc[i][j][jj * 4 + 3] + bv[j][jj][3])};
         const int g = j * 4 + jj;  // granule index within the band row; q selects its half
-        *(lf_u32x2*)(band + l32 * EP_PITCH + ((g ^ (l32 & 7)) << 4) + q * 8) = o;
+        *(lf_u32x2*)(band + l32 * EP_PITCH + ((g ^ (l32 & EP_KEY)) << 4) + q * 8) = o;
       }
 #pragma unroll
     for (int r = 0; r < 32 / RPI; r++) {
       const int row = r * RPI + lane / LPR;
       const int g = lane % LPR;
-      lf_u32x4 v = *(const lf_u32x4*)(band + row * EP_PITCH + ((g ^ (row & 7)) << 4));
+      lf_u32x4 v = *(const lf_u32x4*)(band + row * EP_PITCH + ((g ^ (row & EP_KEY)) << 4));
       const int gm = wrow0 + i * 32 + row;
       if (gm < p.M && out_col < p.N) *(lf_u32x4*)(C + (int64_t)gm * p.ldc + out_col) = v;
     }
@@ -439,6 +441,7 @@ int launch_dtype(const LfGemmParams& p, const LfSegTable& seg, int cfg, hipStrea
     case 2: return launch_cfg<T, 128, 256, 64, 128, NN, LF_NSTAGE>(p, seg, st);
     case 3: return launch_cfg<T, 128, 256, 64, 64, NN, LF_NSTAGE>(p, seg, st);
     case 4: return launch_cfg<T, 128, 128, 64, 64, NN, LF_NSTAGE>(p, seg, st);
+    case 5: return launch_cfg<T, 64, 64, 32, 32, NN, LF_NSTAGE>(p, seg, st);
     default: return LF_EINVAL;
   }
 }
@@ -448,24 +451,45 @@ int launch_dtype(const LfGemmParams& p, const LfSegTable& seg, int cfg, hipStrea
 // Tile choice from a measured cost model: a launch runs in "rounds" of resident workgroups
 // (256 CUs x workgroups per CU); a full round of each configuration costs `unit` (relative to one
 // round of 256x256 tiles), a partly filled last round costs less than a full one.
-static int choose_cfg(int M, int N, bool nn) {
-  struct Cand { int cfg, bm, bn, slots; double unit_nt, unit_nn; };
-  static const Cand cands[3] = {
-      {1, 256, 256, 256, 1.000, 1.000},   // 8 waves, 128x64 per wave
-      {3, 128, 256, 256, 0.539, 0.645},   // 8 waves, 64x64 per wave
-      {4, 128, 128, 512, 0.550, 0.620},   // 4 waves, two workgroups per CU
-  };
+struct TileCand { int cfg, bm, bn, slots; double unit_nt, unit_nn; };
+static const TileCand kCands[] = {
+    {1, 256, 256, 256, 1.000, 1.000},   // 8 waves, 128x64 per wave
+    {3, 128, 256, 256, 0.539, 0.645},   // 8 waves, 64x64 per wave
+    {4, 128, 128, 512, 0.550, 0.620},   // 4 waves, two workgroups per CU
+    {5, 64, 64, 768, 0.200, 0.200},     // 4 waves, 32x32 per wave: only to spread a short row range
+};
+static double launch_cost(const TileCand& c, int M, int N, bool nn) {
+  const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+  const long full = tiles / c.slots;
+  const double fill = (double)(tiles % c.slots) / c.slots;
+  const double unit = nn ? c.unit_nn : c.unit_nt;
+  return unit * (full + (fill > 0 ? 0.45 + 0.55 * fill : 0.0));
+}
+static int choose_cfg(int M, int N, bool nn, double* cost_out = nullptr) {
   int best = 1;
   double best_cost = 1e30;
-  for (const Cand& c : cands) {
-    const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
-    const long full = tiles / c.slots;
-    const double fill = (double)(tiles % c.slots) / c.slots;
-    const double unit = nn ? c.unit_nn : c.unit_nt;
-    const double cost = unit * (full + (fill > 0 ? 0.45 + 0.55 * fill : 0.0));
+  for (const TileCand& c : kCands) {
+    const double cost = launch_cost(c, M, N, nn);
     if (cost < best_cost) { best_cost = cost; best = c.cfg; }
   }
+  if (cost_out) *cost_out = best_cost;
   return best;
+}
+// Rows [0, m_main) in whole rounds of 256x256 tiles, the rest as a second launch with the tile
+// that spreads it best, when that beats one launch (a nearly empty last round of big tiles
+// costs a full tile time).  Returns m_main (0: single launch).
+static int choose_split(int M, int N, bool nn, int* cfg_tail) {
+  constexpr double kLaunch = 0.03;  // a second launch, in units of a 256x256 round
+  const int grid_n = (N + 255) / 256;
+  if (grid_n > 256) return 0;
+  const int rows_per_round = (256 / grid_n) * 256;
+  const int m_main = (M / rows_per_round) * rows_per_round;
+  if (m_main <= 0 || m_main >= M) return 0;
+  double single, tail;
+  choose_cfg(M, N, nn, &single);
+  *cfg_tail = choose_cfg(M - m_main, N, nn, &tail);
+  const double split = launch_cost(kCands[0], m_main, N, nn) + tail + kLaunch;
+  return split < single ? m_main : 0;
 }
 
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st) {
@@ -477,9 +501,24 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
   // tile loads address the operands with 32-bit byte offsets
   if ((int64_t)p.M * p.lda * 2 >= 0x7fffffffLL || (int64_t)(nn ? p.K : p.N) * p.ldb * 2 >= 0x7fffffffLL) return LF_ESHAPE;
   if (seg.table != nullptr && (seg.block_size_m % 64 != 0)) return LF_ESHAPE;
-  int cfg = force_cfg >= 0 ? force_cfg : choose_cfg(p.M, p.N, nn);
-  if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1)) cfg = 2;
-  if (dtype == LF_BF16) return nn ? launch_dtype<__bf16, true>(p, seg, cfg, st) : launch_dtype<__bf16, false>(p, seg, cfg, st);
-  if (dtype == LF_F16) return nn ? launch_dtype<_Float16, true>(p, seg, cfg, st) : launch_dtype<_Float16, false>(p, seg, cfg, st);
-  return LF_EINVAL;
+  auto launch = [&](const LfGemmParams& q, int cfg) {
+    if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1)) cfg = 2;
+    if (dtype == LF_BF16) return nn ? launch_dtype<__bf16, true>(q, seg, cfg, st) : launch_dtype<__bf16, false>(q, seg, cfg, st);
+    if (dtype == LF_F16) return nn ? launch_dtype<_Float16, true>(q, seg, cfg, st) : launch_dtype<_Float16, false>(q, seg, cfg, st);
+    return (int)LF_EINVAL;
+  };
+  if (force_cfg >= 0) return launch(p, force_cfg);
+  int cfg_tail = 1;
+  const int m_main = choose_split(p.M, p.N, nn, &cfg_tail);
+  if (m_main == 0) return launch(p, choose_cfg(p.M, p.N, nn));
+  LfGemmParams head = p, tail = p;
+  head.M = m_main;
+  tail.M = p.M - m_main;
+  tail.row0 = p.row0 + m_main;
+  tail.A = (const char*)p.A + (int64_t)m_main * p.lda * 2;
+  tail.C = (char*)p.C + (int64_t)m_main * p.ldc * 2;
+  if (p.L != nullptr) tail.L = (const char*)p.L + (int64_t)m_main * p.R * 2;
+  if (p.mask != nullptr) tail.mask = p.mask + (int64_t)m_main * p.ldmask;
+  const int rc = launch(head, 1);
+  return rc != LF_OK ? rc : launch(tail, cfg_tail);
 }

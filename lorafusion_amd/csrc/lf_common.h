@@ -48,6 +48,7 @@ struct LfGemmParams {
   int64_t ldmask;
   int mult_mode;      // 0: LoRA term * scale ; 1: LoRA term * 1/(1-p), masked where p > 0
   int grid_m, grid_n;
+  int row0;           // global row of local row 0 (routing lookup when a launch covers a row range)
 };
 
 // launchers (one per translation unit)
