@@ -36,6 +36,9 @@
 namespace {
 
 constexpr int BK = 32;
+#ifndef LF_NSTAGE_SMALL
+#define LF_NSTAGE_SMALL 10
+#endif
 #ifndef LF_NSTAGE
 #define LF_NSTAGE 5
 #endif
@@ -70,6 +73,17 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 __device__ __forceinline__ void load_g2l_16(const void* g, char* lds_wave_base) {
   // 16 bytes per lane, global -> LDS; the LDS destination is lds_wave_base + lane*16.
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_wave_base, 16, 0, 0);
+}
+
+// ds_read_b64_tr_b16 as inline assembly: through the builtin the compiler cannot tell the read
+// from the direct-to-LDS loads still in flight and puts s_waitcnt vmcnt(0) in front of it, which
+// serialises the whole load ring.  The result is valid only after a later s_waitcnt lgkmcnt(0)
+// (the main loop has one before every barrier).
+__device__ __forceinline__ lf_u32x2 lds_read_tr16(const char* p) {
+  lf_u32x2 v;
+  const uint32_t a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(a) : "memory");
+  return v;
 }
 
 template <typename T, int BM, int BN, int WM, int WN, bool NN, int NSTAGE>
@@ -164,11 +178,18 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_ptr_t)(lb + i * NTHREADS * 16), 16, bvoff[i], b_soff, 0, 0);
   };
   // s_waitcnt vmcnt(n) with the other counters untouched (vmcnt = bits 3:0 and 15:14)
-  static_assert(NSTAGE >= 2 && NSTAGE <= 5 && 2 * NL < 64, "ring depth");
+  static_assert(NSTAGE >= 3 && (NSTAGE - 2) * NL < 64, "ring depth");
+  // wait until at most `newer_stages` whole steps of loads are outstanding (clamped to what the
+  // 6-bit counter and the ring allow: waiting for more than asked is always safe)
   auto wait_loads = [&](int newer_stages) {
-    if (newer_stages <= 0) __builtin_amdgcn_s_waitcnt(0x0f70);
-    else if (newer_stages == 1) __builtin_amdgcn_s_waitcnt(0x0f70 | (NL & 15) | ((NL >> 4) << 14));
-    else __builtin_amdgcn_s_waitcnt(0x0f70 | ((2 * NL) & 15) | (((2 * NL) >> 4) << 14));
+    constexpr int MAXS = NSTAGE - 2;
+    constexpr auto imm = [](int n) constexpr { return 0x0f70 | (n & 15) | ((n >> 4) << 14); };
+    if (newer_stages <= 0) __builtin_amdgcn_s_waitcnt(imm(0));
+    else if (newer_stages == 1) __builtin_amdgcn_s_waitcnt(imm(NL));
+    else if (newer_stages == 2 || MAXS <= 2) __builtin_amdgcn_s_waitcnt(imm((MAXS < 2 ? MAXS : 2) * NL));
+    else if (newer_stages < MAXS - 1 || MAXS <= 3) __builtin_amdgcn_s_waitcnt(imm((MAXS < 3 ? MAXS : 3) * NL));
+    else if (newer_stages == MAXS - 1) __builtin_amdgcn_s_waitcnt(imm((MAXS - 1) * NL));
+    else __builtin_amdgcn_s_waitcnt(imm(MAXS * NL));
   };
 
   lf_f32x16 acc[TM][TN];
@@ -278,7 +299,8 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     }
   }
 
-  lf_u32x4 fa[2][TM], fb[2][TN];
+  lf_u32x4 fa[4][TM], fb[4][TN];  // [set * 2 + k-slice]; the anti-phase loop uses one set
+  lf_u32x2 fbt[4][TN][2];  // NN: halves of the B fragments, joined only after the wait that completes them
   auto read_frags = [&](int buf, int stage, int ks) {
     const char* sa = ldsA + stage * A_STAGE;
     const char* sb = ldsB + stage * B_STAGE;
@@ -292,19 +314,67 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         const char* base = sb + b_off[j] + ks * 16 * BPITCH;
-        lf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(base));
-        lf_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(base + 4 * BPITCH));
-        lf_u32x2 lo2 = __builtin_bit_cast(lf_u32x2, lo), hi2 = __builtin_bit_cast(lf_u32x2, hi);
-        fb[buf][j] = lf_u32x4{lo2[0], lo2[1], hi2[0], hi2[1]};
+        fbt[buf][j][0] = lds_read_tr16(base);
+        fbt[buf][j][1] = lds_read_tr16(base + 4 * BPITCH);
       }
     }
   };
   auto mfmas = [&](int buf) {
+    if constexpr (NN) {
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[buf][j] = lf_u32x4{fbt[buf][j][0][0], fbt[buf][j][0][1], fbt[buf][j][1][0], fbt[buf][j][1][1]};
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
       for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(fb[buf][j], fa[buf][i], acc[i][j]);
   };
+  if constexpr (NWAVES <= 4) {
+    // ---- main loop, one wave per SIMD: no neighbour to hide behind, so the fragments of step
+    // kt+1 are read into a second register set while the MFMAs of step kt run; one barrier per
+    // step.  At the top of step kt: tile kt is in registers, tile kt+1 has landed and is visible,
+    // every wave has finished reading the stage of tile kt-1.
+    using std::integral_constant;
+    int stage = 0, kt = 0;
+    auto k_step = [&](auto SET, auto LOAD, auto NEXT, auto NEWER) {
+      constexpr int cur = SET.value, nxt = 1 - SET.value;
+      const int s1 = stage + 1 == NSTAGE ? 0 : stage + 1;
+      if (LOAD.value || kt + NSTAGE - 1 < nk) issue_loads(stage == 0 ? NSTAGE - 1 : stage - 1, kt + NSTAGE - 1);
+      if constexpr (NEXT.value) {
+        read_frags(nxt * 2 + 0, s1, 0);
+        read_frags(nxt * 2 + 1, s1, 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // reads go out before the MFMAs that cover their latency
+      mfmas(cur * 2 + 0);
+      mfmas(cur * 2 + 1);
+      wait_loads(NEWER.value);             // tile kt+2 has landed
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): next fragments are in registers
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      stage = s1;
+      kt++;
+    };
+    using T_ = integral_constant<bool, true>;
+    using F_ = integral_constant<bool, false>;
+    if (NSTAGE - 2 < nk) issue_loads(NSTAGE - 2, NSTAGE - 2);
+    wait_loads(nk > 2 ? NSTAGE - 3 : 0);  // tiles 0 and 1
+    __syncthreads();
+    read_frags(0, 0, 0);
+    read_frags(1, 0, 1);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    while (kt + NSTAGE < nk) {  // two steps per trip: the register sets swap roles
+      k_step(integral_constant<int, 0>{}, T_{}, T_{}, integral_constant<int, NSTAGE - 3>{});
+      k_step(integral_constant<int, 1>{}, T_{}, T_{}, integral_constant<int, NSTAGE - 3>{});
+    }
+    // tail (an even number of steps is left: nk is even): wait for everything
+    while (kt + 2 < nk) {
+      k_step(integral_constant<int, 0>{}, F_{}, T_{}, integral_constant<int, 0>{});
+      k_step(integral_constant<int, 1>{}, F_{}, T_{}, integral_constant<int, 0>{});
+    }
+    k_step(integral_constant<int, 0>{}, F_{}, T_{}, integral_constant<int, 0>{});
+    k_step(integral_constant<int, 1>{}, F_{}, F_{}, integral_constant<int, 0>{});
+  } else {
   // ---- main loop, two wave groups in anti-phase.  Each K step of a wave is a memory phase (issue
   // its share of a later tile's loads, read all fragments of the current tile into registers)
   // followed by a compute phase (the MFMAs of the step, nothing else); every phase ends in a
@@ -367,6 +437,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // tail: no more loads to issue; wait for everything that is still in flight
   while (kt < nk) k_step(integral_constant<bool, false>{}, integral_constant<int, 0>{});
   if (grp == 0) phase_barrier();
+  }
 
   // ---- epilogue: bias, convert, then one 32-row band of the wave's sub-tile at a time through the
   // wave's own LDS region so that global stores are 16 bytes per lane and cover whole rows of
@@ -441,35 +512,38 @@ int launch_dtype(const LfGemmParams& p, const LfSegTable& seg, int cfg, hipStrea
     case 2: return launch_cfg<T, 128, 256, 64, 128, NN, LF_NSTAGE>(p, seg, st);
     case 3: return launch_cfg<T, 128, 256, 64, 64, NN, LF_NSTAGE>(p, seg, st);
     case 4: return launch_cfg<T, 128, 128, 64, 64, NN, LF_NSTAGE>(p, seg, st);
-    case 5: return launch_cfg<T, 64, 64, 32, 32, NN, LF_NSTAGE>(p, seg, st);
+    case 5: return launch_cfg<T, 64, 64, 32, 32, NN, LF_NSTAGE_SMALL>(p, seg, st);
     default: return LF_EINVAL;
   }
 }
 
 }  // namespace
 
-// Tile choice from a measured cost model: a launch runs in "rounds" of resident workgroups
-// (256 CUs x workgroups per CU); a full round of each configuration costs `unit` (relative to one
-// round of 256x256 tiles), a partly filled last round costs less than a full one.
-struct TileCand { int cfg, bm, bn, slots; double unit_nt, unit_nn; };
+// Tile choice from a measured cost model.  A launch runs in "rounds" of resident workgroups
+// (256 CUs x workgroups per CU).  Costs are microseconds measured at K = 4096 (the choice only
+// compares configurations at equal K): the first round costs lat0 + first_b * fill^2 (a lone
+// tile per CU runs latency bound at boost clock, a full round is power limited), every further
+// round next_a + next_b * fill, where fill is the occupied fraction of the round's slots.
+struct TileCand { int cfg, bm, bn, slots; double lat0, first_b, next_a, next_b; };
 static const TileCand kCands[] = {
-    {1, 256, 256, 256, 1.000, 1.000},   // 8 waves, 128x64 per wave
-    {3, 128, 256, 256, 0.539, 0.645},   // 8 waves, 64x64 per wave
-    {4, 128, 128, 512, 0.550, 0.620},   // 4 waves, two workgroups per CU
-    {5, 64, 64, 768, 0.200, 0.200},     // 4 waves, 32x32 per wave: only to spread a short row range
+    {1, 256, 256, 256, 66.0, 50.0, 44.0, 60.0},   // 8 waves, 128x64 per wave
+    {3, 128, 256, 256, 48.0, 28.0, 28.0, 38.0},   // 8 waves, 64x64 per wave
+    {4, 128, 128, 512, 38.0, 47.0, 5.0, 70.0},    // 4 waves, two workgroups per CU
+    {5, 64, 64, 512, 21.0, 15.0, 13.0, 18.0},     // 4 waves, 32x32 per wave: spreads a short row range
 };
-static double launch_cost(const TileCand& c, int M, int N, bool nn) {
+static double launch_cost(const TileCand& c, int M, int N) {
   const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+  if (tiles <= 0) return 0.0;
   const long full = tiles / c.slots;
   const double fill = (double)(tiles % c.slots) / c.slots;
-  const double unit = nn ? c.unit_nn : c.unit_nt;
-  return unit * (full + (fill > 0 ? 0.45 + 0.55 * fill : 0.0));
+  if (full == 0) return c.lat0 + c.first_b * fill * fill;
+  return c.lat0 + c.first_b + (full - 1) * (c.next_a + c.next_b) + (fill > 0 ? c.next_a + c.next_b * fill : 0.0);
 }
-static int choose_cfg(int M, int N, bool nn, double* cost_out = nullptr) {
+static int choose_cfg(int M, int N, double* cost_out = nullptr) {
   int best = 1;
   double best_cost = 1e30;
   for (const TileCand& c : kCands) {
-    const double cost = launch_cost(c, M, N, nn);
+    const double cost = launch_cost(c, M, N);
     if (cost < best_cost) { best_cost = cost; best = c.cfg; }
   }
   if (cost_out) *cost_out = best_cost;
@@ -478,17 +552,17 @@ static int choose_cfg(int M, int N, bool nn, double* cost_out = nullptr) {
 // Rows [0, m_main) in whole rounds of 256x256 tiles, the rest as a second launch with the tile
 // that spreads it best, when that beats one launch (a nearly empty last round of big tiles
 // costs a full tile time).  Returns m_main (0: single launch).
-static int choose_split(int M, int N, bool nn, int* cfg_tail) {
-  constexpr double kLaunch = 0.03;  // a second launch, in units of a 256x256 round
+static int choose_split(int M, int N, int* cfg_tail) {
+  constexpr double kLaunch = 4.0;  // a second launch
   const int grid_n = (N + 255) / 256;
   if (grid_n > 256) return 0;
   const int rows_per_round = (256 / grid_n) * 256;
   const int m_main = (M / rows_per_round) * rows_per_round;
   if (m_main <= 0 || m_main >= M) return 0;
   double single, tail;
-  choose_cfg(M, N, nn, &single);
-  *cfg_tail = choose_cfg(M - m_main, N, nn, &tail);
-  const double split = launch_cost(kCands[0], m_main, N, nn) + tail + kLaunch;
+  choose_cfg(M, N, &single);
+  *cfg_tail = choose_cfg(M - m_main, N, &tail);
+  const double split = launch_cost(kCands[0], m_main, N) + tail + kLaunch;
   return split < single ? m_main : 0;
 }
 
@@ -509,8 +583,8 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
   };
   if (force_cfg >= 0) return launch(p, force_cfg);
   int cfg_tail = 1;
-  const int m_main = choose_split(p.M, p.N, nn, &cfg_tail);
-  if (m_main == 0) return launch(p, choose_cfg(p.M, p.N, nn));
+  const int m_main = choose_split(p.M, p.N, &cfg_tail);
+  if (m_main == 0) return launch(p, choose_cfg(p.M, p.N));
   LfGemmParams head = p, tail = p;
   head.M = m_main;
   tail.M = p.M - m_main;
