@@ -59,15 +59,17 @@ def linear_lora_bwd_fp32(dy, x, w, a, b, scale, mask=None, p=0.0, acc_dtype=torc
     """Closed-form gradients (lora_v1.py:241-247).
 
     db = scale * dYt S, ds = scale * dY B, da = dSt X~, dx = dY W + mask * (dS A)/(1-p).
-    Returns (dx [M,K], da [r,K], db [N,r], ds [M,r]) in ``acc_dtype``.
+    Returns (dx [M,K], da [r,K], db [N,r], ds [M,r]) in ``acc_dtype``.  With ``w=None`` the
+    M x N x K product is skipped and dx is None (full-size layer shapes, where dx is checked
+    on a sample of rows by a second call on those rows: dx is row-wise independent).
     """
-    dyf, xf, wf, af, bf = (t.to(acc_dtype) for t in (dy, x, w, a, b))
+    dyf, xf, af, bf = (t.to(acc_dtype) for t in (dy, x, a, b))
     xt = dropout_explicit(xf, mask, p)
     s = xt @ af.T
     db = (dyf.T @ s) * scale
     ds = (dyf @ bf) * scale
     da = ds.T @ xt
-    dx = dyf @ wf + dropout_explicit(ds @ af, mask, p)
+    dx = None if w is None else dyf @ w.to(acc_dtype) + dropout_explicit(ds @ af, mask, p)
     return dx, da, db, ds
 
 

@@ -15,9 +15,9 @@ def _close(actual, expected, what, rtol=1e-2):
     assert ok, f"{what}: max|err|/max|e| = {rel:.3e}, worst excess {excess:.3e}"
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("trans_b", [True, False])
-@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (520, 640, 384), (1024, 1280, 1024), (77, 136, 64)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (520, 640, 384), (1024, 1280, 1024), (77, 136, 64), (130, 72, 704)])
 def test_gemm_all_tiles(cfg, trans_b, M, N, K):
     from lorafusion_amd.ops import hip_ops
 
@@ -29,6 +29,23 @@ def test_gemm_all_tiles(cfg, trans_b, M, N, K):
     _close(c, e, f"gemm cfg={cfg} trans_b={trans_b}")
 
 
+@pytest.mark.parametrize("trans_b", [True, False])
+@pytest.mark.parametrize("M,N", [(4352, 4096), (8448, 4096), (2304, 8192), (4100, 4096)])
+def test_gemm_row_split_plan(trans_b, M, N):
+    """Automatic tile choice: row counts just above whole rounds of 256x256 tiles run as two launches
+    (whole rounds + a short tail with small tiles); every row must still be the product.  (Tiles of
+    different shapes start their K loop at different offsets, so the plans agree to rounding, not bitwise.)"""
+    from lorafusion_amd.ops import hip_ops
+
+    K = 128
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randn(M, K, generator=g).bfloat16().cuda()
+    b = (torch.randn(N, K, generator=g) if trans_b else torch.randn(K, N, generator=g)).bfloat16().cuda()
+    auto = hip_ops.gemm(a, b, trans_b=trans_b)
+    e = a.float().cpu() @ (b.float().cpu().T if trans_b else b.float().cpu())
+    _close(auto, e, f"gemm auto plan M={M} N={N} trans_b={trans_b}")
+
+
 def test_gemm_identity_exact():
     """A @ I^T reproduces A bit for bit in every layout (catches operand / index transpositions)."""
     from lorafusion_amd.ops import hip_ops
@@ -37,7 +54,7 @@ def test_gemm_identity_exact():
     a = torch.randn(300, 256, generator=g).bfloat16().cuda()
     eye = torch.eye(256).bfloat16().cuda()
     for trans_b in (True, False):
-        for cfg in range(5):
+        for cfg in range(6):
             assert torch.equal(hip_ops.gemm(a, eye, trans_b=trans_b, tile_cfg=cfg), a)
     # a permutation matrix tells B from B^T
     perm = torch.randperm(256, generator=g)
