@@ -36,6 +36,9 @@
 namespace {
 
 constexpr int BK = 32;
+#ifndef LF_STAG
+#define LF_STAG 15
+#endif
 #ifndef LF_NSTAGE_SMALL
 #define LF_NSTAGE_SMALL 10
 #endif
@@ -127,7 +130,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // offsets (one 128-byte step apart) so their tile loads spread over the memory channels
   // instead of all hitting the same channel when the row pitch is a power of two.
   const int nk = p.K / BK;
-  const int kstart = (2 * ((pid_m + pid_n) & 15)) % nk;
+  const int kstart = (2 * ((pid_m + pid_n) & LF_STAG)) % nk;
 
   // ---- direct-to-LDS buffer loads: per thread one 32-bit byte offset per 16-byte granule (row part,
   // clamped at the matrix edge); the K position of a tile is a scalar offset shared by the wave.
@@ -177,20 +180,30 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     for (int i = 0; i < NLB; i++)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_ptr_t)(lb + i * NTHREADS * 16), 16, bvoff[i], b_soff, 0, 0);
   };
-  // s_waitcnt vmcnt(n) with the other counters untouched (vmcnt = bits 3:0 and 15:14)
-  static_assert(NSTAGE >= 3 && (NSTAGE - 2) * NL < 64, "ring depth");
-  // wait until at most `newer_stages` whole steps of loads are outstanding (clamped to what the
-  // 6-bit counter and the ring allow: waiting for more than asked is always safe)
-  auto wait_loads = [&](int newer_stages) {
-    constexpr int MAXS = NSTAGE - 2;
-    constexpr auto imm = [](int n) constexpr { return 0x0f70 | (n & 15) | ((n >> 4) << 14); };
-    if (newer_stages <= 0) __builtin_amdgcn_s_waitcnt(imm(0));
-    else if (newer_stages == 1) __builtin_amdgcn_s_waitcnt(imm(NL));
-    else if (newer_stages == 2 || MAXS <= 2) __builtin_amdgcn_s_waitcnt(imm((MAXS < 2 ? MAXS : 2) * NL));
-    else if (newer_stages < MAXS - 1 || MAXS <= 3) __builtin_amdgcn_s_waitcnt(imm((MAXS < 3 ? MAXS : 3) * NL));
-    else if (newer_stages == MAXS - 1) __builtin_amdgcn_s_waitcnt(imm((MAXS - 1) * NL));
-    else __builtin_amdgcn_s_waitcnt(imm(MAXS * NL));
+  // one of the NL loads of a step (idx < NLA: operand A)
+  auto issue_load_one = [&](int stage, int tile, int idx) {
+    int kt_pos = kstart + tile;
+    if (kt_pos >= nk) kt_pos -= nk;
+    const int a_soff = kt_pos * (BK * 2);
+    if (idx < NLA) {
+      char* la = ldsA + stage * A_STAGE + wave * 1024;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_ptr_t)(la + idx * NTHREADS * 16), 16, avoff[idx < NLA ? idx : 0], a_soff, 0, 0);
+    } else {
+      const int i = idx - NLA;
+      char* lb = ldsB + stage * B_STAGE + wave * 1024;
+      const int b_soff = NN ? kt_pos * BK * (int)p.ldb * 2 : a_soff;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_ptr_t)(lb + i * NTHREADS * 16), 16, bvoff[i >= 0 && i < NLB ? i : 0], b_soff, 0, 0);
+    }
   };
+  // s_waitcnt vmcnt(n) with the other counters untouched (vmcnt = bits 3:0 and 15:14): wait until
+  // at most STEPS whole K steps of this thread's loads are outstanding
+  auto wait_loads = [&](auto STEPS) {
+    constexpr int n = STEPS.value * NL;
+    static_assert(n >= 0 && n < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+  };
+  using std::integral_constant;
+  using Steps0 = integral_constant<int, 0>;
 
   lf_f32x16 acc[TM][TN];
 #pragma unroll
@@ -200,8 +213,14 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
+  // K steps are loaded in pairs (2T, 2T+1): the two 64-byte halves of the same 128-byte lines,
+  // issued back to back so that the second request for a line meets the first in the L1 instead
+  // of fetching the line from L2 again a step later (half the L2 read requests; 1.25 -> 1.35
+  // PFLOP/s at 8192x4096x4096, at a higher clock: the kernel is power limited).  PAIR0 = steps
+  // issued before the loop.
+  constexpr int PAIR0 = (NSTAGE - 1) & ~1;
 #pragma unroll
-  for (int t = 0; t < NSTAGE - 2; t++)
+  for (int t = 0; t < PAIR0; t++)
     if (t < nk) issue_loads(t, t);
 
   // ---- LoRA term seeds the accumulator (overlaps with the first tile's loads)
@@ -319,6 +338,28 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
       }
     }
   };
+  // one fragment of k-slice ks (idx < TM: A fragment idx, else B fragment idx - TM)
+  auto read_one = [&](int buf, int stage, int ks, int idx) {
+    const int slot = ((2 * ks + q) ^ sw) << 4;
+    if (idx < TM) {
+      fa[buf][idx < TM ? idx : 0] = *(const lf_u32x4*)(ldsA + stage * A_STAGE + a_off[idx < TM ? idx : 0] + slot);
+    } else {
+      const int j = idx - TM < TN ? idx - TM : 0;
+      const char* sb = ldsB + stage * B_STAGE;
+      if constexpr (!NN) {
+        fb[buf][j] = *(const lf_u32x4*)(sb + b_off[j] + slot);
+      } else {
+        const char* base = sb + b_off[j] + ks * 16 * BPITCH;
+        fbt[buf][j][0] = lds_read_tr16(base);
+        fbt[buf][j][1] = lds_read_tr16(base + 4 * BPITCH);
+      }
+    }
+  };
+  auto mfma_one = [&](int buf, int idx) {
+    const int i = idx / TN, j = idx % TN;
+    if constexpr (NN) fb[buf][j] = lf_u32x4{fbt[buf][j][0][0], fbt[buf][j][0][1], fbt[buf][j][1][0], fbt[buf][j][1][1]};
+    acc[i][j] = MfmaOp<T>::run(fb[buf][j], fa[buf][i], acc[i][j]);
+  };
   auto mfmas = [&](int buf) {
     if constexpr (NN) {
 #pragma unroll
@@ -333,21 +374,40 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     // ---- main loop, one wave per SIMD: no neighbour to hide behind, so the fragments of step
     // kt+1 are read into a second register set while the MFMAs of step kt run; one barrier per
     // step.  At the top of step kt: tile kt is in registers, tile kt+1 has landed and is visible,
-    // every wave has finished reading the stage of tile kt-1.
-    using std::integral_constant;
+    // every wave has finished reading the stages of tiles kt-1 and kt.  Even steps issue the pair
+    // (kt+PAIR0, kt+PAIR0+1) into those two stages and, at their end, wait for the pair
+    // (kt+2, kt+3), issued two steps earlier.
     int stage = 0, kt = 0;
-    auto k_step = [&](auto SET, auto LOAD, auto NEXT, auto NEWER) {
+    auto k_step = [&](auto SET, auto LOAD, auto NEXT) {
       constexpr int cur = SET.value, nxt = 1 - SET.value;
       const int s1 = stage + 1 == NSTAGE ? 0 : stage + 1;
-      if (LOAD.value || kt + NSTAGE - 1 < nk) issue_loads(stage == 0 ? NSTAGE - 1 : stage - 1, kt + NSTAGE - 1);
-      if constexpr (NEXT.value) {
-        read_frags(nxt * 2 + 0, s1, 0);
-        read_frags(nxt * 2 + 1, s1, 1);
+      // Source order is the issue order (a scheduling fence after every MFMA): the LDS reads of the
+      // next step go out with the first half of the MFMAs, so that the second half covers the read
+      // latency, and the tile loads spread evenly over the step -- the texture addresser takes
+      // 16 cycles per load, and a wave that cannot issue a load cannot issue the MFMAs behind it.
+      constexpr int NFR = TM + TN, NM1 = TM * TN, NM = 2 * NM1, NR = 2 * NFR;
+      constexpr int NLD = LOAD.value ? 2 * NL : 0;  // lo/hi halves alternate: load l is half l&1 of load l>>1
+      constexpr int LSTEP = NLD > 0 && NM / NLD > 0 ? NM / NLD : 1;
+      constexpr int HALF = NM / 2 > 0 ? NM / 2 : 1, RPS = (NR + HALF - 1) / HALF;  // reads per MFMA slot
+      int st_lo = stage + PAIR0, st_hi = stage + PAIR0 + 1;  // stage of unit u is u % NSTAGE
+      st_lo = st_lo >= NSTAGE ? st_lo - NSTAGE : st_lo;
+      st_hi = st_hi >= NSTAGE ? st_hi - NSTAGE : st_hi;
+      st_hi = st_hi >= NSTAGE ? st_hi - NSTAGE : st_hi;
+      auto load_l = [&](int l) { issue_load_one((l & 1) ? st_hi : st_lo, kt + PAIR0 + (l & 1), l >> 1); };
+#pragma unroll
+      for (int m = 0; m < NM; m++) {
+        if (m % LSTEP == 0 && m / LSTEP < NLD) load_l(m / LSTEP);
+        if constexpr (NEXT.value) {
+#pragma unroll
+          for (int r = m * RPS; r < (m + 1) * RPS && r < NR; r++) read_one(nxt * 2 + r / NFR, s1, r / NFR, r % NFR);
+        }
+        mfma_one(cur * 2 + m / NM1, m % NM1);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);  // reads go out before the MFMAs that cover their latency
-      mfmas(cur * 2 + 0);
-      mfmas(cur * 2 + 1);
-      wait_loads(NEWER.value);             // tile kt+2 has landed
+#pragma unroll
+      for (int l = (NM + LSTEP - 1) / LSTEP; l < NLD; l++) load_l(l);  // more loads than MFMA slots
+      __builtin_amdgcn_sched_barrier(0);   // the waits stay behind the MFMAs that cover the read latency
+      if constexpr (cur == 0) wait_loads(integral_constant<int, LOAD.value ? PAIR0 - 2 : 0>{});  // the pair (kt+2, kt+3) has landed
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): next fragments are in registers
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_barrier();
@@ -357,23 +417,24 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     };
     using T_ = integral_constant<bool, true>;
     using F_ = integral_constant<bool, false>;
-    if (NSTAGE - 2 < nk) issue_loads(NSTAGE - 2, NSTAGE - 2);
-    wait_loads(nk > 2 ? NSTAGE - 3 : 0);  // tiles 0 and 1
+    if (nk > 2) wait_loads(integral_constant<int, PAIR0 - 2>{});  // tiles 0 and 1
+    else wait_loads(Steps0{});
     __syncthreads();
     read_frags(0, 0, 0);
     read_frags(1, 0, 1);
     __builtin_amdgcn_s_waitcnt(0xc07f);
-    while (kt + NSTAGE < nk) {  // two steps per trip: the register sets swap roles
-      k_step(integral_constant<int, 0>{}, T_{}, T_{}, integral_constant<int, NSTAGE - 3>{});
-      k_step(integral_constant<int, 1>{}, T_{}, T_{}, integral_constant<int, NSTAGE - 3>{});
+    __syncthreads();  // every wave has read stage 0: step 0 may refill it
+    while (kt + PAIR0 + 1 < nk) {  // two steps per trip: the register sets swap roles
+      k_step(integral_constant<int, 0>{}, T_{}, T_{});
+      k_step(integral_constant<int, 1>{}, F_{}, T_{});
     }
-    // tail (an even number of steps is left: nk is even): wait for everything
+    // tail (an even number of steps is left: nk is even): no more loads, wait for everything
     while (kt + 2 < nk) {
-      k_step(integral_constant<int, 0>{}, F_{}, T_{}, integral_constant<int, 0>{});
-      k_step(integral_constant<int, 1>{}, F_{}, T_{}, integral_constant<int, 0>{});
+      k_step(integral_constant<int, 0>{}, F_{}, T_{});
+      k_step(integral_constant<int, 1>{}, F_{}, T_{});
     }
-    k_step(integral_constant<int, 0>{}, F_{}, T_{}, integral_constant<int, 0>{});
-    k_step(integral_constant<int, 1>{}, F_{}, F_{}, integral_constant<int, 0>{});
+    k_step(integral_constant<int, 0>{}, F_{}, T_{});
+    k_step(integral_constant<int, 1>{}, F_{}, F_{});
   } else {
   // ---- main loop, two wave groups in anti-phase.  Each K step of a wave is a memory phase (issue
   // its share of a later tile's loads, read all fragments of the current tile into registers)
@@ -384,58 +445,73 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // not depend on instruction-level interleaving.
   //   phase 2k   : group 0 reads tile k        | group 1 computes tile k-1
   //   phase 2k+1 : group 0 computes tile k     | group 1 reads tile k
-  // Tile k is read in phases 2k and 2k+1.  Every wave waits for its own share of tile k at the end
-  // of its memory phase k-1 (phases 2k-2 / 2k-1), so the barrier closing phase 2k-1 publishes the
-  // whole tile.  The stage of tile k-1 is last read in phase 2k-1 and refilled (tile k+NSTAGE-1)
-  // from phase 2k on.  A load is in flight for 2*NSTAGE-4 phases.
+  // Tile k is read in phases 2k and 2k+1; every wave waits for its own share of it in a memory
+  // phase that ends no later than phase 2k-1, so the barrier closing that phase publishes the tile.
   const int grp = wave >= NWAVES / 2 ? 1 : 0;
   auto phase_barrier = [&]() {
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
-  // One K step of a wave.  The loads of step kt+NSTAGE-1 (into the stage of step kt-1, last read
-  // in phase 2kt-1) are issued from the compute phase, spread between the MFMAs: the texture
-  // addresser takes 16 cycles per 64-lane 16-byte load, and a burst of loads at the head of a
-  // memory phase (four waves of a CU at once) would hold those waves' LDS reads back behind it.
-  // LOAD: step kt+NSTAGE-1 exists.  NEWER: steps after kt+1 whose loads may still be in flight
-  // when the memory phase ends (step kt+1 itself must have landed).
-  using std::integral_constant;
+  // Two K steps of a wave.  Loads are issued from the compute phase of every odd step kt, spread
+  // between the MFMAs (the texture addresser takes 16 cycles per 64-lane 16-byte load: a burst of
+  // loads at the head of a memory phase would hold the LDS reads of four waves back behind it):
+  // the pair (kt+3, kt+4) goes into the stages of steps kt-2 and kt-1 (last read in phase 2kt-1).
+  // At the end of the memory phase of an odd step the pair (kt+1, kt+2), issued two steps earlier,
+  // must have landed.
   int stage = 0, kt = 0;
-  auto k_step = [&](auto LOAD, auto NEWER) {
+  static_assert(NSTAGE == 5, "the anti-phase loop is written for a ring of five stages");
+  auto step_pair = [&](auto LOAD) {
+    // even step
     read_frags(0, stage, 0);
     read_frags(1, stage, 1);
-    wait_loads(NEWER.value);
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): fragments are in registers
+    __builtin_amdgcn_s_waitcnt(0xc07f);
     phase_barrier();
     __builtin_amdgcn_s_setprio(1);
-    if constexpr (LOAD.value) issue_loads(stage == 0 ? NSTAGE - 1 : stage - 1, kt + NSTAGE - 1);
+    mfmas(0);
+    mfmas(1);
+    __builtin_amdgcn_s_setprio(0);
+    phase_barrier();
+    stage = stage + 1 == NSTAGE ? 0 : stage + 1;
+    kt++;
+    // odd step: the pair (kt+1, kt+2) must have landed; issue the pair (kt+3, kt+4)
+    read_frags(0, stage, 0);
+    read_frags(1, stage, 1);
+    wait_loads(Steps0{});
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    phase_barrier();
+    __builtin_amdgcn_s_setprio(1);
+    if constexpr (LOAD.value) {
+      const int s3 = stage + 3 >= NSTAGE ? stage + 3 - NSTAGE : stage + 3;
+      const int s4 = stage + 4 >= NSTAGE ? stage + 4 - NSTAGE : stage + 4;
+#pragma unroll
+      for (int i = 0; i < NL; i++) {
+        issue_load_one(s3, kt + 3, i);
+        issue_load_one(s4, kt + 4, i);
+      }
+    }
     mfmas(0);
     mfmas(1);
     if constexpr (LOAD.value) {
-      constexpr int NM = 2 * TM * TN, PER = NM / NL;
+      constexpr int NM = 2 * TM * TN, PER = NM / (2 * NL);
 #pragma unroll
-      for (int r = 0; r < NL; r++) {
+      for (int r = 0; r < 2 * NL; r++) {
         __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * NL, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * 2 * NL, 0);
     }
     __builtin_amdgcn_s_setprio(0);
     phase_barrier();
     stage = stage + 1 == NSTAGE ? 0 : stage + 1;
     kt++;
   };
-  // steps 0..NSTAGE-3 were issued before the accumulator was seeded; step NSTAGE-2 is issued by
-  // the compute phase of step -1, which does not exist: issue it here.
-  if (NSTAGE - 2 < nk) issue_loads(NSTAGE - 2, NSTAGE - 2);
-  wait_loads(nk >= NSTAGE - 1 ? NSTAGE - 2 : nk - 1);
+  if (nk > 2) wait_loads(integral_constant<int, 2>{});
+  else wait_loads(Steps0{});
   __syncthreads();
   if (grp == 1) phase_barrier();
-  // at the end of memory phase kt the loads of steps kt+1 .. kt+NSTAGE-2 are outstanding
-  while (kt + NSTAGE - 1 < nk) k_step(integral_constant<bool, true>{}, integral_constant<int, NSTAGE - 3>{});
-  // tail: no more loads to issue; wait for everything that is still in flight
-  while (kt < nk) k_step(integral_constant<bool, false>{}, integral_constant<int, 0>{});
+  while (kt + 5 < nk) step_pair(integral_constant<bool, true>{});
+  while (kt < nk) step_pair(integral_constant<bool, false>{});
   if (grp == 0) phase_barrier();
   }
 
