@@ -247,6 +247,29 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         use_mask = p.mask != nullptr && pb > 0.f;
       }
     }
+    // Keep-mask of this wave's sub-tile: 16-byte loads that cover whole rows of the sub-tile (issued
+    // here so that their latency overlaps the seeding MFMAs), handed to the lanes that own the
+    // accumulator elements through the wave's slice of the last ring stage, which no tile load
+    // targets before the main loop.  Granule g of row r sits at slot g ^ ((r / MRW) & (MLPR-1)):
+    // the 4-byte reads of 32 rows then spread over the banks (2-way instead of 16-way conflicts).
+    constexpr int MLPR = WN / 16, MRPI = 64 / MLPR, MNI = 32 / MRPI, MRW = 256 / WN;
+    static_assert(NWM == 2 && MNI >= 1, "mask staging: 32 rows x WN bytes per wave fit B_STAGE / NWAVES");
+    char* mreg = ldsB + (NSTAGE - 1) * B_STAGE + wave * (B_STAGE / NWAVES);
+    const int mrow = lane / MLPR, mg = lane % MLPR;
+    constexpr bool MEARLY = TM * MNI <= 8;  // all mask loads up front while they fit in 32 registers
+    lf_u32x4 mv[TM][MNI];
+    const int mcol = min(n0 + wn * WN + mg * 16, p.N - 16);
+    auto load_mask_band = [&](int i) {
+#pragma unroll
+      for (int ii = 0; ii < MNI; ii++) {
+        const int gm = min(wrow0 + i * 32 + ii * MRPI + mrow, p.M - 1);
+        mv[i][ii] = *(const lf_u32x4*)(p.mask + (int64_t)gm * p.ldmask + mcol);
+      }
+    };
+    if (use_mask && MEARLY) {
+#pragma unroll
+      for (int i = 0; i < TM; i++) load_mask_band(i);
+    }
     for (int t = 0; t < p.R / 16; t++) {
       const int r0 = t * 16 + q * 8;
       lf_u32x4 lf[TM], rf[TN];
@@ -279,22 +302,30 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(rf[j], lf[i], acc[i][j]);
     }
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < TM; i++) {
+      if (use_mask) {
+        if constexpr (!MEARLY) load_mask_band(i);
+#pragma unroll
+        for (int ii = 0; ii < MNI; ii++) {
+          const int r = ii * MRPI + mrow;
+          *(lf_u32x4*)(mreg + r * WN + ((mg ^ ((r / MRW) & (MLPR - 1))) << 4)) = mv[i][ii];
+        }
+      }
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         acc[i][j] *= mult;
         if (use_mask) {
-          int gm = min(wrow0 + i * 32 + l32, p.M - 1);
 #pragma unroll
           for (int jj = 0; jj < 4; jj++) {
-            int gn = min(n0 + wn * WN + j * 32 + jj * 8 + q * 4, p.N - 4);
-            uint32_t mk = *(const uint32_t*)(p.mask + (int64_t)gm * p.ldmask + gn);
+            const int dw = j * 8 + jj * 2 + q;  // dword of the 4 columns j*32 + jj*8 + q*4 ..
+            const uint32_t mk = *(const uint32_t*)(mreg + l32 * WN + (((dw >> 2) ^ ((l32 / MRW) & (MLPR - 1))) << 4) + (dw & 3) * 4);
 #pragma unroll
             for (int e = 0; e < 4; e++)
               acc[i][j][jj * 4 + e] = ((mk >> (8 * e)) & 0xffu) ? acc[i][j][jj * 4 + e] : 0.f;
           }
         }
       }
+    }
   }
 
   // ---- per-lane LDS fragment offsets
@@ -648,6 +679,8 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
   // 16-byte output stores
   if (p.ldc % 8 != 0 || ((uintptr_t)p.C & 15) != 0) return LF_ESHAPE;
   if (p.L != nullptr && (p.R % 16 != 0 || p.R <= 0 || p.R > LF_MAX_RANK)) return LF_ESHAPE;
+  // the keep-mask is read 16 bytes at a time
+  if (p.mask != nullptr && (p.N % 16 != 0 || p.ldmask % 16 != 0 || ((uintptr_t)p.mask & 15) != 0)) return LF_ESHAPE;
   // tile loads address the operands with 32-bit byte offsets
   if ((int64_t)p.M * p.lda * 2 >= 0x7fffffffLL || (int64_t)(nn ? p.K : p.N) * p.ldb * 2 >= 0x7fffffffLL) return LF_ESHAPE;
   if (seg.table != nullptr && (seg.block_size_m % 64 != 0)) return LF_ESHAPE;
