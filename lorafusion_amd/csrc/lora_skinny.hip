@@ -141,77 +141,122 @@ __device__ __forceinline__ lf_u32x4 tile_tr_frag(const char* tile, int row, int 
 }
 
 // ------------------------------------------------------------------------------------ xa
-// grid (n_blocks, ksplit); 4 waves, wave w owns rows 32w..32w+31 of the block.
-// part[ks][row][R] (fp32) = sum over this K slice of mask*X*A^T  (unscaled).
-// LDS: two X tiles + the A slice [RT*16][kslice] (row pitch kslice*2+16 bytes: 16 rows land on
-// 16 different bank groups).
+// One workgroup of 8 waves (fewer for ranks above 32) per 16 rows; no partial sums leave the workgroup.  The K range is dealt
+// to the waves in 64-column steps (step s goes to wave s % waves), each wave streams its steps of the
+// 16 rows with coalesced 16-byte loads (8 lanes cover one 128-byte line), all loads of a batch
+// of steps in flight at once, applies the keep-mask in registers and turns the row-major
+// granules into MFMA row fragments through a 2 KB LDS patch of its own (same-wave LDS traffic is
+// ordered: no barrier).  The adapter matrix A (L2 resident) takes the same route: fragment-shaped
+// loads would put the four lanes of every quad on four different rows, a quarter of the
+// coalesced rate in the texture addresser.  The eight partial [16, R] accumulators are added in a fixed order through LDS,
+// scaled by 1/(1-p), zeroed in padded rows and beyond the adapter's rank, and stored as S.
+constexpr int XA_ROWS = 16;
+// waves per workgroup and steps in flight per wave, by rank tiles (LDS: 2 KB * (1+RT) per wave; registers: 8 * RT per step)
+constexpr int xa_waves(int rt) { return rt <= 2 ? 8 : rt <= 4 ? 4 : 2; }
+constexpr int xa_unroll(int rt) { return rt <= 1 ? 4 : rt <= 2 ? 2 : 1; }
+
 template <typename T, int RT>
-__global__ void __launch_bounds__(256)
-lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, float* __restrict__ part,
-               int M, int K, int R, int kslice, const LfSegTable seg) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  char* xs = lds;
-  char* as = lds + 2 * TILE_BYTES;
-  const int blk = blockIdx.x, ks = blockIdx.y;
+__global__ void __launch_bounds__(xa_waves(RT) * 64)
+lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, T* __restrict__ S,
+               int M, int K, int R, const LfSegTable seg) {
+  constexpr int XA_WAVES = xa_waves(RT), XA_U = xa_unroll(RT);
+  __shared__ __attribute__((aligned(16))) char patch_all[XA_WAVES * 2048 * (1 + RT)];
+  __shared__ float red[XA_WAVES][XA_ROWS][RT * 16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, qq = lane >> 4;
+  const int row0 = blockIdx.x * XA_ROWS;
+  const int blk = row0 / ROWS;
   const BlockInfo bi = block_info(seg, blk, M);
   const T* __restrict__ A = (const T*)seg.ptr[bi.seg];
   const bool use_mask = mask != nullptr && bi.p > 0.f;
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
-  const int k_begin = ks * kslice;
-  const int ntiles = kslice / 64;
-  const int apitch = kslice * 2 + 16;
+  const int nsteps = K / 64;
+  char* patch = patch_all + wave * 2048 * (1 + RT);  // X patch, then one patch per 16 rank rows of A
 
-  TileRegs tr;
-  tile_load(tr, X, mask, K, blk * ROWS, Mrows, k_begin, tid, use_mask);
-  for (int g = tid; g < RT * 16 * (kslice / 8); g += 256) {
-    const int r = g / (kslice / 8), c = g % (kslice / 8);
-    lf_u32x4 v = {0, 0, 0, 0};
-    if (r < bi.rank) v = *(const lf_u32x4*)(A + (int64_t)r * K + k_begin + c * 8);
-    *(lf_u32x4*)(as + r * apitch + c * 16) = v;
+  // loader mapping: lane -> (row lane>>3 (+8), granule lane&7); fragment mapping: (row li, granule 4h+qq)
+  const int lrow = lane >> 3, lg = lane & 7;
+  const T* xrow[2];
+  const uint8_t* mrow[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = min(row0 + i * 8 + lrow, Mrows - 1);
+    xrow[i] = X + (int64_t)r * K + lg * 8;
+    mrow[i] = mask + (int64_t)r * K + lg * 8;
   }
-  tile_store(tr, xs, tid, use_mask);
-  if (ntiles > 1) tile_load(tr, X, mask, K, blk * ROWS, Mrows, k_begin + 64, tid, use_mask);
-  __syncthreads();
+  const int wr_off[2] = {lrow * 128 + ((lg ^ ((lrow >> 1) & 7)) << 4), (8 + lrow) * 128 + ((lg ^ (((8 + lrow) >> 1) & 7)) << 4)};
+  const int rd_row = li * 128, rd_key = (li >> 1) & 7;
 
-  lf_f32x4 acc[2][RT];
+  lf_f32x4 acc[RT];
 #pragma unroll
-  for (int a = 0; a < 2; a++)
-#pragma unroll
-    for (int c = 0; c < RT; c++) acc[a][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < RT; c++) acc[c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int t = 0; t < ntiles; t++) {
-    const char* cur = xs + (t & 1) * TILE_BYTES;
+  // (a second register set to overlap the next batch's loads costs occupancy and measured slower)
+  lf_u32x4 xv[1][XA_U][2], av[1][XA_U][RT][2];
+  lf_u32x2 mv[1][XA_U][2];
+  auto load_batch = [&](int b, int s0) {
 #pragma unroll
-    for (int step = 0; step < 2; step++) {
-      lf_u32x4 xf[2];
+    for (int u = 0; u < XA_U; u++) {
+      const int s = s0 + u * XA_WAVES;
+      if (s < nsteps) {
 #pragma unroll
-      for (int rt = 0; rt < 2; rt++) xf[rt] = tile_row_frag(cur, wave * 32 + rt * 16 + li, step * 4 + qq);
+        for (int i = 0; i < 2; i++) {
+          xv[b][u][i] = __builtin_nontemporal_load((const lf_u32x4*)(xrow[i] + s * 64));
+          if (use_mask) mv[b][u][i] = __builtin_nontemporal_load((const lf_u32x2*)(mrow[i] + s * 64));
 #pragma unroll
-      for (int c = 0; c < RT; c++) {
-        const lf_u32x4 af = *(const lf_u32x4*)(as + (c * 16 + li) * apitch + (t * 64 + step * 32 + qq * 8) * 2);
-#pragma unroll
-        for (int rt = 0; rt < 2; rt++) acc[rt][c] = Mfma16<T>::run(xf[rt], af, acc[rt][c]);
+          for (int c = 0; c < RT; c++) {
+            const int ar = c * 16 + i * 8 + lrow;
+            av[b][u][c][i] = lf_u32x4{0, 0, 0, 0};
+            if (ar < bi.rank) av[b][u][c][i] = *(const lf_u32x4*)(A + (int64_t)ar * K + s * 64 + lg * 8);
+          }
+        }
       }
     }
-    if (t + 1 < ntiles) {
-      tile_store(tr, xs + ((t + 1) & 1) * TILE_BYTES, tid, use_mask);
-      if (t + 2 < ntiles) tile_load(tr, X, mask, K, blk * ROWS, Mrows, k_begin + (t + 2) * 64, tid, use_mask);
+  };
+  auto use_batch = [&](int b, int s0) {
+#pragma unroll
+    for (int u = 0; u < XA_U; u++) {
+      const int s = s0 + u * XA_WAVES;
+      if (s < nsteps) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+          *(lf_u32x4*)(patch + wr_off[i]) = use_mask ? apply_mask8(xv[b][u][i], mv[b][u][i]) : xv[b][u][i];
+#pragma unroll
+          for (int c = 0; c < RT; c++) *(lf_u32x4*)(patch + (1 + c) * 2048 + wr_off[i]) = av[b][u][c][i];
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int fo = rd_row + (((h * 4 + qq) ^ rd_key) << 4);
+          const lf_u32x4 xf = *(const lf_u32x4*)(patch + fo);
+#pragma unroll
+          for (int c = 0; c < RT; c++) acc[c] = Mfma16<T>::run(xf, *(const lf_u32x4*)(patch + (1 + c) * 2048 + fo), acc[c]);
+        }
+      }
     }
-    __syncthreads();
+  };
+  for (int s0 = wave; s0 < nsteps; s0 += XA_WAVES * XA_U) {
+    load_batch(0, s0);
+    use_batch(0, s0);
   }
   // C layout: lane holds column (lane & 15), rows 4*(lane >> 4) + e
-  float* out = part + (int64_t)ks * Mrows * R;
 #pragma unroll
-  for (int rt = 0; rt < 2; rt++)
+  for (int c = 0; c < RT; c++)
 #pragma unroll
-    for (int c = 0; c < RT; c++)
+    for (int e = 0; e < 4; e++) red[wave][qq * 4 + e][c * 16 + li] = acc[c][e];
+  __syncthreads();
+  const float mult = bi.p > 0.f ? 1.f / (1.f - bi.p) : 1.f;
+  for (int o = tid; o < XA_ROWS * RT * 16; o += XA_WAVES * 64) {
+    const int r = o / (RT * 16), c = o % (RT * 16);
+    const int row = row0 + r;
+    if (row < Mrows && c < R) {
+      float v = 0.f;
+      if (row - blk * ROWS < bi.valid && c < bi.rank) {
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const int row = blk * ROWS + wave * 32 + rt * 16 + qq * 4 + e;
-        if (row < Mrows) out[(int64_t)row * R + c * 16 + li] = acc[rt][c][e];
+        for (int w = 0; w < XA_WAVES; w++) v += red[w][r][c];
+        v *= mult;
       }
+      ((uint16_t*)S)[(int64_t)row * R + c] = Mfma16<T>::cvt(v);
+    }
+  }
 }
 
 // S[row][col] = cast( mult * sum_p part[p][row][col] ), zero for padded rows / rank columns.
@@ -513,44 +558,27 @@ static int pick_split(int nblk, int len, int min_split) {
   return split;
 }
 
-static int xa_split(int nblk, int K, int R) { return pick_split(nblk, K, (K * rt_of(R) + 2047) / 2048); }
 
-size_t lf_xa_workspace(int M, int K, int R, const LfSegTable& seg) {
-  const int nblk = n_row_blocks(M, seg);
-  const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  return (size_t)xa_split(nblk, K, R) * rows * R * sizeof(float);
-}
+size_t lf_xa_workspace(int, int, int, const LfSegTable&) { return 0; }
 
 template <typename T, int RT>
-static int xa_launch(const void* X, const uint8_t* mask, float* part, int M, int K, int R, int kslice, dim3 grid,
+static int xa_launch(const void* X, const uint8_t* mask, void* S, int M, int K, int R, int64_t rows,
                      const LfSegTable& seg, hipStream_t st) {
-  auto kern = lora_xa_kernel<T, RT>;
-  const int smem = 2 * TILE_BYTES + RT * 16 * (kslice * 2 + 16);
-  if (smem > 160 * 1024) return LF_ESHAPE;
-  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return LF_ELAUNCH;
-  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)X, mask, part, M, K, R, kslice, seg);
+  const unsigned grid = (unsigned)((rows + XA_ROWS - 1) / XA_ROWS);
+  hipLaunchKernelGGL((lora_xa_kernel<T, RT>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, (T*)S, M, K, R, seg);
   return lf_check_launch();
 }
 
 template <typename T>
-static int xa_impl(const void* X, const uint8_t* mask, void* S, void* ws, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
+static int xa_impl(const void* X, const uint8_t* mask, void* S, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  const int split = xa_split(nblk, K, R);
-  const int kslice = K / split;
-  float* part = (float*)ws;
-  dim3 grid(nblk, split);
-  int rc;
   switch (rt_of(R)) {
-    case 1: rc = xa_launch<T, 1>(X, mask, part, M, K, R, kslice, grid, seg, st); break;
-    case 2: rc = xa_launch<T, 2>(X, mask, part, M, K, R, kslice, grid, seg, st); break;
-    case 4: rc = xa_launch<T, 4>(X, mask, part, M, K, R, kslice, grid, seg, st); break;
-    default: rc = xa_launch<T, 8>(X, mask, part, M, K, R, kslice, grid, seg, st); break;
+    case 1: return xa_launch<T, 1>(X, mask, S, M, K, R, rows, seg, st);
+    case 2: return xa_launch<T, 2>(X, mask, S, M, K, R, rows, seg, st);
+    case 4: return xa_launch<T, 4>(X, mask, S, M, K, R, rows, seg, st);
+    default: return xa_launch<T, 8>(X, mask, S, M, K, R, rows, seg, st);
   }
-  if (rc != LF_OK) return rc;
-  const int64_t n = rows * R;
-  hipLaunchKernelGGL((reduce_rows_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float*)part, (T*)S, split, M, R, 0, seg);
-  return lf_check_launch();
 }
 
 int lf_launch_xa(const void* X, const uint8_t* mask, void* S, void* ws, size_t ws_bytes, int M, int K, int R,
@@ -558,9 +586,9 @@ int lf_launch_xa(const void* X, const uint8_t* mask, void* S, void* ws, size_t w
   if (!X || !S || M <= 0 || K <= 0) return LF_EINVAL;
   if (K % 128 != 0 || R % 16 != 0 || R <= 0 || R > LF_MAX_RANK) return LF_ESHAPE;
   if (seg.table && seg.block_size_m != ROWS) return LF_ESHAPE;
-  if (!ws || ws_bytes < lf_xa_workspace(M, K, R, seg)) return LF_EWORKSPACE;
-  if (dtype == LF_BF16) return xa_impl<__bf16>(X, mask, S, ws, M, K, R, seg, st);
-  if (dtype == LF_F16) return xa_impl<_Float16>(X, mask, S, ws, M, K, R, seg, st);
+  (void)ws; (void)ws_bytes;  // no partial sums leave the workgroups
+  if (dtype == LF_BF16) return xa_impl<__bf16>(X, mask, S, M, K, R, seg, st);
+  if (dtype == LF_F16) return xa_impl<_Float16>(X, mask, S, M, K, R, seg, st);
   return LF_EINVAL;
 }
 
