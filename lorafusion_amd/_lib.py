@@ -17,10 +17,11 @@ LIB_PATH = os.path.join(_HERE, "liblorafusion_hip.so")
 LF_BF16, LF_F16 = 0, 1
 LF_MAX_SEG = 32
 LF_OP_XA, LF_OP_DYS_DYB, LF_OP_DA, LF_OP_FWD, LF_OP_BWD = range(5)
+LF_OK, LF_EINVAL, LF_ESHAPE, LF_EWORKSPACE, LF_ELAUNCH, LF_ELIMIT = 0, -1, -2, -3, -4, -5
 
 EXPORTS = (
     "lf_version", "lf_strerror", "lf_workspace_bytes", "lf_lora_xa", "lf_lora_xw_sb", "lf_lora_dys_dyb",
-    "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant",
+    "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant", "lf_dropout_mask",
 )
 
 
@@ -72,6 +73,7 @@ def lib() -> ctypes.CDLL:
     l.lf_lora_bwd.argtypes = [vp] * 12 + [sz, i, i, i, i, rp, i, vp]
     l.lf_gemm.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, vp]
     l.lf_nf4_dequant.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, i, i, i, vp]
+    l.lf_dropout_mask.argtypes = [vp, i, i, ctypes.c_float, rp, ctypes.c_uint64, vp]
     for name in EXPORTS:
         if name not in ("lf_strerror", "lf_workspace_bytes"):
             getattr(l, name).restype = i

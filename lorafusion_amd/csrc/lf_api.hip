@@ -6,6 +6,7 @@ int lf_launch_nf4_dequant(const uint8_t*, const void*, const float*, const float
 int lf_launch_xa(const void*, const uint8_t*, void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
 int lf_launch_dys_dyb(const void*, const void*, void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
 int lf_launch_da(const void*, const uint8_t*, const void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
+int lf_launch_dropout_mask(uint8_t*, int, int, float, const float*, int, uint64_t, hipStream_t);
 size_t lf_xa_workspace(int, int, int, const LfSegTable&);
 size_t lf_dys_dyb_workspace(int, int, int, const LfSegTable&);
 size_t lf_da_workspace(int, int, int, const LfSegTable&);
@@ -185,6 +186,18 @@ int lf_nf4_dequant(const uint8_t* packed, const void* absmax, const float* code2
                    void* stream) {
   return lf_launch_nf4_dequant(packed, absmax, code2, absmax2, offset, out, n_elems, blocksize, blocksize2,
                                out_dtype, (hipStream_t)stream);
+}
+
+int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream) {
+  const float* block_p = nullptr;
+  int bs = 0;
+  if (routing != nullptr && routing->block_table != nullptr) {
+    if (!routing->block_p || routing->block_size_m <= 0) return LF_EINVAL;
+    if ((int64_t)routing->n_blocks * routing->block_size_m != M) return LF_ESHAPE;
+    block_p = routing->block_p;
+    bs = routing->block_size_m;
+  }
+  return lf_launch_dropout_mask(mask, M, K, p, block_p, bs, seed, (hipStream_t)stream);
 }
 
 }  // extern "C"

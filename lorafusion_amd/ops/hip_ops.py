@@ -8,6 +8,9 @@ done by liblorafusion_hip.so through ctypes.  Single-adapter functions take plai
 
 from __future__ import annotations
 
+import ctypes
+import random
+
 import torch
 
 from lorafusion_amd import _lib as L
@@ -124,24 +127,44 @@ def _xa(x, mask, a_list, routing, M, K, R):
     return s
 
 
-def make_dropout_mask(shape, p, seed: int | None, device) -> torch.Tensor:
-    """Bernoulli(1-p) keep-mask, bool.  ``p`` is a float or a per-row tensor."""
-    gen = None
-    if seed is not None:
-        gen = torch.Generator(device=device)
-        gen.manual_seed(int(seed))
-    u = torch.rand(shape, device=device, generator=gen)
-    if isinstance(p, torch.Tensor):
-        return u >= p.to(device=device, dtype=torch.float32).reshape(-1, 1)
-    return u >= p
+def make_dropout_mask(shape, p, seed: int | None, device, routing: "MultiRouting | None" = None) -> torch.Tensor:
+    """Bernoulli(1-p) keep-mask, bool ``[M, K]``, drawn on the device by the HIP Philox kernel.
+
+    The mask half of ``seeded_dropout`` (lorafusion/ops/triton_ops/dropout.py:71-93); with
+    ``routing`` the per-block p of the packed batch is used (blocked_seeded_dropout,
+    lorafusion/ops/triton_ops/blocked_dropout.py:78-135) and ``p`` is ignored.  ``seed=None``
+    draws a seed on the host, as the reference does (dropout.py:75-76).
+    """
+    M, K = int(shape[0]), int(shape[1])
+    if K % 16 != 0:
+        raise ValueError(f"the mask kernel needs K % 16 == 0, got K={K}.")
+    if seed is None:
+        seed = random.randrange(int(1e6))  # noqa: S311
+    dev = torch.device(device)
+    if dev.type != "cuda":
+        raise ValueError("make_dropout_mask draws the mask on the GPU; got device " + str(device))
+    if dev.index is None:
+        dev = torch.device("cuda", torch.cuda.current_device())
+    mask = torch.empty((M, K), dtype=torch.bool, device=dev)
+    rc = None
+    if routing is not None:
+        if routing.M != M:
+            raise ValueError(f"routing covers {routing.M} rows, mask has {M}.")
+        rc, pv = ctypes.byref(routing.c), 0.0
+    else:
+        _check_p(float(p))
+        pv = float(p)
+    with torch.cuda.device(dev):
+        L.check(L.lib().lf_dropout_mask(L.ptr(mask), M, K, ctypes.c_float(pv), rc, ctypes.c_uint64(int(seed) & 0xFFFFFFFFFFFFFFFF),
+                                        L.stream_of(mask)), "lf_dropout_mask")
+    return mask
 
 
 def seeded_dropout(x: torch.Tensor, p: float, seed: int, *, store_mask: bool = True):
     """``(where(mask, x/(1-p), 0), mask)`` -- lorafusion/ops/triton_ops/dropout.py:71-93.
 
-    Kept for API parity; the fused path never materialises the dropped tensor.  The mask
-    comes from torch's generator seeded with ``seed`` (the reference's Philox stream is not
-    reproduced).
+    Kept for API parity; the fused path never materialises the dropped tensor.  The mask comes
+    from the HIP Philox4x32-10 kernel keyed by ``seed`` (a stream of its own, not Triton's).
     """
     _check_p(p)
     mask = make_dropout_mask(x.shape, p, seed, x.device)

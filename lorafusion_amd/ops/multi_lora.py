@@ -171,8 +171,7 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
             else:
                 if seed is None:
                     seed = random.randrange(int(1e6))  # noqa: S311
-                row_p = routing.p.repeat_interleave(routing.block_size_m)
-                mask = hip_ops.make_dropout_mask((M, K), row_p, seed, x2d.device)
+                mask = hip_ops.make_dropout_mask((M, K), None, seed, x2d.device, routing=routing)
         bias = linear_bias.contiguous() if linear_bias is not None else None
         y, s = hip_ops.lora_forward(x2d, linear_w, a_list, b_list, routing.c, routing.R, mask, bias)
 
