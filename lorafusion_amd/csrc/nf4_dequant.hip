@@ -44,33 +44,46 @@ nf4_dequant_kernel(const uint32_t* __restrict__ packed, const void* __restrict__
                    int shift /* log2(blocksize) - 3: packed dword -> block */, int shift2 /* log2(blocksize2) */) {
   __shared__ float lut[16];
   __shared__ float lut2[256];
+  __shared__ float am_lds[NF4_THREADS * NF4_STEPS];  // block scales of this workgroup's span (at most one per packed dword)
   const int tid = threadIdx.x;
   if (tid < 16) lut[tid] = kNf4Code[tid];
   if (NESTED) lut2[tid] = code2[tid];
-  __syncthreads();
-  float offset = 0.f;
-  if (NESTED) offset = offset_p[0];
-
-  const int64_t base = (int64_t)blockIdx.x * (NF4_THREADS * NF4_STEPS) + tid;
+  const int64_t wg_base = (int64_t)blockIdx.x * (NF4_THREADS * NF4_STEPS);
+  const int64_t base = wg_base + tid;
+  // packed data first: these are the loads the stores wait for
   uint32_t w[NF4_STEPS];
-  float am[NF4_STEPS];
 #pragma unroll
   for (int s = 0; s < NF4_STEPS; s++) {
     const int64_t i = base + (int64_t)s * NF4_THREADS;
-    w[s] = 0;
-    am[s] = 0.f;
-    if (i < n_words) {
-      w[s] = __builtin_nontemporal_load(packed + i);
-      const int64_t blk = i >> shift;
+    w[s] = i < n_words ? __builtin_nontemporal_load(packed + i) : 0u;
+  }
+  if (NESTED) __syncthreads();  // lut2 is complete
+  // One scale per quantisation block of the span, computed once (a lane-per-dword lookup would
+  // issue a byte load and a float load per lane and step: twice the vector-memory instructions
+  // of the data itself, and the texture addresser takes 16 cycles for each).
+  const int64_t blk0 = wg_base >> shift;
+  const int nblk = ((NF4_THREADS * NF4_STEPS) >> shift) > 0 ? (NF4_THREADS * NF4_STEPS) >> shift : 1;
+  const int64_t nblk_total = (n_words + ((int64_t)1 << shift) - 1) >> shift;
+  float offset = 0.f;
+  if (NESTED) offset = offset_p[0];
+  for (int j = tid; j < nblk; j += NF4_THREADS) {
+    const int64_t blk = blk0 + j;
+    float a = 0.f;
+    if (blk < nblk_total) {
       if (NESTED) {
         const uint8_t aq = ((const uint8_t*)absmax_in)[blk];
         // single-rounding fused multiply-add, as tl.fma in the reference
-        am[s] = __builtin_fmaf(lut2[aq], absmax2[blk >> shift2], offset);
+        a = __builtin_fmaf(lut2[aq], absmax2[blk >> shift2], offset);
       } else {
-        am[s] = ((const float*)absmax_in)[blk];
+        a = ((const float*)absmax_in)[blk];
       }
     }
+    am_lds[j] = a;
   }
+  __syncthreads();
+  float am[NF4_STEPS];
+#pragma unroll
+  for (int s = 0; s < NF4_STEPS; s++) am[s] = am_lds[(s * NF4_THREADS + tid) >> shift];
 #pragma unroll
   for (int s = 0; s < NF4_STEPS; s++) {
     const int64_t i = base + (int64_t)s * NF4_THREADS;
