@@ -33,8 +33,11 @@ template <> __device__ __forceinline__ uint32_t pack2<_Float16>(float lo, float 
   return __builtin_bit_cast(uint32_t, v);
 }
 
+#ifndef LF_NF4_STEPS
+#define LF_NF4_STEPS 16
+#endif
 constexpr int NF4_THREADS = 256;
-constexpr int NF4_STEPS = 8;
+constexpr int NF4_STEPS = LF_NF4_STEPS;
 
 template <typename T, bool NESTED>
 __global__ void __launch_bounds__(NF4_THREADS)
