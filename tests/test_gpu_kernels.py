@@ -15,7 +15,7 @@ def _close(actual, expected, what, rtol=1e-2):
     assert ok, f"{what}: max|err|/max|e| = {rel:.3e}, worst excess {excess:.3e}"
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("trans_b", [True, False])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (520, 640, 384), (1024, 1280, 1024), (77, 136, 64), (130, 72, 704)])
 def test_gemm_all_tiles(cfg, trans_b, M, N, K):
@@ -54,7 +54,7 @@ def test_gemm_identity_exact():
     a = torch.randn(300, 256, generator=g).bfloat16().cuda()
     eye = torch.eye(256).bfloat16().cuda()
     for trans_b in (True, False):
-        for cfg in range(6):
+        for cfg in range(7):
             assert torch.equal(hip_ops.gemm(a, eye, trans_b=trans_b, tile_cfg=cfg), a)
     # a permutation matrix tells B from B^T
     perm = torch.randperm(256, generator=g)
