@@ -261,11 +261,10 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, T* __r
 
 // S[row][col] = cast( mult * sum_p part[p][row][col] ), zero for padded rows / rank columns.
 template <typename T>
-__global__ void __launch_bounds__(256)
-reduce_rows_kernel(const float* __restrict__ part, T* __restrict__ out, int nparts, int M, int R,
+__device__ __forceinline__ void reduce_rows_body(int bx, const float* __restrict__ part, T* __restrict__ out, int nparts, int M, int R,
                    int mode /*0: times 1/(1-p); 1: times scale*/, const LfSegTable seg) {
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t idx = (int64_t)bx * 256 + threadIdx.x;
   if (idx >= (int64_t)Mrows * R) return;
   const int row = (int)(idx / R), col = (int)(idx % R);
   const int blk = row / ROWS;
@@ -276,6 +275,12 @@ reduce_rows_kernel(const float* __restrict__ part, T* __restrict__ out, int npar
     v *= (mode == 0) ? (bi.p > 0.f ? 1.f / (1.f - bi.p) : 1.f) : bi.scale;
   }
   ((uint16_t*)out)[idx] = Mfma16<T>::cvt(v);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+reduce_rows_kernel(const float* __restrict__ part, T* __restrict__ out, int nparts, int M, int R, int mode, const LfSegTable seg) {
+  reduce_rows_body<T>((int)blockIdx.x, part, out, nparts, M, R, mode, seg);
 }
 
 // ------------------------------------------------------------------------------- dys_dyb
@@ -420,12 +425,10 @@ __device__ __forceinline__ void segment_blocks(const LfSegTable& seg, int s, int
 //   transposed == 1 (dA): parts are the segment's chunks, part[(s*max_chunks + ch)][R][rows] -> out [rank, rows]
 //   mult_mode 0: segment scale ; 1: 1/(1-p) of the segment.
 template <typename T>
-__global__ void __launch_bounds__(256)
-reduce_segments_kernel(const float* __restrict__ part, int rows, int R, int transposed, int mult_mode, int M,
+__device__ __forceinline__ void reduce_segments_body(int bx, int s, const float* __restrict__ part, int rows, int R, int transposed, int mult_mode, int M,
                        int group, int max_chunks, const LfSegTable seg) {
-  const int s = blockIdx.y;
   const int rank = seg.rank[s];
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index into the output [rows, rank] or [rank, rows]
+  const int64_t idx = (int64_t)bx * 256 + threadIdx.x;  // index into the output [rows, rank] or [rank, rows]
   if (idx >= (int64_t)rows * rank) return;
   int b0, b1;
   segment_blocks(seg, s, M, b0, b1);
@@ -448,6 +451,28 @@ reduce_segments_kernel(const float* __restrict__ part, int rows, int R, int tran
     for (int ch = 0; ch < nch; ch++) v += part[((int64_t)s * max_chunks + ch) * R * rows + pidx];
   }
   ((uint16_t*)seg.out[s])[idx] = Mfma16<T>::cvt(v * mult);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+reduce_segments_kernel(const float* __restrict__ part, int rows, int R, int transposed, int mult_mode, int M,
+                       int group, int max_chunks, const LfSegTable seg) {
+  reduce_segments_body<T>((int)blockIdx.x, (int)blockIdx.y, part, rows, R, transposed, mult_mode, M, group, max_chunks, seg);
+}
+
+// Second stage of dys_dyb in one launch: blocks [0, nb_rows) reduce the dS partials, the rest the
+// dB partials (nb_seg blocks per segment).
+template <typename T>
+__global__ void __launch_bounds__(256)
+reduce_ds_db_kernel(const float* __restrict__ ds_part, T* __restrict__ dS, int nparts, int M, int R, int nb_rows,
+                    const float* __restrict__ db_part, int N, int nb_seg, const LfSegTable seg) {
+  const int b = blockIdx.x;
+  if (b < nb_rows) {
+    reduce_rows_body<T>(b, ds_part, dS, nparts, M, R, 1, seg);
+  } else {
+    const int c = b - nb_rows;
+    reduce_segments_body<T>(c % nb_seg, c / nb_seg, db_part, N, R, 0, 0, M, 1, 1, seg);
+  }
 }
 
 // ------------------------------------------------------------------------------------ da
@@ -627,13 +652,13 @@ static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M
   }
   if (rc != LF_OK) return rc;
   const int64_t n = rows * R;
-  hipLaunchKernelGGL((reduce_rows_kernel<T>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const float*)ds_part, (T*)dS, split, M, R, 1, seg);
-  if (lf_check_launch() != LF_OK) return LF_ELAUNCH;
   const int nseg = seg.table ? seg.n_seg : 1;
   int maxrank = 0;
   for (int s = 0; s < nseg; s++) maxrank = seg.rank[s] > maxrank ? seg.rank[s] : maxrank;
   const int64_t nout = (int64_t)N * maxrank;
-  hipLaunchKernelGGL((reduce_segments_kernel<T>), dim3((unsigned)((nout + 255) / 256), nseg), dim3(256), 0, st, (const float*)db_part, N, R, 0, 0, M, 1, 1, seg);
+  const int nb_rows = (int)((n + 255) / 256), nb_seg = (int)((nout + 255) / 256);
+  hipLaunchKernelGGL((reduce_ds_db_kernel<T>), dim3((unsigned)(nb_rows + nb_seg * nseg)), dim3(256), 0, st, (const float*)ds_part,
+                     (T*)dS, split, M, R, nb_rows, (const float*)db_part, N, nb_seg, seg);
   return lf_check_launch();
 }
 
