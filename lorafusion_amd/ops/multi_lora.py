@@ -20,7 +20,7 @@ from __future__ import annotations
 import random
 from collections import deque
 from dataclasses import dataclass
-from typing import Any
+from typing import Any, Sequence
 
 import numpy as np
 import torch
@@ -131,6 +131,57 @@ def prepare_multi_lora_batch_info(
         micro_batch_info=micro_batch_info,
         allow_empty_micro_batch_info=allow_empty_micro_batch_info,
     )
+
+
+def batch_info_from_micro_batch(
+    micro_batch_info: Any,
+    lora_configs: "Sequence[Any] | dict[int, Any]",
+    block_size_m: int = FUSED_MULTI_LORA_BLOCK_SIZE_M,
+    output_dtype: torch.dtype = torch.float32,
+    device: str | torch.device | None = None,
+) -> MultiLoRABatchInfo:
+    """Routing tables straight from a scheduler micro-batch descriptor.
+
+    Restates the conversion the reference's data provider does before every micro-batch
+    (lorafusion/train/training_utils.py:1250-1334): adapters in ascending index order, one segment per
+    adapter with ``adapter_num_tokens_pairs[idx]`` tokens, rank / dropout / multiplier from
+    ``lora_configs[idx]`` (``.r``, ``.lora_dropout``, ``.lora_alpha`` -- the reference hands the raw
+    ``lora_alpha`` to the kernels as the multiplier there, training_utils.py:1323).  ``micro_batch_info``
+    is duck-typed on the fields of ``MicroBatchInfo`` (lorafusion/solver/proposed_solver.py:51-131):
+    ``adapter_group_info``, ``adapter_num_tokens_pairs``, ``padded_adapter_num_tokens_pairs``,
+    ``adapter_padding_multiple``; the descriptor's own padding must be the kernels' block size.
+    """
+    if getattr(micro_batch_info, "is_empty_marker", False):
+        raise ValueError("an empty-marker micro-batch carries no tokens; there is nothing to route.")
+    pad = getattr(micro_batch_info, "adapter_padding_multiple", block_size_m)
+    if pad != block_size_m:
+        raise ValueError(
+            f"micro-batch padding multiple {pad} differs from the kernels' block size {block_size_m}."
+        )
+    adapters = sorted(micro_batch_info.adapter_group_info)
+    if not adapters:
+        raise ValueError("the micro-batch names no adapter.")
+    seq_len_list = [int(micro_batch_info.adapter_num_tokens_pairs[a]) for a in adapters]
+    cfgs = [lora_configs[a] for a in adapters]
+    info = prepare_multi_lora_batch_info(
+        seq_len_list=seq_len_list,
+        lora_idx_list=list(adapters),
+        lora_rank_list=[int(c.r) for c in cfgs],
+        dropout_p_list=[float(c.lora_dropout) for c in cfgs],
+        alpha_list=[float(c.lora_alpha) for c in cfgs],
+        block_size_m=block_size_m,
+        output_dtype=output_dtype,
+        micro_batch_info=micro_batch_info,
+        device=device,
+    )
+    padded_pairs = getattr(micro_batch_info, "padded_adapter_num_tokens_pairs", None)
+    if padded_pairs is not None:
+        expect = [int(padded_pairs[a]) for a in adapters]
+        if expect != info.padded_seq_len_list:
+            raise ValueError(
+                f"padded token counts of the micro-batch {expect} differ from the routing tables {info.padded_seq_len_list}."
+            )
+    return info
 
 
 class FusedLinearMultiLoRA(torch.autograd.Function):

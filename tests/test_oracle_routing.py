@@ -85,3 +85,34 @@ def test_product_table_builder_errors_and_bf16_option():
     assert info.block_to_dropout_p.dtype == torch.bfloat16
     assert float(info.block_to_dropout_p[0]) == 0.10009765625
     assert info.lora_idx_list == [3, 1]
+
+
+def test_batch_info_from_micro_batch_descriptor():
+    """The scheduler's micro-batch descriptor (duck-typed) drives the routing tables:
+    lorafusion/train/training_utils.py:1304-1334 restated."""
+    from types import SimpleNamespace
+
+    import torch
+
+    from lorafusion_amd.ops.multi_lora import batch_info_from_micro_batch
+
+    tokens = {3: 129, 0: 130, 7: 128}
+    mb = SimpleNamespace(
+        adapter_group_info=set(tokens), adapter_num_tokens_pairs=tokens,
+        padded_adapter_num_tokens_pairs={a: ((n - 1) // 128 + 1) * 128 for a, n in tokens.items()},
+        adapter_padding_multiple=128, is_empty_marker=False)
+    cfgs = {a: SimpleNamespace(r=16 * (1 + a % 2), lora_dropout=0.05 * (a % 3), lora_alpha=16.0 + a) for a in tokens}
+    info = batch_info_from_micro_batch(mb, cfgs, device="cpu")
+    assert info.lora_idx_list == [0, 3, 7] and info.seq_len_list == [130, 129, 128]
+    padded, lookup, block_p, block_alpha, *_ = routing.block_tables([130, 129, 128], [16, 32, 32], [0.0, 0.0, 0.05],
+                                                                    [16.0, 19.0, 23.0], 128)
+    assert info.padded_seq_len_list == padded == [256, 256, 128]
+    assert np.array_equal(info.block_to_lookup_table.numpy(), lookup)
+    assert np.allclose(info.block_to_dropout_p.numpy(), block_p) and np.allclose(info.block_to_alpha.numpy(), block_alpha)
+    assert info.micro_batch_info is mb and info.max_r == 32
+    # a descriptor padded to another multiple cannot drive 128-row kernels
+    mb.adapter_padding_multiple = 64
+    with pytest.raises(ValueError):
+        batch_info_from_micro_batch(mb, cfgs, device="cpu")
+    with pytest.raises(ValueError):
+        batch_info_from_micro_batch(SimpleNamespace(is_empty_marker=True), cfgs, device="cpu")
