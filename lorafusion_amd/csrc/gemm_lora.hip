@@ -637,8 +637,8 @@ static const TileCand kCands[] = {
     {1, 256, 256, 256, 66.0, 50.0, 44.0, 60.0},   // 8 waves, 128x64 per wave
     {3, 128, 256, 256, 48.0, 28.0, 28.0, 38.0},   // 8 waves, 64x64 per wave
     {4, 128, 128, 512, 38.0, 47.0, 5.0, 70.0},    // 4 waves, two workgroups per CU
-    {5, 64, 64, 512, 21.0, 15.0, 13.0, 18.0},     // 4 waves, 32x32 per wave: spreads a short row range
-    {6, 128, 64, 256, 21.0, 6.0, 13.0, 14.0},     // 4 waves, 64x32 per wave: less operand traffic per flop than 64x64
+    {5, 64, 64, 512, 19.0, 17.0, 13.0, 18.0},     // 4 waves, 32x32 per wave: spreads a short row range
+    {6, 128, 64, 256, 22.5, 4.5, 13.0, 14.0},     // 4 waves, 64x32 per wave: less operand traffic per flop than 64x64
 };
 static double launch_cost(const TileCand& c, int M, int N) {
   const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
