@@ -219,6 +219,7 @@ def main():
     t_dys = event_time_ms(lambda: hip_ops.fused_multi_lora_dys_dyb(dyd, s, bd, routing), reps)
     t_da = event_time_ms(lambda: hip_ops.fused_multi_lora_da(xd, ds, routing, mask), reps)
     t_mask = event_time_ms(lambda: hip_ops.make_dropout_mask(xd.shape, None, 1234, dev, routing=routing), reps)
+    t_fwd_seeded = event_time_ms(lambda: hip_ops.lora_forward_seeded(xd, wd, ad, bd, routing.c, routing.R, 1234, None), reps)
     # ---- dominant kernel: the 256x256-tile MFMA GEMM of the dX path.  The library runs rows
     # [0, 8192) of the 8448 in whole rounds of that tile and the last 256 rows as a second, small
     # launch; the roofline entry times the big launch alone (same grid, same data: the first 64
@@ -282,7 +283,7 @@ def main():
         },
         "kernels_ms": {
             "xa": round(t_xa, 4), "gemm_fwd": round(t_fwd, 4), "dys_dyb": round(t_dys, 4), "da": round(t_da, 4),
-            "gemm_bwd": round(t_bwd, 4), "seeded_mask": round(t_mask, 4), "plain_gemm_nt": round(t_plain_nt, 4), "plain_gemm_nn": round(t_plain_nn, 4),
+            "gemm_bwd": round(t_bwd, 4), "seeded_mask": round(t_mask, 4), "fwd_seeded_xa_plus_gemm": round(t_fwd_seeded, 4), "plain_gemm_nt": round(t_plain_nt, 4), "plain_gemm_nn": round(t_plain_nn, 4),
         },
         "lora_overhead_vs_plain_gemms": round((t_xa + t_fwd + t_dys + t_da + t_bwd) / (t_plain_nt + t_plain_nn) - 1.0, 4),
         "nf4_dequant": {

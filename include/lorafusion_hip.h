@@ -79,6 +79,14 @@ size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* 
 int lf_lora_xa(const void* X, const uint8_t* mask, const void* const* a_ptrs, void* S, void* workspace,
                size_t ws_bytes, int M, int K, int R, const lf_routing* routing, int dtype, void* stream);
 
+/* lf_lora_xa with the keep-mask drawn inside the kernel instead of read: the reference's default
+ * forward, where seeded_dropout makes the mask and the dropped input in one pass
+ * (lorafusion/ops/lora_v1.py:111-116; fused_dropout_matmul with store_mask,
+ * fused_dropout_matmul.py:300-352).  mask_out [M,K] receives exactly the bytes lf_dropout_mask
+ * writes for the same (seed, routing): rows of a block with p = 0 are all ones. */
+int lf_lora_xa_seeded(const void* X, uint8_t* mask_out, const void* const* a_ptrs, void* S, int M, int K, int R,
+                      const lf_routing* routing, uint64_t seed, int dtype, void* stream);
+
 /* Y = X W^T + scale * S B^T + bias.  Stands in for fused_lora_xw_sb / fused_lora_xw_sb_tma
  * (lorafusion/ops/triton_ops/fused_lora_xw_sb.py:209-316, fused_lora_xw_sb_tma.py:244-392) and
  * fused_multi_lora_xw_sb (fused_multi_lora_xw_sb.py:221-339).  bias may be NULL.  With S = NULL
@@ -110,6 +118,12 @@ int lf_lora_dyw_dsa(const void* dY, const void* W, const void* dS, const void* c
 int lf_lora_fwd(const void* X, const void* W, const void* bias, const uint8_t* mask, const void* const* a_ptrs,
                 const void* const* b_ptrs, void* Y, void* S_out, void* workspace, size_t ws_bytes, int M, int N,
                 int K, int R, const lf_routing* routing, int dtype, void* stream);
+
+/* Whole forward with the mask drawn from `seed`: lf_lora_xa_seeded then lf_lora_xw_sb
+ * (lorafusion/ops/lora_v1.py:87-129 called without a precomputed mask). */
+int lf_lora_fwd_seeded(const void* X, const void* W, const void* bias, uint8_t* mask_out, const void* const* a_ptrs,
+                       const void* const* b_ptrs, void* Y, void* S_out, int M, int N, int K, int R,
+                       const lf_routing* routing, uint64_t seed, int dtype, void* stream);
 
 /* Whole backward: lf_lora_dys_dyb, lf_lora_da, and (dX != NULL) lf_lora_dyw_dsa.  Stands in
  * for _fused_linear_lora_backward (lorafusion/ops/lora_v1.py:132-166) and

@@ -22,6 +22,7 @@ LF_OK, LF_EINVAL, LF_ESHAPE, LF_EWORKSPACE, LF_ELAUNCH, LF_ELIMIT = 0, -1, -2, -
 EXPORTS = (
     "lf_version", "lf_strerror", "lf_workspace_bytes", "lf_lora_xa", "lf_lora_xw_sb", "lf_lora_dys_dyb",
     "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant", "lf_dropout_mask",
+    "lf_lora_xa_seeded", "lf_lora_fwd_seeded",
 )
 
 
@@ -74,6 +75,8 @@ def lib() -> ctypes.CDLL:
     l.lf_gemm.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, vp]
     l.lf_nf4_dequant.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, i, i, i, vp]
     l.lf_dropout_mask.argtypes = [vp, i, i, ctypes.c_float, rp, ctypes.c_uint64, vp]
+    l.lf_lora_xa_seeded.argtypes = [vp, vp, vp, vp, i, i, i, rp, ctypes.c_uint64, i, vp]
+    l.lf_lora_fwd_seeded.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, rp, ctypes.c_uint64, i, vp]
     for name in EXPORTS:
         if name not in ("lf_strerror", "lf_workspace_bytes"):
             getattr(l, name).restype = i

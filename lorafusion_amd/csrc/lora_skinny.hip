@@ -27,6 +27,7 @@
 // 4-row x 16-column patch; lane 4j+c addresses row j, columns 4c..4c+3; each lane receives
 // its column's 4 rows).
 #include "lf_common.h"
+#include "philox.h"
 
 namespace {
 
@@ -155,10 +156,13 @@ constexpr int XA_ROWS = 16;
 constexpr int xa_waves(int rt) { return rt <= 2 ? 8 : rt <= 4 ? 4 : 2; }
 constexpr int xa_unroll(int rt) { return rt <= 1 ? 4 : rt <= 2 ? 2 : 1; }
 
-template <typename T, int RT>
+// GEN: the keep-mask is not read but drawn here (Philox, the definition of the standalone mask
+// kernel) from (seed, element index) and written to `mask_out` for the backward pass: the integer
+// work hides behind the X stream, and one launch and one 1-byte-per-element read disappear.
+template <typename T, int RT, bool GEN>
 __global__ void __launch_bounds__(xa_waves(RT) * 64)
-lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, T* __restrict__ S,
-               int M, int K, int R, const LfSegTable seg) {
+lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_t* __restrict__ mask_out,
+               uint32_t seed_lo, uint32_t seed_hi, T* __restrict__ S, int M, int K, int R, const LfSegTable seg) {
   constexpr int XA_WAVES = xa_waves(RT), XA_U = xa_unroll(RT);
   __shared__ __attribute__((aligned(16))) char patch_all[XA_WAVES * 2048 * (1 + RT)];
   __shared__ float red[XA_WAVES][XA_ROWS][RT * 16];
@@ -168,7 +172,8 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, T* __r
   const int blk = row0 / ROWS;
   const BlockInfo bi = block_info(seg, blk, M);
   const T* __restrict__ A = (const T*)seg.ptr[bi.seg];
-  const bool use_mask = mask != nullptr && bi.p > 0.f;
+  const bool use_mask = GEN ? true : (mask != nullptr && bi.p > 0.f);
+  const uint32_t thr = lf_keep_threshold(bi.p);
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
   const int nsteps = K / 64;
   char* patch = patch_all + wave * 2048 * (1 + RT);  // X patch, then one patch per 16 rank rows of A
@@ -177,11 +182,15 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, T* __r
   const int lrow = lane >> 3, lg = lane & 7;
   const T* xrow[2];
   const uint8_t* mrow[2];
+  int64_t erow[2];    // GEN: element index of this lane's first column in each of its two rows
+  bool row_real[2];   // GEN: the row exists (is not a clamped duplicate): its mask bytes are written
 #pragma unroll
   for (int i = 0; i < 2; i++) {
     const int r = min(row0 + i * 8 + lrow, Mrows - 1);
     xrow[i] = X + (int64_t)r * K + lg * 8;
     mrow[i] = mask + (int64_t)r * K + lg * 8;
+    erow[i] = (int64_t)r * K + lg * 8;
+    row_real[i] = row0 + i * 8 + lrow < Mrows;
   }
   const int wr_off[2] = {lrow * 128 + ((lg ^ ((lrow >> 1) & 7)) << 4), (8 + lrow) * 128 + ((lg ^ (((8 + lrow) >> 1) & 7)) << 4)};
   const int rd_row = li * 128, rd_key = (li >> 1) & 7;
@@ -201,7 +210,9 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, T* __r
 #pragma unroll
         for (int i = 0; i < 2; i++) {
           xv[b][u][i] = __builtin_nontemporal_load((const lf_u32x4*)(xrow[i] + s * 64));
-          if (use_mask) mv[b][u][i] = __builtin_nontemporal_load((const lf_u32x2*)(mrow[i] + s * 64));
+          if constexpr (!GEN) {
+            if (use_mask) mv[b][u][i] = __builtin_nontemporal_load((const lf_u32x2*)(mrow[i] + s * 64));
+          }
 #pragma unroll
           for (int c = 0; c < RT; c++) {
             const int ar = c * 16 + i * 8 + lrow;
@@ -219,6 +230,11 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, T* __r
       if (s < nsteps) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
+          if constexpr (GEN) {
+            const uint64_t ctr = (uint64_t)(erow[i] + s * 64) >> 2;
+            mv[b][u][i] = lf_u32x2{lf_keep4(ctr, thr, seed_lo, seed_hi), lf_keep4(ctr + 1, thr, seed_lo, seed_hi)};
+            if (row_real[i]) __builtin_nontemporal_store(mv[b][u][i], (lf_u32x2*)(mask_out + erow[i] + s * 64));
+          }
           *(lf_u32x4*)(patch + wr_off[i]) = use_mask ? apply_mask8(xv[b][u][i], mv[b][u][i]) : xv[b][u][i];
 #pragma unroll
           for (int c = 0; c < RT; c++) *(lf_u32x4*)(patch + (1 + c) * 2048 + wr_off[i]) = av[b][u][c][i];
@@ -587,33 +603,40 @@ static int pick_split(int nblk, int len, int min_split) {
 size_t lf_xa_workspace(int, int, int, const LfSegTable&) { return 0; }
 
 template <typename T, int RT>
-static int xa_launch(const void* X, const uint8_t* mask, void* S, int M, int K, int R, int64_t rows,
-                     const LfSegTable& seg, hipStream_t st) {
+static int xa_launch(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t seed, void* S, int M, int K, int R,
+                     int64_t rows, const LfSegTable& seg, hipStream_t st) {
   const unsigned grid = (unsigned)((rows + XA_ROWS - 1) / XA_ROWS);
-  hipLaunchKernelGGL((lora_xa_kernel<T, RT>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, (T*)S, M, K, R, seg);
+  if (mask_out != nullptr)
+    hipLaunchKernelGGL((lora_xa_kernel<T, RT, true>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
+                       (uint32_t)seed, (uint32_t)(seed >> 32), (T*)S, M, K, R, seg);
+  else
+    hipLaunchKernelGGL((lora_xa_kernel<T, RT, false>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
+                       0u, 0u, (T*)S, M, K, R, seg);
   return lf_check_launch();
 }
 
 template <typename T>
-static int xa_impl(const void* X, const uint8_t* mask, void* S, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
+static int xa_impl(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t seed, void* S, int M, int K, int R,
+                   const LfSegTable& seg, hipStream_t st) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
   switch (rt_of(R)) {
-    case 1: return xa_launch<T, 1>(X, mask, S, M, K, R, rows, seg, st);
-    case 2: return xa_launch<T, 2>(X, mask, S, M, K, R, rows, seg, st);
-    case 4: return xa_launch<T, 4>(X, mask, S, M, K, R, rows, seg, st);
-    default: return xa_launch<T, 8>(X, mask, S, M, K, R, rows, seg, st);
+    case 1: return xa_launch<T, 1>(X, mask, mask_out, seed, S, M, K, R, rows, seg, st);
+    case 2: return xa_launch<T, 2>(X, mask, mask_out, seed, S, M, K, R, rows, seg, st);
+    case 4: return xa_launch<T, 4>(X, mask, mask_out, seed, S, M, K, R, rows, seg, st);
+    default: return xa_launch<T, 8>(X, mask, mask_out, seed, S, M, K, R, rows, seg, st);
   }
 }
 
-int lf_launch_xa(const void* X, const uint8_t* mask, void* S, void* ws, size_t ws_bytes, int M, int K, int R,
+// mask_out != nullptr: draw the keep-mask from `seed` (written to mask_out [rows, K]) instead of reading `mask`.
+int lf_launch_xa(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t seed, void* S, int M, int K, int R,
                  const LfSegTable& seg, int dtype, hipStream_t st) {
   if (!X || !S || M <= 0 || K <= 0) return LF_EINVAL;
   if (K % 128 != 0 || R % 16 != 0 || R <= 0 || R > LF_MAX_RANK) return LF_ESHAPE;
   if (seg.table && seg.block_size_m != ROWS) return LF_ESHAPE;
-  (void)ws; (void)ws_bytes;  // no partial sums leave the workgroups
-  if (dtype == LF_BF16) return xa_impl<__bf16>(X, mask, S, M, K, R, seg, st);
-  if (dtype == LF_F16) return xa_impl<_Float16>(X, mask, S, M, K, R, seg, st);
+  if (mask_out != nullptr && ((uintptr_t)mask_out & 7) != 0) return LF_ESHAPE;
+  if (dtype == LF_BF16) return xa_impl<__bf16>(X, mask, mask_out, seed, S, M, K, R, seg, st);
+  if (dtype == LF_F16) return xa_impl<_Float16>(X, mask, mask_out, seed, S, M, K, R, seg, st);
   return LF_EINVAL;
 }
 

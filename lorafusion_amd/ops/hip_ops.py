@@ -431,6 +431,21 @@ def lora_forward(x, w, a_list, b_list, routing_c, R, mask, bias):
     return y, s
 
 
+def lora_forward_seeded(x, w, a_list, b_list, routing_c, R, seed: int, bias):
+    """As ``lora_forward`` with the keep-mask drawn inside the rank-r kernel from ``seed``.
+    Returns (y, s, mask); the mask equals ``make_dropout_mask`` for the same seed and routing."""
+    M, K = x.shape
+    N = w.shape[0]
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    s = torch.empty((M, R), dtype=x.dtype, device=x.device)
+    mask = torch.empty((M, K), dtype=torch.bool, device=x.device)
+    rc = L.lib().lf_lora_fwd_seeded(L.ptr(x), L.ptr(w), L.ptr(bias), L.ptr(mask), L.ptr_array(a_list), L.ptr_array(b_list),
+                                    L.ptr(y), L.ptr(s), M, N, K, R, routing_c, ctypes.c_uint64(int(seed) & 0xFFFFFFFFFFFFFFFF),
+                                    L.dtype_id(x.dtype), L.stream_of(x))
+    L.check(rc, "lf_lora_fwd_seeded")
+    return y, s, mask
+
+
 def lora_backward(dy, x, w, a_list, b_list, s, routing_c, R, mask, rank_list, requires_dx: bool = True):
     """One C call: dS/dB, dA and (optionally) dX.  Returns (dx | None, da_list, db_list)."""
     M, N = dy.shape

@@ -63,18 +63,20 @@ class FusedLinearLoRA(torch.autograd.Function):
         linear_w, lora_a, lora_b = linear_w.contiguous(), lora_a.contiguous(), lora_b.contiguous()
         M, N, K, r = _validate(x2d, linear_w, lora_a, lora_b, linear_bias, dropout_p)
 
-        mask = None
-        if dropout_p > 0:
-            if dropout_mask is not None:
-                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
-            else:
-                if seed is None:
-                    seed = random.randrange(int(1e6))  # noqa: S311
-                mask = hip_ops.make_dropout_mask((M, K), dropout_p, seed, x2d.device)
         R = L.round_rank(r)
-        routing = L.single_routing(r, alpha, dropout_p if mask is not None else 0.0)
         bias = linear_bias.contiguous() if linear_bias is not None else None
-        y, s = hip_ops.lora_forward(x2d, linear_w, [lora_a], [lora_b], routing, R, mask, bias)
+        mask = None
+        if dropout_p > 0 and dropout_mask is None:
+            # the reference's default path: the keep-mask is drawn while X streams through the rank-r pass
+            if seed is None:
+                seed = random.randrange(int(1e6))  # noqa: S311
+            routing = L.single_routing(r, alpha, dropout_p)
+            y, s, mask = hip_ops.lora_forward_seeded(x2d, linear_w, [lora_a], [lora_b], routing, R, seed, bias)
+        else:
+            if dropout_p > 0:
+                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+            routing = L.single_routing(r, alpha, dropout_p if mask is not None else 0.0)
+            y, s = hip_ops.lora_forward(x2d, linear_w, [lora_a], [lora_b], routing, R, mask, bias)
 
         ctx.save_for_backward(x2d, linear_w, lora_a, lora_b, mask, s)
         ctx.alpha = alpha

@@ -216,15 +216,16 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
             raise ValueError(f"linear_bias must have shape [{N}] and dtype {x2d.dtype}.")
 
         mask = None
-        if routing.enable_dropout:
-            if dropout_mask is not None:
-                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
-            else:
-                if seed is None:
-                    seed = random.randrange(int(1e6))  # noqa: S311
-                mask = hip_ops.make_dropout_mask((M, K), None, seed, x2d.device, routing=routing)
         bias = linear_bias.contiguous() if linear_bias is not None else None
-        y, s = hip_ops.lora_forward(x2d, linear_w, a_list, b_list, routing.c, routing.R, mask, bias)
+        if routing.enable_dropout and dropout_mask is None:
+            # per-block p from the routing table, mask drawn inside the rank-r pass
+            if seed is None:
+                seed = random.randrange(int(1e6))  # noqa: S311
+            y, s, mask = hip_ops.lora_forward_seeded(x2d, linear_w, a_list, b_list, routing.c, routing.R, seed, bias)
+        else:
+            if routing.enable_dropout:
+                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+            y, s = hip_ops.lora_forward(x2d, linear_w, a_list, b_list, routing.c, routing.R, mask, bias)
 
         ctx.save_for_backward(x2d, linear_w, mask, s, *a_list, *b_list)
         ctx.routing = routing

@@ -180,17 +180,19 @@ class FusedLinearLoRANF4(torch.autograd.Function):
         lora_a, lora_b = lora_a.contiguous(), lora_b.contiguous()
         M, N, K, r = _validate(x2d, w, lora_a, lora_b, linear_bias, dropout_p)
         mask = None
-        if dropout_p > 0:
-            if dropout_mask is not None:
-                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
-            else:
-                if seed is None:
-                    seed = random.randrange(int(1e6))  # noqa: S311
-                mask = hip_ops.make_dropout_mask((M, K), dropout_p, seed, x2d.device)
-        p_eff = dropout_p if mask is not None else 0.0
-        routing = L.single_routing(r, alpha, p_eff)
         bias = linear_bias.contiguous() if linear_bias is not None else None
-        y, s = hip_ops.lora_forward(x2d, w, [lora_a], [lora_b], routing, L.round_rank(r), mask, bias)
+        if dropout_p > 0 and dropout_mask is None:
+            if seed is None:
+                seed = random.randrange(int(1e6))  # noqa: S311
+            p_eff = dropout_p
+            routing = L.single_routing(r, alpha, p_eff)
+            y, s, mask = hip_ops.lora_forward_seeded(x2d, w, [lora_a], [lora_b], routing, L.round_rank(r), seed, bias)
+        else:
+            if dropout_p > 0:
+                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+            p_eff = dropout_p if mask is not None else 0.0
+            routing = L.single_routing(r, alpha, p_eff)
+            y, s = hip_ops.lora_forward(x2d, w, [lora_a], [lora_b], routing, L.round_rank(r), mask, bias)
         ctx.save_for_backward(x2d, packed_w, lora_a, lora_b, mask, s)
         ctx.quant_state, ctx.alpha, ctx.p, ctx.lead = quant_state, alpha, p_eff, lead
         return y if lead is None else y.reshape(*lead, N)

@@ -89,3 +89,58 @@ def test_fused_ops_draw_their_mask_on_the_device():
     mask = torch.from_numpy(od.keep_mask(256, 512, p, seed)).bool().cuda()
     y_ref = fused_linear_lora(x, w, a, b, 2.0, dropout_p=p, dropout_mask=mask)
     assert torch.equal(y, y_ref)
+
+
+@pytest.mark.parametrize("ranks", [[16, 16, 16, 16], [8, 64, 32, 128]])
+def test_seeded_forward_draws_the_oracle_mask(ranks):
+    """The rank-r forward kernel that draws its own mask writes exactly the oracle's bytes (per-block p,
+    padded rows included) and produces the same S and Y, bit for bit, as the run fed that mask."""
+    from lorafusion_amd.ops import hip_ops
+    from lorafusion_amd.ops.multi_lora import prepare_multi_lora_batch_info
+    from tests.util import multi_inputs
+
+    seq, p_list, scales = [100, 300, 64, 257], [0.0, 0.05, 0.1, 0.3], [1.0, 2.0, 2.0, 4.0]
+    K, N, seed = 512, 384, 31337
+    d = multi_inputs(seq, K, N, ranks, p_list, seed=5)
+    info = prepare_multi_lora_batch_info(seq, [0, 1, 2, 3], ranks, p_list, scales, 128, output_dtype=torch.float32)
+    routing = hip_ops.MultiRouting(info.padded_seq_len_list, ranks, info.block_to_lookup_table, info.block_to_alpha,
+                                   info.block_to_dropout_p)
+    x, w = d["x"].cuda(), d["w"].cuda()
+    a_list, b_list = [t.cuda() for t in d["a_list"]], [t.cuda() for t in d["b_list"]]
+    y, s, mask = hip_ops.lora_forward_seeded(x, w, a_list, b_list, routing.c, routing.R, seed, None)
+    M = x.shape[0]
+    row_p = np.repeat(info.block_to_dropout_p.float().cpu().numpy(), 128)
+    expect = od.keep_mask(M, K, row_p, seed)
+    assert np.array_equal(mask.cpu().numpy().astype(np.uint8), expect)
+    y2, s2 = hip_ops.lora_forward(x, w, a_list, b_list, routing.c, routing.R, torch.from_numpy(expect).bool().cuda(), None)
+    assert torch.equal(s, s2) and torch.equal(y, y2)
+
+
+def test_seeded_multi_op_backward_uses_the_drawn_mask():
+    """fused_linear_multi_lora without an explicit mask: forward and backward agree with the oracle
+    evaluated on the mask the kernel drew."""
+    from lorafusion_amd.ops.multi_lora import fused_linear_multi_lora, prepare_multi_lora_batch_info
+    from oracle import lora_ref
+    from tests.util import multi_inputs
+
+    seq, ranks, p_list, scales = [200, 130], [16, 32], [0.1, 0.25], [2.0, 1.0]
+    K, N, seed = 256, 384, 77
+    d = multi_inputs(seq, K, N, ranks, p_list, seed=2)
+    info = prepare_multi_lora_batch_info(seq, [0, 1], ranks, p_list, scales, 128, output_dtype=torch.float32)
+    x = d["x"].cuda().requires_grad_(True)
+    a = [t.cuda().requires_grad_(True) for t in d["a_list"]]
+    b = [t.cuda().requires_grad_(True) for t in d["b_list"]]
+    y = fused_linear_multi_lora(
+        x.unsqueeze(0), d["w"].cuda(), lora_a_list=a, lora_b_list=b, seq_len_list=seq,
+        padded_seq_len_list=info.padded_seq_len_list, block_to_lookup_table=info.block_to_lookup_table,
+        block_to_dropout_p=info.block_to_dropout_p, block_to_alpha=info.block_to_alpha, enable_dropout=True,
+        same_dropout_p_value=None, max_r=32, seed=seed)
+    y.backward(d["dy"].cuda().unsqueeze(0))
+    M = x.shape[0]
+    mask = torch.from_numpy(od.keep_mask(M, K, np.repeat(info.block_to_dropout_p.float().cpu().numpy(), 128), seed)).bool()
+    ye, _ = lora_ref.linear_multi_lora_fwd_fp32(d["x"], d["w"], d["a_list"], d["b_list"], seq, d["padded"], scales, p_list, mask)
+    dxe, dae, dbe, _ = lora_ref.linear_multi_lora_bwd_fp32(d["dy"], d["x"], d["w"], d["a_list"], d["b_list"], seq, d["padded"],
+                                                           scales, p_list, mask)
+    for got, exp, name in [(y[0], ye, "y"), (x.grad, dxe, "dx"), (a[0].grad, dae[0], "da0"), (b[1].grad, dbe[1], "db1")]:
+        ok, rel, _ = lora_ref.check_close(got.detach().float().cpu(), exp, rtol=1e-2)
+        assert ok, f"{name}: {rel:.3e}"
