@@ -308,7 +308,7 @@ reduce_rows_kernel(const float* __restrict__ part, T* __restrict__ out, int npar
 template <typename T, int RT>
 __global__ void __launch_bounds__(256)
 lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __restrict__ ds_part,
-                    float* __restrict__ db_part, int M, int N, int R, int nslice, const LfSegTable seg) {
+                    float* __restrict__ db_part, int M, int N, int R, int tiles_per_wg, const LfSegTable seg) {
   constexpr int RP = RT * 32 + 32;
   extern __shared__ __attribute__((aligned(16))) char lds[];
   char* ys = lds;
@@ -321,8 +321,8 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
   const BlockInfo bi = block_info(seg, blk, M);
   const T* __restrict__ Bl = (const T*)seg.ptr[bi.seg];
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
-  const int n_begin = ns * nslice;
-  const int ntiles = nslice / 64;
+  const int n_begin = ns * tiles_per_wg * 64;
+  const int ntiles = min(tiles_per_wg, N / 64 - ns * tiles_per_wg);  // the last slice may be shorter
 
   auto load_b = [&](lf_u32x4 (&br)[(64 * RT * 2 + 255) / 256], int n0) {
 #pragma unroll
@@ -592,13 +592,31 @@ static int n_row_blocks(int M, const LfSegTable& seg) { return seg.table ? seg.n
 
 // Split of a length-`len` axis into slices (multiples of 64) so that blocks * split fills the
 // chip; `min_split` bounds the slice length from above.
-static int pick_split(int nblk, int len, int min_split) {
-  int split = 1;
-  while (split < min_split && (len % (split * 2 * 64)) == 0) split *= 2;
-  while (nblk * split < 512 && len / (split * 2) >= 128 && (len % (split * 2 * 64)) == 0) split *= 2;
-  return split;
+// Work split of the streaming passes.  A launch runs in rounds of resident workgroups (LDS-limited
+// slots per CU x 256 CUs); a workgroup walks `t` tiles in sequence, so the pass takes about
+// rounds * t tile times, plus a little per extra partial sum that the second stage must add.
+// Picks the t that minimises that (ties: larger t, fewer partials).  count(t) = workgroups at t.
+template <typename Count>
+static int pick_tiles_per_wg(int max_t, int slots, Count count) {
+  int best = 1;
+  double best_cost = 1e30;
+  for (int t = 1; t <= max_t; t++) {
+    const long wgs = count(t);
+    const double cost = (double)((wgs + slots - 1) / slots) * t + 0.15 * (double)wgs / (double)count(max_t);
+    if (cost <= best_cost) { best_cost = cost; best = t; }
+  }
+  return best;
 }
-
+static int lds_slots(int smem_bytes) {
+  const int per_cu = (160 * 1024) / smem_bytes;
+  return 256 * (per_cu > 0 ? per_cu : 1);
+}
+static int dys_smem(int rt) { return 2 * TILE_BYTES + ROWS * (rt * 32 + 32) + 2 * 64 * (rt * 32 + 32); }
+// 64-column dY tiles per workgroup; slices per row block = ceil((N/64) / t)
+static int dys_tiles_per_wg(int nblk, int N, int R) {
+  const int T = N / 64;
+  return pick_tiles_per_wg(T, lds_slots(dys_smem(rt_of(R))), [&](int t) { return (long)nblk * ((T + t - 1) / t); });
+}
 
 size_t lf_xa_workspace(int, int, int, const LfSegTable&) { return 0; }
 
@@ -643,17 +661,20 @@ int lf_launch_xa(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t
 size_t lf_dys_dyb_workspace(int M, int N, int R, const LfSegTable& seg) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  return ((size_t)pick_split(nblk, N, 1) * rows * R + (size_t)nblk * N * R) * sizeof(float);
+  const int t = dys_tiles_per_wg(nblk, N, R);
+  const int nsl = (N / 64 + t - 1) / t;
+  return ((size_t)nsl * rows * R + (size_t)nblk * N * R) * sizeof(float);
 }
 
 template <typename T, int RT>
-static int dys_launch(const void* dY, const void* S, float* ds_part, float* db_part, int M, int N, int R, int nslice,
+static int dys_launch(const void* dY, const void* S, float* ds_part, float* db_part, int M, int N, int R, int tiles_per_wg,
                       dim3 grid, const LfSegTable& seg, hipStream_t st) {
   auto kern = lora_dys_dyb_kernel<T, RT>;
   constexpr int RP = RT * 32 + 32;
-  const int smem = 2 * TILE_BYTES + ROWS * RP + 2 * 64 * RP;
+  const int smem = dys_smem(RT);
+  static_assert(RP == RT * 32 + 32, "");
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return LF_ELAUNCH;
-  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, nslice, seg);
+  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, tiles_per_wg, seg);
   return lf_check_launch();
 }
 
@@ -661,8 +682,8 @@ template <typename T>
 static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M, int N, int R, const LfSegTable& seg, hipStream_t st) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  const int split = pick_split(nblk, N, 1);
-  const int nslice = N / split;
+  const int nslice = dys_tiles_per_wg(nblk, N, R);       // tiles per workgroup
+  const int split = (N / 64 + nslice - 1) / nslice;       // slices per row block = partial sums of dS
   float* ds_part = (float*)ws;
   float* db_part = ds_part + (int64_t)split * rows * R;
   dim3 grid(nblk, split);
@@ -698,25 +719,32 @@ int lf_launch_dys_dyb(const void* dY, const void* S, void* dS, void* ws, size_t 
   return LF_EINVAL;
 }
 
-// dA chunking: `group` consecutive blocks per workgroup, chosen so the grid has >= ~1024 workgroups.
-static void da_shape(int M, int K, const LfSegTable& seg, int& group, int& max_chunks) {
+// dA chunking: `group` consecutive 128-row blocks of a segment per workgroup, chosen by the same
+// round model as the other passes (a segment of b blocks gives ceil(b / group) chunks per K tile).
+static int da_smem(int rt) { return 2 * TILE_BYTES + 2 * ROWS * (rt * 32 + 32); }
+static void da_shape(int M, int K, int R, const LfSegTable& seg, int& group, int& max_chunks) {
   const int nseg = seg.table ? seg.n_seg : 1;
+  int blocks[LF_MAX_SEG];
   int max_blocks = 0;
   for (int s = 0; s < nseg; s++) {
     int b0 = seg.table ? seg.first_block[s] : 0;
     int b1 = seg.table ? ((s + 1 < nseg) ? seg.first_block[s + 1] : seg.n_blocks) : (M + ROWS - 1) / ROWS;
-    max_blocks = (b1 - b0) > max_blocks ? (b1 - b0) : max_blocks;
+    blocks[s] = b1 - b0;
+    max_blocks = blocks[s] > max_blocks ? blocks[s] : max_blocks;
   }
-  const int nblk = n_row_blocks(M, seg);
-  group = 8;
-  while (group > 1 && (int64_t)(K / 64) * ((nblk + group - 1) / group) < 1024) group /= 2;
+  if (max_blocks < 1) max_blocks = 1;
+  group = pick_tiles_per_wg(max_blocks < 16 ? max_blocks : 16, lds_slots(da_smem(rt_of(R))), [&](int g) {
+    long chunks = 0;
+    for (int s = 0; s < nseg; s++) chunks += (blocks[s] + g - 1) / g;
+    return (long)(K / 64) * chunks;
+  });
   max_chunks = (max_blocks + group - 1) / group;
   if (max_chunks < 1) max_chunks = 1;
 }
 
 size_t lf_da_workspace(int M, int K, int R, const LfSegTable& seg) {
   int group, max_chunks;
-  da_shape(M, K, seg, group, max_chunks);
+  da_shape(M, K, R, seg, group, max_chunks);
   const int nseg = seg.table ? seg.n_seg : 1;
   return (size_t)nseg * max_chunks * R * K * sizeof(float);
 }
@@ -735,7 +763,7 @@ static int da_launch(const void* X, const uint8_t* mask, const void* dS, float* 
 template <typename T>
 static int da_impl(const void* X, const uint8_t* mask, const void* dS, void* ws, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
   int group, max_chunks;
-  da_shape(M, K, seg, group, max_chunks);
+  da_shape(M, K, R, seg, group, max_chunks);
   const int nseg = seg.table ? seg.n_seg : 1;
   float* part = (float*)ws;
   dim3 grid(K / 64, max_chunks, nseg);
