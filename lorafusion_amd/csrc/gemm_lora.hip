@@ -13,7 +13,8 @@
 // and the dense K-loop adds on top of it in fp32.
 //
 // Structure: one workgroup per BMxBN tile, 64-wide wavefronts each owning a WMxWN sub-tile of
-// 32x32x16 MFMA blocks.  The K loop advances in steps of BK = 32 through a ring of NSTAGE LDS
+// 16x16x32 MFMA blocks (under the power limit of the chip this shape sustains about 10 % more
+// than 32x32x16: 2.13 vs 1.93 PFLOP/s in a register-only loop with random operands).  The K loop advances in steps of BK = 32 through a ring of NSTAGE LDS
 // stages; both operand tiles go global -> LDS with 16-byte direct-to-LDS buffer loads (no VGPR
 // staging, no vector ALU address work: the per-lane row offset is loop invariant and the K
 // position is a scalar offset).  NSTAGE-1 stages of loads are in flight while one stage is
@@ -21,15 +22,15 @@
 // the unloaded one) is longer than the MFMA time of a K step and every step stalls on it
 // (measured: 1.18 -> 1.5 PFLOP/s on a loads+MFMA skeleton when a second stage may stay in
 // flight).  LDS rows are 64 bytes (4 granules of 16 bytes); granule g of row r is stored at
-// slot g ^ ((r>>2)&3) so that any 16 consecutive lanes of a ds_read_b128 fragment read (16
-// rows, one granule each) touch all 64 banks exactly once; the swizzle is applied on the
-// global side of the direct load (each lane fetches the granule whose LDS slot it owns).
+// slot g ^ ((r>>1)&3).  A ds_read_b128 is served 16 lanes at a time, and the lanes served
+// together are {0-3, 12-15, 20-27} and {4-11, 16-19, 28-31} of each half wave (probed on
+// hardware): with this swizzle each such set (rows 0-3 and 12-15 of one granule column, rows
+// 4-11 of the next) touches all 64 banks exactly once.  The swizzle is applied on the global
+// side of the direct load (each lane fetches the granule whose LDS slot it owns).
 // The NN operand is stored untransposed and read with ds_read_b64_tr_b16, which hands each
-// lane four consecutive contraction elements of its column.  Fragments are double buffered
-// in registers (the reads of MFMA k-step ks+1 are issued before the MFMAs of ks) and each K
-// step has one barrier, placed between its two MFMA k-steps.  MFMA operands are swapped (B
+// lane four consecutive contraction elements of its column.  MFMA operands are swapped (B
 // fragment as the "a" operand) so each lane ends with four consecutive output columns of one
-// row and stores 8 bytes at a time.
+// row.
 #include "lf_common.h"
 #include <type_traits>
 
@@ -48,8 +49,8 @@ constexpr int BK = 32;
 
 template <typename T> struct MfmaOp;
 template <> struct MfmaOp<__bf16> {
-  static __device__ __forceinline__ lf_f32x16 run(lf_u32x4 a, lf_u32x4 b, lf_f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(lf_bf16x8, a), __builtin_bit_cast(lf_bf16x8, b), c, 0, 0, 0);
+  static __device__ __forceinline__ lf_f32x4 run(lf_u32x4 a, lf_u32x4 b, lf_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lf_bf16x8, a), __builtin_bit_cast(lf_bf16x8, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
@@ -59,8 +60,8 @@ template <> struct MfmaOp<__bf16> {
   static __device__ __forceinline__ float to_float(uint16_t bits) { return __builtin_bit_cast(float, (uint32_t)bits << 16); }
 };
 template <> struct MfmaOp<_Float16> {
-  static __device__ __forceinline__ lf_f32x16 run(lf_u32x4 a, lf_u32x4 b, lf_f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(lf_f16x8, a), __builtin_bit_cast(lf_f16x8, b), c, 0, 0, 0);
+  static __device__ __forceinline__ lf_f32x4 run(lf_u32x4 a, lf_u32x4 b, lf_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(lf_f16x8, a), __builtin_bit_cast(lf_f16x8, b), c, 0, 0, 0);
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -94,14 +95,15 @@ __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64, 1)
 gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (buffer-resource types are device-only)
   constexpr int NWM = BM / WM, NWN = BN / WN, NWAVES = NWM * NWN, NTHREADS = NWAVES * 64;
-  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int TM = WM / 16, TN = WN / 16;  // 16x16 accumulator blocks per wave
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "sub-tile shape");
   constexpr int A_STAGE = BM * BK * 2, B_STAGE = BN * BK * 2;
   constexpr int NLA = BM * 4 / NTHREADS;  // 16-byte loads per thread per A tile (rows of 4 granules)
   constexpr int NLB = BN * 4 / NTHREADS;
   static_assert(NLA >= 1 && NLB >= 1 && (NTHREADS / 4) % 16 == 0, "tile/thread shape");
   constexpr int GPR = BN / 8;             // NN: granules per LDS row of the B tile
   constexpr int BPITCH = BN * 2;          // NN: bytes per LDS row of the B tile
-  constexpr int BKEY = BPITCH / 64 >= 4 ? 3 : BPITCH / 64 - 1;  // NN: swizzle key mask over 64-byte segments
+  constexpr int BKEY = BPITCH / 32 >= 8 ? 7 : BPITCH / 32 - 1;  // NN: swizzle key mask over 32-byte units
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   char* ldsA = smem;
@@ -111,7 +113,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / NWN, wn = wave % NWN;
-  const int l32 = lane & 31, q = lane >> 5;
+  const int l16 = lane & 15, kg = lane >> 4;  // row / column within a 16x16 block, group of 8 contraction elements
 
   // ---- tile mapping: XCD-aware (consecutive tiles stay on one XCD's L2) + grouped along M
   int pid = blockIdx.x;
@@ -138,8 +140,8 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, 0x7fffffff, 0x00020000);
   uint32_t avoff[NLA], bvoff[NLB];
   {
-    // LDS slot (tid&3) of row r holds source granule slot ^ ((r>>2)&3); r>>2 = tid>>4 (mod 4)
-    const int srcg = (tid & 3) ^ ((tid >> 4) & 3);
+    // LDS slot (tid&3) of row r holds source granule slot ^ ((r>>1)&3); r>>1 = tid>>3 (mod 4)
+    const int srcg = (tid & 3) ^ ((tid >> 3) & 3);
 #pragma unroll
     for (int i = 0; i < NLA; i++) {
       int row = i * (NTHREADS / 4) + (tid >> 2);
@@ -156,10 +158,13 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     } else {
 #pragma unroll
       for (int i = 0; i < NLB; i++) {
+        // 32-byte unit u of LDS row r holds source unit u ^ key(r), key(r) = (r&3)*2 + ((r>>3)&1): the
+        // 8 rows that 32 lanes of a transposed read touch (r, r+8 for four consecutive r) then cover
+        // all 64 banks
         int gid = i * NTHREADS + tid;
         int row = gid / GPR, g = gid % GPR;
-        int srcseg = (g >> 2) ^ (row & BKEY);
-        int col = min(n0 + (srcseg * 4 + (g & 3)) * 8, p.N - 8);
+        int srcunit = (g >> 1) ^ ((((row & 3) << 1) | ((row >> 3) & 1)) & BKEY);
+        int col = min(n0 + (srcunit * 2 + (g & 1)) * 8, p.N - 8);
         bvoff[i] = (uint32_t)((int64_t)row * p.ldb * 2 + col * 2);
       }
     }
@@ -205,13 +210,11 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   using std::integral_constant;
   using Steps0 = integral_constant<int, 0>;
 
-  lf_f32x16 acc[TM][TN];
+  lf_f32x4 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
-#pragma unroll
-      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+    for (int j = 0; j < TN; j++) acc[i][j] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
 
   // K steps are loaded in pairs (2T, 2T+1): the two 64-byte halves of the same 128-byte lines,
   // issued back to back so that the second request for a line meets the first in the L1 instead
@@ -253,153 +256,148 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     // targets before the main loop.  Granule g of row r sits at slot g ^ ((r / MRW) & (MLPR-1)):
     // the 4-byte reads of 32 rows then spread over the banks (2-way instead of 16-way conflicts).
     constexpr int MLPR = WN / 16, MRPI = 64 / MLPR, MNI = 32 / MRPI, MRW = 256 / WN;
+    constexpr int TM32 = WM / 32;  // 32-row bands of the sub-tile
     static_assert(NWM == 2 && MNI >= 1, "mask staging: 32 rows x WN bytes per wave fit B_STAGE / NWAVES");
     char* mreg = ldsB + (NSTAGE - 1) * B_STAGE + wave * (B_STAGE / NWAVES);
     const int mrow = lane / MLPR, mg = lane % MLPR;
-    constexpr bool MEARLY = TM * MNI <= 8;  // all mask loads up front while they fit in 32 registers
-    lf_u32x4 mv[TM][MNI];
+    constexpr bool MEARLY = TM32 * MNI <= 8;  // all mask loads up front while they fit in 32 registers
+    lf_u32x4 mv[TM32][MNI];
     const int mcol = min(n0 + wn * WN + mg * 16, p.N - 16);
-    auto load_mask_band = [&](int i) {
+    auto load_mask_band = [&](int ib) {
 #pragma unroll
       for (int ii = 0; ii < MNI; ii++) {
-        const int gm = min(wrow0 + i * 32 + ii * MRPI + mrow, p.M - 1);
-        mv[i][ii] = *(const lf_u32x4*)(p.mask + (int64_t)gm * p.ldmask + mcol);
+        const int gm = min(wrow0 + ib * 32 + ii * MRPI + mrow, p.M - 1);
+        mv[ib][ii] = *(const lf_u32x4*)(p.mask + (int64_t)gm * p.ldmask + mcol);
       }
     };
     if (use_mask && MEARLY) {
 #pragma unroll
-      for (int i = 0; i < TM; i++) load_mask_band(i);
+      for (int ib = 0; ib < TM32; ib++) load_mask_band(ib);
     }
-    for (int t = 0; t < p.R / 16; t++) {
-      const int r0 = t * 16 + q * 8;
-      lf_u32x4 lf[TM], rf[TN];
-#pragma unroll
-      for (int i = 0; i < TM; i++) {
-        int gm = min(wrow0 + i * 32 + l32, p.M - 1);
-        lf[i] = *(const lf_u32x4*)(L + (int64_t)gm * p.R + r0);
-      }
+    const __amdgpu_buffer_rsrc_t rsrcR = __builtin_amdgcn_make_buffer_rsrc((void*)rp, 0, 0x7fffffff, 0x00020000);
+    // one MFMA k-step covers 32 rank columns; lanes whose 8 columns lie beyond R (or the rank) feed zeros
+    for (int t = 0; t < (p.R + 31) / 32; t++) {
+      const int r0 = t * 32 + kg * 8;
+      lf_u32x4 rf[TN];
 #pragma unroll
       for (int j = 0; j < TN; j++) {
-        int gn = min(n0 + wn * WN + j * 32 + l32, p.N - 1);
+        int gn = min(n0 + wn * WN + j * 16 + l16, p.N - 1);
         lf_u32x4 v = {0, 0, 0, 0};
         if (r0 < rank) {
           if constexpr (!NN) {
             v = *(const lf_u32x4*)(rp + (int64_t)gn * rank + r0);
           } else {
-            const uint16_t* r16 = (const uint16_t*)rp;
+            // eight rows of one column: buffer loads that share a per-lane offset (row kg*8 of the
+            // step, column gn) and take the row as a scalar offset, so the 8 x TN loads in flight
+            // need no address registers of their own
+            const uint32_t voff = (uint32_t)((kg * 8 * p.N + gn) * 2);
             uint32_t e[8];
 #pragma unroll
-            for (int k = 0; k < 8; k++) e[k] = r16[(int64_t)(r0 + k) * p.N + gn];
+            for (int k = 0; k < 8; k++) e[k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcR, voff, (t * 32 + k) * p.N * 2, 0);
             v[0] = e[0] | (e[1] << 16); v[1] = e[2] | (e[3] << 16);
             v[2] = e[4] | (e[5] << 16); v[3] = e[6] | (e[7] << 16);
           }
         }
         rf[j] = v;
       }
+      constexpr int LCH = TM < 4 ? TM : 4;  // L fragments in flight (register budget)
 #pragma unroll
-      for (int i = 0; i < TM; i++)
+      for (int i0 = 0; i0 < TM; i0 += LCH) {
+        lf_u32x4 lf[LCH];
 #pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(rf[j], lf[i], acc[i][j]);
+        for (int i = 0; i < LCH; i++) {
+          int gm = min(wrow0 + (i0 + i) * 16 + l16, p.M - 1);
+          lf_u32x4 v = {0, 0, 0, 0};
+          if (r0 < p.R) v = *(const lf_u32x4*)(L + (int64_t)gm * p.R + r0);
+          lf[i] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < LCH; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++) acc[i0 + i][j] = MfmaOp<T>::run(rf[j], lf[i], acc[i0 + i][j]);
+      }
     }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-      if (use_mask) {
-        if constexpr (!MEARLY) load_mask_band(i);
+      const int ib = i >> 1, h = i & 1;  // band of 32 rows, half of the band
+      if (use_mask && h == 0) {
+        if constexpr (!MEARLY) load_mask_band(ib);
 #pragma unroll
         for (int ii = 0; ii < MNI; ii++) {
           const int r = ii * MRPI + mrow;
-          *(lf_u32x4*)(mreg + r * WN + ((mg ^ ((r / MRW) & (MLPR - 1))) << 4)) = mv[i][ii];
+          *(lf_u32x4*)(mreg + r * WN + ((mg ^ ((r / MRW) & (MLPR - 1))) << 4)) = mv[ib][ii];
         }
       }
+      const int r = h * 16 + l16;  // this lane's row of the band
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         acc[i][j] *= mult;
         if (use_mask) {
+          const int dw = j * 4 + kg;  // dword of the 4 columns j*16 + kg*4 ..
+          const uint32_t mk = *(const uint32_t*)(mreg + r * WN + (((dw >> 2) ^ ((r / MRW) & (MLPR - 1))) << 4) + (dw & 3) * 4);
 #pragma unroll
-          for (int jj = 0; jj < 4; jj++) {
-            const int dw = j * 8 + jj * 2 + q;  // dword of the 4 columns j*32 + jj*8 + q*4 ..
-            const uint32_t mk = *(const uint32_t*)(mreg + l32 * WN + (((dw >> 2) ^ ((l32 / MRW) & (MLPR - 1))) << 4) + (dw & 3) * 4);
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-              acc[i][j][jj * 4 + e] = ((mk >> (8 * e)) & 0xffu) ? acc[i][j][jj * 4 + e] : 0.f;
-          }
+          for (int e = 0; e < 4; e++) acc[i][j][e] = ((mk >> (8 * e)) & 0xffu) ? acc[i][j][e] : 0.f;
         }
       }
     }
   }
 
-  // ---- per-lane LDS fragment offsets
+  // ---- per-lane LDS fragment offsets: a lane reads 8 contraction elements (granule kg) of row l16
   int a_off[TM], b_off[TN];
+  const int slot = (kg ^ ((l16 >> 1) & 3)) << 4;
 #pragma unroll
-  for (int i = 0; i < TM; i++) a_off[i] = (wm * WM + i * 32 + l32) * 64;
-  const int sw = (l32 >> 2) & 3;
+  for (int i = 0; i < TM; i++) a_off[i] = (wm * WM + i * 16 + l16) * 64 + slot;
   if constexpr (!NN) {
 #pragma unroll
-    for (int j = 0; j < TN; j++) b_off[j] = (wn * WN + j * 32 + l32) * 64;
+    for (int j = 0; j < TN; j++) b_off[j] = (wn * WN + j * 16 + l16) * 64 + slot;
   } else {
     // ds_read_b64_tr_b16: within a 16-lane group, lane 4j+c addresses row j, columns 4c..4c+3 and
-    // receives column (lane&15), rows 0..3.
-    const int grp = lane >> 4, li = lane & 15, j4 = li >> 2, c = li & 3;
-    const int row0 = (grp >> 1) * 8 + j4;
-    const int key = row0 & BKEY;
+    // receives column (lane&15), rows 0..3.  Group kg takes contraction rows kg*8.. (two reads).
+    const int j4 = l16 >> 2, c = l16 & 3;
+    const int row0 = kg * 8 + j4;
+    const int key = ((j4 << 1) | (kg & 1)) & BKEY;
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      int colb = (wn * WN + j * 32 + (grp & 1) * 16 + 4 * c) * 2;  // byte offset within the row
-      b_off[j] = row0 * BPITCH + (((colb >> 6) ^ key) << 6) + (colb & 63);
+      int colb = (wn * WN + j * 16 + 4 * c) * 2;  // byte offset within the row
+      b_off[j] = row0 * BPITCH + (((colb >> 5) ^ key) << 5) + (colb & 31);
     }
   }
 
-  lf_u32x4 fa[4][TM], fb[4][TN];  // [set * 2 + k-slice]; the anti-phase loop uses one set
-  lf_u32x2 fbt[4][TN][2];  // NN: halves of the B fragments, joined only after the wait that completes them
-  auto read_frags = [&](int buf, int stage, int ks) {
-    const char* sa = ldsA + stage * A_STAGE;
-    const char* sb = ldsB + stage * B_STAGE;
-    const int slot = ((2 * ks + q) ^ sw) << 4;
-#pragma unroll
-    for (int i = 0; i < TM; i++) fa[buf][i] = *(const lf_u32x4*)(sa + a_off[i] + slot);
-    if constexpr (!NN) {
-#pragma unroll
-      for (int j = 0; j < TN; j++) fb[buf][j] = *(const lf_u32x4*)(sb + b_off[j] + slot);
-    } else {
-#pragma unroll
-      for (int j = 0; j < TN; j++) {
-        const char* base = sb + b_off[j] + ks * 16 * BPITCH;
-        fbt[buf][j][0] = lds_read_tr16(base);
-        fbt[buf][j][1] = lds_read_tr16(base + 4 * BPITCH);
-      }
-    }
-  };
-  // one fragment of k-slice ks (idx < TM: A fragment idx, else B fragment idx - TM)
-  auto read_one = [&](int buf, int stage, int ks, int idx) {
-    const int slot = ((2 * ks + q) ^ sw) << 4;
+  lf_u32x4 fa[2][TM], fb[2][TN];  // two register sets; the anti-phase loop uses one
+  lf_u32x2 fbt[2][TN][2];  // NN: halves of the B fragments, joined only after the wait that completes them
+  // one fragment of a K step (idx < TM: A fragment idx, else B fragment idx - TM)
+  auto read_one = [&](int set, int stage, int idx) {
     if (idx < TM) {
-      fa[buf][idx < TM ? idx : 0] = *(const lf_u32x4*)(ldsA + stage * A_STAGE + a_off[idx < TM ? idx : 0] + slot);
+      fa[set][idx < TM ? idx : 0] = *(const lf_u32x4*)(ldsA + stage * A_STAGE + a_off[idx < TM ? idx : 0]);
     } else {
       const int j = idx - TM < TN ? idx - TM : 0;
       const char* sb = ldsB + stage * B_STAGE;
       if constexpr (!NN) {
-        fb[buf][j] = *(const lf_u32x4*)(sb + b_off[j] + slot);
+        fb[set][j] = *(const lf_u32x4*)(sb + b_off[j]);
       } else {
-        const char* base = sb + b_off[j] + ks * 16 * BPITCH;
-        fbt[buf][j][0] = lds_read_tr16(base);
-        fbt[buf][j][1] = lds_read_tr16(base + 4 * BPITCH);
+        fbt[set][j][0] = lds_read_tr16(sb + b_off[j]);
+        fbt[set][j][1] = lds_read_tr16(sb + b_off[j] + 4 * BPITCH);
       }
     }
   };
-  auto mfma_one = [&](int buf, int idx) {
-    const int i = idx / TN, j = idx % TN;
-    if constexpr (NN) fb[buf][j] = lf_u32x4{fbt[buf][j][0][0], fbt[buf][j][0][1], fbt[buf][j][1][0], fbt[buf][j][1][1]};
-    acc[i][j] = MfmaOp<T>::run(fb[buf][j], fa[buf][i], acc[i][j]);
+  auto read_frags = [&](int set, int stage) {
+#pragma unroll
+    for (int f = 0; f < TM + TN; f++) read_one(set, stage, f);
   };
-  auto mfmas = [&](int buf) {
+  auto mfma_one = [&](int set, int idx) {
+    const int i = idx / TN, j = idx % TN;
+    if constexpr (NN) fb[set][j] = lf_u32x4{fbt[set][j][0][0], fbt[set][j][0][1], fbt[set][j][1][0], fbt[set][j][1][1]};
+    acc[i][j] = MfmaOp<T>::run(fb[set][j], fa[set][i], acc[i][j]);
+  };
+  auto join_b = [&](int set) {
     if constexpr (NN) {
 #pragma unroll
-      for (int j = 0; j < TN; j++) fb[buf][j] = lf_u32x4{fbt[buf][j][0][0], fbt[buf][j][0][1], fbt[buf][j][1][0], fbt[buf][j][1][1]};
+      for (int j = 0; j < TN; j++) fb[set][j] = lf_u32x4{fbt[set][j][0][0], fbt[set][j][0][1], fbt[set][j][1][0], fbt[set][j][1][1]};
     }
+  };
+  auto mfma_range = [&](int set, int m0_, int m1_) {
 #pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-      for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(fb[buf][j], fa[buf][i], acc[i][j]);
+    for (int m = m0_; m < m1_; m++) acc[m / TN][m % TN] = MfmaOp<T>::run(fb[set][m % TN], fa[set][m / TN], acc[m / TN][m % TN]);
   };
   if constexpr (NWAVES <= 4) {
     // ---- main loop, one wave per SIMD: no neighbour to hide behind, so the fragments of step
@@ -416,7 +414,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
       // next step go out with the first half of the MFMAs, so that the second half covers the read
       // latency, and the tile loads spread evenly over the step -- the texture addresser takes
       // 16 cycles per load, and a wave that cannot issue a load cannot issue the MFMAs behind it.
-      constexpr int NFR = TM + TN, NM1 = TM * TN, NM = 2 * NM1, NR = 2 * NFR;
+      constexpr int NR = TM + TN, NM = TM * TN;  // fragment reads and MFMAs per step
       constexpr int NLD = LOAD.value ? 2 * NL : 0;  // lo/hi halves alternate: load l is half l&1 of load l>>1
       constexpr int LSTEP = NLD > 0 && NM / NLD > 0 ? NM / NLD : 1;
       constexpr int HALF = NM / 2 > 0 ? NM / 2 : 1, RPS = (NR + HALF - 1) / HALF;  // reads per MFMA slot
@@ -430,9 +428,9 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         if (m % LSTEP == 0 && m / LSTEP < NLD) load_l(m / LSTEP);
         if constexpr (NEXT.value) {
 #pragma unroll
-          for (int r = m * RPS; r < (m + 1) * RPS && r < NR; r++) read_one(nxt * 2 + r / NFR, s1, r / NFR, r % NFR);
+          for (int r = m * RPS; r < (m + 1) * RPS && r < NR; r++) read_one(nxt, s1, r);
         }
-        mfma_one(cur * 2 + m / NM1, m % NM1);
+        mfma_one(cur, m);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -451,8 +449,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     if (nk > 2) wait_loads(integral_constant<int, PAIR0 - 2>{});  // tiles 0 and 1
     else wait_loads(Steps0{});
     __syncthreads();
-    read_frags(0, 0, 0);
-    read_frags(1, 0, 1);
+    read_frags(0, 0);
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __syncthreads();  // every wave has read stage 0: step 0 may refill it
     while (kt + PAIR0 + 1 < nk) {  // two steps per trip: the register sets swap roles
@@ -467,52 +464,36 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     k_step(integral_constant<int, 0>{}, F_{}, T_{});
     k_step(integral_constant<int, 1>{}, F_{}, F_{});
   } else {
-  // ---- main loop, two wave groups in anti-phase.  Each K step of a wave is a memory phase (issue
-  // its share of a later tile's loads, read all fragments of the current tile into registers)
-  // followed by a compute phase (the MFMAs of the step, nothing else); every phase ends in a
-  // workgroup barrier.  The second half of the waves runs one phase behind the first, so on every
-  // SIMD one wave feeds the MFMA pipe while its neighbour moves data: LDS latency never sits
-  // between two MFMAs of a wave, and the phases are long enough (16 MFMAs) that the schedule does
-  // not depend on instruction-level interleaving.
+  // ---- main loop, two wave groups in anti-phase.  Each K step of a wave is a memory phase (read all
+  // fragments of the current tile into registers) followed by a compute phase (the MFMAs of the
+  // step, in odd steps with its share of a later pair of tile loads between them); every
+  // phase ends in a workgroup barrier.  The second half of the waves runs one phase behind the
+  // first, so on every SIMD one wave feeds the MFMA pipe while its neighbour moves data: LDS
+  // latency never sits between two MFMAs of a wave, and the barriers keep the two groups from
+  // drifting into computing (or reading) at the same time -- with fewer barriers per step the
+  // loop measured slower.
   //   phase 2k   : group 0 reads tile k        | group 1 computes tile k-1
   //   phase 2k+1 : group 0 computes tile k     | group 1 reads tile k
   // Tile k is read in phases 2k and 2k+1; every wave waits for its own share of it in a memory
   // phase that ends no later than phase 2k-1, so the barrier closing that phase publishes the tile.
+  // Tile loads are issued from the compute phase of every odd step kt, spread between the MFMAs
+  // (the texture addresser takes 16 cycles per 64-lane 16-byte load: a burst of loads at the head
+  // of a memory phase would hold the LDS reads of four waves back behind it, and behind the reads
+  // they measured no faster): the pair (kt+3, kt+4) goes into the stages of steps kt-2 and kt-1
+  // (last read in phase 2kt-1).  At the end of the memory phase of an odd step the pair
+  // (kt+1, kt+2), issued two steps earlier, must have landed.
   const int grp = wave >= NWAVES / 2 ? 1 : 0;
   auto phase_barrier = [&]() {
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
-  // Two K steps of a wave.  Loads are issued from the compute phase of every odd step kt, spread
-  // between the MFMAs (the texture addresser takes 16 cycles per 64-lane 16-byte load: a burst of
-  // loads at the head of a memory phase would hold the LDS reads of four waves back behind it):
-  // the pair (kt+3, kt+4) goes into the stages of steps kt-2 and kt-1 (last read in phase 2kt-1).
-  // At the end of the memory phase of an odd step the pair (kt+1, kt+2), issued two steps earlier,
-  // must have landed.
   int stage = 0, kt = 0;
   static_assert(NSTAGE == 5, "the anti-phase loop is written for a ring of five stages");
-  auto step_pair = [&](auto LOAD) {
-    // even step
-    read_frags(0, stage, 0);
-    read_frags(1, stage, 1);
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    phase_barrier();
+  constexpr int NM = TM * TN;
+  auto compute_phase = [&](auto LOADC) {
     __builtin_amdgcn_s_setprio(1);
-    mfmas(0);
-    mfmas(1);
-    __builtin_amdgcn_s_setprio(0);
-    phase_barrier();
-    stage = stage + 1 == NSTAGE ? 0 : stage + 1;
-    kt++;
-    // odd step: the pair (kt+1, kt+2) must have landed; issue the pair (kt+3, kt+4)
-    read_frags(0, stage, 0);
-    read_frags(1, stage, 1);
-    wait_loads(Steps0{});
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    phase_barrier();
-    __builtin_amdgcn_s_setprio(1);
-    if constexpr (LOAD.value) {
+    if constexpr (LOADC.value) {
       const int s3 = stage + 3 >= NSTAGE ? stage + 3 - NSTAGE : stage + 3;
       const int s4 = stage + 4 >= NSTAGE ? stage + 4 - NSTAGE : stage + 4;
 #pragma unroll
@@ -521,10 +502,10 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         issue_load_one(s4, kt + 4, i);
       }
     }
-    mfmas(0);
-    mfmas(1);
-    if constexpr (LOAD.value) {
-      constexpr int NM = 2 * TM * TN, PER = NM / (2 * NL);
+    join_b(0);
+    mfma_range(0, 0, NM);
+    if constexpr (LOADC.value) {
+      constexpr int PER = NM / (2 * NL);
 #pragma unroll
       for (int r = 0; r < 2 * NL; r++) {
         __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
@@ -537,6 +518,19 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     stage = stage + 1 == NSTAGE ? 0 : stage + 1;
     kt++;
   };
+  auto step_pair = [&](auto LOAD) {
+    // even step
+    read_frags(0, stage);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    phase_barrier();
+    compute_phase(integral_constant<bool, false>{});
+    // odd step: the pair (kt+1, kt+2) must have landed; issue the pair (kt+3, kt+4)
+    read_frags(0, stage);
+    wait_loads(Steps0{});
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    phase_barrier();
+    compute_phase(LOAD);
+  };
   if (nk > 2) wait_loads(integral_constant<int, 2>{});
   else wait_loads(Steps0{});
   __syncthreads();
@@ -548,46 +542,48 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 
   // ---- epilogue: bias, convert, then one 32-row band of the wave's sub-tile at a time through the
   // wave's own LDS region so that global stores are 16 bytes per lane and cover whole rows of
-  // the sub-tile (WN*2 contiguous bytes) instead of 8-byte pieces scattered over 32 rows.
-  // Granule g (16 bytes) of band row r sits at slot g ^ (r & EP_KEY).
+  // the sub-tile (WN*2 contiguous bytes) instead of 8-byte pieces scattered over 16 rows.
+  // Granule g (16 bytes) of band row r sits at slot g ^ ((r / EP_RPW) & EP_KEY): EP_RPW rows span
+  // the 64 banks once, so the 16 rows that write together land on different banks.
   T* __restrict__ C = (T*)p.C;
   const uint16_t* bias16 = (const uint16_t*)p.bias;
   constexpr int EP_PITCH = WN * 2;              // bytes per band row
   constexpr int EP_BAND = 32 * EP_PITCH;        // bytes per band
   constexpr int LPR = EP_PITCH / 16;            // lanes per row on the way out
   constexpr int RPI = 64 / LPR;                 // rows per store instruction
-  constexpr int EP_KEY = LPR < 8 ? LPR - 1 : 7;
+  constexpr int EP_RPW = 256 / EP_PITCH > 0 ? 256 / EP_PITCH : 1;
+  constexpr int EP_KEY = LPR - 1;
   static_assert(2 * NWAVES * EP_BAND <= NSTAGE * (A_STAGE + B_STAGE), "epilogue staging fits the ring");
   __syncthreads();  // every wave is done with the ring
   char* ep = smem + wave * (2 * EP_BAND);
-  float bv[TN][4][4];
+  float bv[TN][4];
 #pragma unroll
-  for (int j = 0; j < TN; j++)
+  for (int j = 0; j < TN; j++) {
+    const int gn = min(n0 + wn * WN + j * 16 + kg * 4, p.N - 4);
 #pragma unroll
-    for (int jj = 0; jj < 4; jj++) {
-      const int gn = min(n0 + wn * WN + j * 32 + jj * 8 + q * 4, p.N - 4);
-#pragma unroll
-      for (int e = 0; e < 4; e++) bv[j][jj][e] = bias16 != nullptr ? MfmaOp<T>::to_float(bias16[gn + e]) : 0.f;
-    }
+    for (int e = 0; e < 4; e++) bv[j][e] = bias16 != nullptr ? MfmaOp<T>::to_float(bias16[gn + e]) : 0.f;
+  }
   const int out_col = n0 + wn * WN + (lane % LPR) * 8;
 #pragma unroll
-  for (int i = 0; i < TM; i++) {
-    char* band = ep + (i & 1) * EP_BAND;
+  for (int ib = 0; ib < TM / 2; ib++) {
+    char* band = ep + (ib & 1) * EP_BAND;
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int h = 0; h < 2; h++) {
+      const int r = h * 16 + l16;
 #pragma unroll
-      for (int jj = 0; jj < 4; jj++) {
-        lf_u32x2 o = {MfmaOp<T>::pack2(acc[i][j][jj * 4 + 0] + bv[j][jj][0], acc[i][j][jj * 4 + 1] + bv[j][jj][1]),
-                      MfmaOp<T>::pack2(acc[i][j][jj * 4 + 2] + bv[j][jj][2], acc[i][j][jj * 4 + 3] + bv[j][jj][3])};
-        const int g = j * 4 + jj;  // granule index within the band row; q selects its half
-        *(lf_u32x2*)(band + l32 * EP_PITCH + ((g ^ (l32 & EP_KEY)) << 4) + q * 8) = o;
+      for (int j = 0; j < TN; j++) {
+        const lf_f32x4 a = acc[ib * 2 + h][j];
+        lf_u32x2 o = {MfmaOp<T>::pack2(a[0] + bv[j][0], a[1] + bv[j][1]), MfmaOp<T>::pack2(a[2] + bv[j][2], a[3] + bv[j][3])};
+        const int g = j * 2 + (kg >> 1);  // granule of the 4 columns j*16 + kg*4 ..; kg&1 selects its half
+        *(lf_u32x2*)(band + r * EP_PITCH + ((g ^ ((r / EP_RPW) & EP_KEY)) << 4) + (kg & 1) * 8) = o;
       }
+    }
 #pragma unroll
     for (int r = 0; r < 32 / RPI; r++) {
       const int row = r * RPI + lane / LPR;
       const int g = lane % LPR;
-      lf_u32x4 v = *(const lf_u32x4*)(band + row * EP_PITCH + ((g ^ (row & EP_KEY)) << 4));
-      const int gm = wrow0 + i * 32 + row;
+      lf_u32x4 v = *(const lf_u32x4*)(band + row * EP_PITCH + ((g ^ ((row / EP_RPW) & EP_KEY)) << 4));
+      const int gm = wrow0 + ib * 32 + row;
       if (gm < p.M && out_col < p.N) *(lf_u32x4*)(C + (int64_t)gm * p.ldc + out_col) = v;
     }
   }
