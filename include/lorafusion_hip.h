@@ -67,6 +67,8 @@ typedef struct lf_routing {
 #define LF_OP_DA 2
 #define LF_OP_FWD 3
 #define LF_OP_BWD 4
+#define LF_OP_NF4_FWD 5
+#define LF_OP_NF4_BWD 6
 
 int lf_version(void);
 const char* lf_strerror(int code);
@@ -148,6 +150,32 @@ int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int 
 int lf_nf4_dequant(const uint8_t* packed, const void* absmax, const float* code2, const float* absmax2,
                    const float* offset, void* out, int64_t n_elems, int blocksize, int blocksize2, int out_dtype,
                    void* stream);
+
+/* An NF4 base weight [N,K] in the layout lf_nf4_dequant reads (the tensors of a bitsandbytes
+ * QuantState: lorafusion/ops/triton_ops/dequantize_nf4.py:288-315). */
+typedef struct lf_nf4_weight {
+  const uint8_t* packed;  /* uint8 [N*K/2] */
+  const void* absmax;     /* uint8 [N*K/blocksize] when blocksize2 > 0, else float32 */
+  const float* code2;     /* float32 [256] or NULL */
+  const float* absmax2;   /* float32 [N*K/blocksize/blocksize2] or NULL */
+  const float* offset;    /* float32 [1] or NULL */
+  int32_t blocksize;
+  int32_t blocksize2;     /* 0: absmax is float32 (not nested) */
+} lf_nf4_weight;
+
+/* QLoRA forward / backward: the base weight is stored as NF4, dequantised into the head of
+ * `workspace` (2*N*K bytes, rounded up to 256) and fed to lf_lora_fwd / lf_lora_bwd, whose own
+ * workspace follows it; sizes from lf_workspace_bytes(LF_OP_NF4_FWD / LF_OP_NF4_BWD, ...).  Stands
+ * in for dequantize_nf4_triton followed by the fused LoRA linear, the flow the reference sketches
+ * in lorafusion/ops/experimental/fused_quantized_nf4_lora_xw_sb_tma.py:280-428.  With dX == NULL
+ * the backward needs no weight and dequantises nothing. */
+int lf_nf4_lora_fwd(const void* X, const lf_nf4_weight* W, const void* bias, const uint8_t* mask,
+                    const void* const* a_ptrs, const void* const* b_ptrs, void* Y, void* S_out, void* workspace,
+                    size_t ws_bytes, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream);
+int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const uint8_t* mask, const void* S,
+                    const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
+                    void* const* db_ptrs, void* dS_out, void* workspace, size_t ws_bytes, int M, int N, int K, int R,
+                    const lf_routing* routing, int dtype, void* stream);
 
 /* Seeded dropout keep-mask (1 = keep), uint8 [M, K], K % 16 == 0.  Stands in for the mask output of
  * seeded_dropout (lorafusion/ops/triton_ops/dropout.py:71-93) and, with `routing` carrying a block

@@ -16,13 +16,13 @@ LIB_PATH = os.path.join(_HERE, "liblorafusion_hip.so")
 
 LF_BF16, LF_F16 = 0, 1
 LF_MAX_SEG = 32
-LF_OP_XA, LF_OP_DYS_DYB, LF_OP_DA, LF_OP_FWD, LF_OP_BWD = range(5)
+LF_OP_XA, LF_OP_DYS_DYB, LF_OP_DA, LF_OP_FWD, LF_OP_BWD, LF_OP_NF4_FWD, LF_OP_NF4_BWD = range(7)
 LF_OK, LF_EINVAL, LF_ESHAPE, LF_EWORKSPACE, LF_ELAUNCH, LF_ELIMIT = 0, -1, -2, -3, -4, -5
 
 EXPORTS = (
     "lf_version", "lf_strerror", "lf_workspace_bytes", "lf_lora_xa", "lf_lora_xw_sb", "lf_lora_dys_dyb",
     "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant", "lf_dropout_mask",
-    "lf_lora_xa_seeded", "lf_lora_fwd_seeded",
+    "lf_lora_xa_seeded", "lf_lora_fwd_seeded", "lf_nf4_lora_fwd", "lf_nf4_lora_bwd",
 )
 
 
@@ -41,6 +41,20 @@ class Routing(ctypes.Structure):
         ("p", ctypes.c_float),
         ("seg_first_block", ctypes.c_int32 * LF_MAX_SEG),
         ("seg_rank", ctypes.c_int32 * LF_MAX_SEG),
+    ]
+
+
+class NF4Weight(ctypes.Structure):
+    """struct lf_nf4_weight."""
+
+    _fields_ = [
+        ("packed", ctypes.c_void_p),
+        ("absmax", ctypes.c_void_p),
+        ("code2", ctypes.c_void_p),
+        ("absmax2", ctypes.c_void_p),
+        ("offset", ctypes.c_void_p),
+        ("blocksize", ctypes.c_int32),
+        ("blocksize2", ctypes.c_int32),
     ]
 
 
@@ -77,6 +91,9 @@ def lib() -> ctypes.CDLL:
     l.lf_dropout_mask.argtypes = [vp, i, i, ctypes.c_float, rp, ctypes.c_uint64, vp]
     l.lf_lora_xa_seeded.argtypes = [vp, vp, vp, vp, i, i, i, rp, ctypes.c_uint64, i, vp]
     l.lf_lora_fwd_seeded.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, rp, ctypes.c_uint64, i, vp]
+    wp = ctypes.POINTER(NF4Weight)
+    l.lf_nf4_lora_fwd.argtypes = [vp, wp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, rp, i, vp]
+    l.lf_nf4_lora_bwd.argtypes = [vp, vp, wp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, rp, i, vp]
     for name in EXPORTS:
         if name not in ("lf_strerror", "lf_workspace_bytes"):
             getattr(l, name).restype = i

@@ -81,6 +81,12 @@ size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* 
       size_t a = lf_dys_dyb_workspace(M, N, R, t), b = lf_da_workspace(M, K, R, t);
       return align256(a > b ? a : b);
     }
+    case LF_OP_NF4_FWD:
+      return align256((size_t)N * K * 2) + align256(lf_xa_workspace(M, K, R, t));
+    case LF_OP_NF4_BWD: {
+      size_t a = lf_dys_dyb_workspace(M, N, R, t), b = lf_da_workspace(M, K, R, t);
+      return align256((size_t)N * K * 2) + align256(a > b ? a : b);
+    }
     default: return 0;
   }
 }
@@ -205,6 +211,36 @@ int lf_nf4_dequant(const uint8_t* packed, const void* absmax, const float* code2
                    void* stream) {
   return lf_launch_nf4_dequant(packed, absmax, code2, absmax2, offset, out, n_elems, blocksize, blocksize2,
                                out_dtype, (hipStream_t)stream);
+}
+
+int lf_nf4_lora_fwd(const void* X, const lf_nf4_weight* W, const void* bias, const uint8_t* mask,
+                    const void* const* a_ptrs, const void* const* b_ptrs, void* Y, void* S_out, void* workspace,
+                    size_t ws_bytes, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  if (!W || !W->packed || !W->absmax || N <= 0 || K <= 0) return LF_EINVAL;
+  const size_t wbytes = align256((size_t)N * K * 2);
+  if (!workspace || ws_bytes < wbytes || ((uintptr_t)workspace & 255) != 0) return LF_EWORKSPACE;
+  int rc = lf_launch_nf4_dequant(W->packed, W->absmax, W->code2, W->absmax2, W->offset, workspace, (int64_t)N * K,
+                                 W->blocksize, W->blocksize2, dtype, (hipStream_t)stream);
+  if (rc != LF_OK) return rc;
+  return lf_lora_fwd(X, workspace, bias, mask, a_ptrs, b_ptrs, Y, S_out, (char*)workspace + wbytes, ws_bytes - wbytes,
+                     M, N, K, R, routing, dtype, stream);
+}
+
+int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const uint8_t* mask, const void* S,
+                    const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
+                    void* const* db_ptrs, void* dS_out, void* workspace, size_t ws_bytes, int M, int N, int K, int R,
+                    const lf_routing* routing, int dtype, void* stream) {
+  if (N <= 0 || K <= 0) return LF_EINVAL;
+  const size_t wbytes = align256((size_t)N * K * 2);
+  if (!workspace || ws_bytes < wbytes || ((uintptr_t)workspace & 255) != 0) return LF_EWORKSPACE;
+  if (dX) {
+    if (!W || !W->packed || !W->absmax) return LF_EINVAL;
+    int rc = lf_launch_nf4_dequant(W->packed, W->absmax, W->code2, W->absmax2, W->offset, workspace, (int64_t)N * K,
+                                   W->blocksize, W->blocksize2, dtype, (hipStream_t)stream);
+    if (rc != LF_OK) return rc;
+  }
+  return lf_lora_bwd(dY, X, workspace, mask, S, a_ptrs, b_ptrs, dX, da_ptrs, db_ptrs, dS_out, (char*)workspace + wbytes,
+                     ws_bytes - wbytes, M, N, K, R, routing, dtype, stream);
 }
 
 int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream) {

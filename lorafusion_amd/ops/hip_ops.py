@@ -462,6 +462,37 @@ def lora_backward(dy, x, w, a_list, b_list, s, routing_c, R, mask, rank_list, re
     return dx, da_list, db_list
 
 
+def nf4_lora_forward(x, wref, a_list, b_list, routing_c, R, mask, bias):
+    """``lora_forward`` with the base weight given as NF4 (``nf4.NF4WeightRef``): one C call dequantises it
+    into the call's workspace and runs the forward on it.  Returns (y, s)."""
+    M, K = x.shape
+    N = wref.shape[0]
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    s = torch.empty((M, R), dtype=x.dtype, device=x.device)
+    ws, nbytes = _ws(L.LF_OP_NF4_FWD, M, N, K, R, routing_c, x.device)
+    rc = L.lib().lf_nf4_lora_fwd(L.ptr(x), ctypes.byref(wref.c), L.ptr(bias), L.ptr(mask), L.ptr_array(a_list),
+                                 L.ptr_array(b_list), L.ptr(y), L.ptr(s), L.ptr(ws), nbytes, M, N, K, R, routing_c,
+                                 L.dtype_id(x.dtype), L.stream_of(x))
+    L.check(rc, "lf_nf4_lora_fwd")
+    return y, s
+
+
+def nf4_lora_backward(dy, x, wref, a_list, b_list, s, routing_c, R, mask, rank_list, requires_dx: bool = True):
+    """``lora_backward`` with the base weight given as NF4.  Returns (dx | None, da_list, db_list)."""
+    M, N = dy.shape
+    K = x.shape[1]
+    dx = torch.empty((M, K), dtype=dy.dtype, device=dy.device) if requires_dx else None
+    da_list = [torch.empty((r, K), dtype=dy.dtype, device=dy.device) for r in rank_list]
+    db_list = [torch.empty((N, r), dtype=dy.dtype, device=dy.device) for r in rank_list]
+    ds = torch.empty((M, R), dtype=dy.dtype, device=dy.device)
+    ws, nbytes = _ws(L.LF_OP_NF4_BWD, M, N, K, R, routing_c, dy.device)
+    rc = L.lib().lf_nf4_lora_bwd(L.ptr(dy), L.ptr(x), ctypes.byref(wref.c), L.ptr(mask), L.ptr(s), L.ptr_array(a_list),
+                                 L.ptr_array(b_list), L.ptr(dx), L.ptr_array(da_list), L.ptr_array(db_list), L.ptr(ds),
+                                 L.ptr(ws), nbytes, M, N, K, R, routing_c, L.dtype_id(dy.dtype), L.stream_of(dy))
+    L.check(rc, "lf_nf4_lora_bwd")
+    return dx, da_list, db_list
+
+
 def gemm(a: torch.Tensor, b: torch.Tensor, *, trans_b: bool = True, bias=None, tile_cfg: int = -1) -> torch.Tensor:
     """Plain ``a @ b.T`` (trans_b) or ``a @ b`` with the same MFMA kernel, no LoRA term."""
     _check_2d(a, "a")

@@ -24,15 +24,23 @@ from lorafusion_amd.ops import hip_ops
 
 
 def _validate(x2d, linear_w, lora_a, lora_b, linear_bias, dropout_p):
-    for name, t in (("x", x2d), ("linear_w", linear_w), ("lora_a", lora_a), ("lora_b", lora_b)):
+    L.require_gpu(linear_w, "linear_w")
+    return _validate_shapes(x2d, tuple(linear_w.shape), linear_w.dtype, lora_a, lora_b, linear_bias, dropout_p)
+
+
+def _validate_shapes(x2d, w_shape, w_dtype, lora_a, lora_b, linear_bias, dropout_p):
+    """Shape / dtype checks of one LoRA linear; the base weight is given by shape and (dequantised) dtype."""
+    for name, t in (("x", x2d), ("lora_a", lora_a), ("lora_b", lora_b)):
         L.require_gpu(t, name)
         if t.dtype != x2d.dtype:
             raise ValueError(f"{name} must have dtype {x2d.dtype}, but got {t.dtype}.")
+    if w_dtype != x2d.dtype:
+        raise ValueError(f"linear_w must have dtype {x2d.dtype}, but got {w_dtype}.")
     L.dtype_id(x2d.dtype)
     M, K = x2d.shape
-    if linear_w.ndim != 2 or linear_w.shape[1] != K:
-        raise ValueError(f"linear_w must have shape [N, {K}], but got {tuple(linear_w.shape)}.")
-    N = linear_w.shape[0]
+    if len(w_shape) != 2 or w_shape[1] != K:
+        raise ValueError(f"linear_w must have shape [N, {K}], but got {tuple(w_shape)}.")
+    N = w_shape[0]
     if lora_a.ndim != 2 or lora_a.shape[1] != K:
         raise ValueError(f"lora_a must have shape [r, {K}], but got {tuple(lora_a.shape)}.")
     r = lora_a.shape[0]

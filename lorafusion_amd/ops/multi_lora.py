@@ -188,7 +188,8 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
     """Packed multi-adapter LoRA linear.  Adapter tensors are passed as ``*a_list, *b_list``."""
 
     @staticmethod
-    def forward(ctx, padded_x, linear_w, linear_bias, dropout_mask, seed, routing: MultiRouting, n_adapters, *ab):
+    def forward(ctx, padded_x, linear_w, linear_bias, dropout_mask, seed, routing: MultiRouting, quant_state,
+                n_adapters, *ab):
         if padded_x.ndim == THREE_DIM:
             if padded_x.shape[0] != 1:
                 raise ValueError("currently, we only support batch size 1 for multi-linear LoRA")
@@ -203,11 +204,20 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
         a_list = [t.contiguous() for t in ab[:n_adapters]]
         b_list = [t.contiguous() for t in ab[n_adapters:]]
         M, K = x2d.shape
-        N = linear_w.shape[0]
+        wref = None
+        if quant_state is not None:
+            # NF4 base weight: linear_w holds the packed codes, quant_state its bitsandbytes-style state
+            from lorafusion_amd.ops.nf4 import NF4WeightRef
+
+            wref = NF4WeightRef(linear_w, quant_state)
+            w_shape, w_dtype = tuple(wref.shape), wref.dtype
+        else:
+            w_shape, w_dtype = tuple(linear_w.shape), linear_w.dtype
         if M != routing.M:
             raise ValueError(f"padded_x has {M} rows but the batch info covers {routing.M}.")
-        if linear_w.ndim != 2 or linear_w.shape[1] != K or linear_w.dtype != x2d.dtype:
+        if len(w_shape) != 2 or w_shape[1] != K or w_dtype != x2d.dtype:
             raise ValueError(f"linear_w must have shape [N, {K}] and dtype {x2d.dtype}.")
+        N = w_shape[0]
         L.require_gpu(x2d, "padded_x")
         L.dtype_id(x2d.dtype)
         hip_ops._check_dims(M, N, K)
@@ -217,7 +227,13 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
 
         mask = None
         bias = linear_bias.contiguous() if linear_bias is not None else None
-        if routing.enable_dropout and dropout_mask is None:
+        if wref is not None:
+            if routing.enable_dropout:
+                if dropout_mask is None:
+                    dropout_mask = hip_ops.make_dropout_mask((M, K), 0.0, seed, x2d.device, routing=routing)
+                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+            y, s = hip_ops.nf4_lora_forward(x2d, wref, a_list, b_list, routing.c, routing.R, mask, bias)
+        elif routing.enable_dropout and dropout_mask is None:
             # per-block p from the routing table, mask drawn inside the rank-r pass
             if seed is None:
                 seed = random.randrange(int(1e6))  # noqa: S311
@@ -229,6 +245,7 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
 
         ctx.save_for_backward(x2d, linear_w, mask, s, *a_list, *b_list)
         ctx.routing = routing
+        ctx.quant_state = quant_state
         ctx.n_adapters = n_adapters
         ctx.lead = lead
         return y.reshape(1, M, N) if lead else y
@@ -248,13 +265,21 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
         else:
             raise ValueError(f"dy must be a 3D tensor, but got {dy.ndim}")
         dy2d = dy2d.contiguous()
-        dx, da_list, db_list = hip_ops.lora_backward(
-            dy2d, x2d, linear_w, a_list, b_list, s, routing.c, routing.R, mask, routing.rank_list,
-            requires_dx=ctx.needs_input_grad[0],
-        )
+        if ctx.quant_state is not None:
+            from lorafusion_amd.ops.nf4 import NF4WeightRef
+
+            dx, da_list, db_list = hip_ops.nf4_lora_backward(
+                dy2d, x2d, NF4WeightRef(linear_w, ctx.quant_state), a_list, b_list, s, routing.c, routing.R, mask,
+                routing.rank_list, requires_dx=ctx.needs_input_grad[0],
+            )
+        else:
+            dx, da_list, db_list = hip_ops.lora_backward(
+                dy2d, x2d, linear_w, a_list, b_list, s, routing.c, routing.R, mask, routing.rank_list,
+                requires_dx=ctx.needs_input_grad[0],
+            )
         if dx is not None and ctx.lead:
             dx = dx.reshape(1, *dx.shape)
-        return (dx, None, None, None, None, None, None, *da_list, *db_list)
+        return (dx, None, None, None, None, None, None, None, *da_list, *db_list)
 
 
 def fused_linear_multi_lora(
@@ -274,12 +299,15 @@ def fused_linear_multi_lora(
     linear_bias: torch.Tensor | None = None,
     dropout_mask: torch.Tensor | None = None,
     seed: int | None = None,
+    quant_state=None,
 ) -> torch.Tensor:
     """Fused multi-adapter LoRA linear (lorafusion/ops/multi_lora.py:762-830).
 
     ``padded_x`` is ``[1, sum(padded_seq_len_list), K]``; adapter i owns rows
     ``[cur_i, cur_i + seq_len_list[i])`` with ``cur`` advancing by the padded lengths.
-    ``dropout_mask`` / ``seed`` are extensions for reproducible runs.
+    ``dropout_mask`` / ``seed`` are extensions for reproducible runs.  With ``quant_state`` (the
+    bitsandbytes-style state ``dequantize_nf4_triton`` takes) ``linear_w`` holds packed NF4 codes and
+    is dequantised inside the forward and backward calls.
     """
     if len(lora_a_list) != len(lora_b_list):
         raise ValueError("lora_a_list and lora_b_list must have the same length")
@@ -294,7 +322,7 @@ def fused_linear_multi_lora(
         raise ValueError(f"max_r={max_r} is smaller than the largest adapter rank {max(rank_list)}")
     routing = MultiRouting(padded_seq_len_list, rank_list, block_to_lookup_table, block_to_alpha,
                            block_to_dropout_p, enable_dropout=enable_dropout)
-    return FusedLinearMultiLoRA.apply(padded_x, linear_w, linear_bias, dropout_mask, seed, routing,
+    return FusedLinearMultiLoRA.apply(padded_x, linear_w, linear_bias, dropout_mask, seed, routing, quant_state,
                                       len(lora_a_list), *lora_a_list, *lora_b_list)
 
 

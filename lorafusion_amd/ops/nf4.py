@@ -51,8 +51,8 @@ class QuantState:
         return self.state2 is not None
 
 
-def dequantize_nf4_triton(A: torch.Tensor, quant_state, out: torch.Tensor | None = None) -> torch.Tensor:
-    """Dequantise packed NF4 weights to ``quant_state.dtype`` (bf16 / fp16), shape ``quant_state.shape``."""
+def _checked_state(A: torch.Tensor, quant_state):
+    """Validate packed codes + quant state; returns the contiguous device tensors the kernels read."""
     L.require_gpu(A, "A")
     if A.dtype != torch.uint8:
         raise ValueError(f"A must be a uint8 tensor of packed 4-bit codes, but got {A.dtype}.")
@@ -87,6 +87,13 @@ def dequantize_nf4_triton(A: torch.Tensor, quant_state, out: torch.Tensor | None
         if absmax.dtype != torch.float32:
             raise ValueError("non-nested quant state: absmax must be float32.")
         bs2, code, absmax2, offset = 0, None, None, None
+    return A, absmax, code, absmax2, offset, blocksize, bs2, shape, out_dtype
+
+
+def dequantize_nf4_triton(A: torch.Tensor, quant_state, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Dequantise packed NF4 weights to ``quant_state.dtype`` (bf16 / fp16), shape ``quant_state.shape``."""
+    A, absmax, code, absmax2, offset, blocksize, bs2, shape, out_dtype = _checked_state(A, quant_state)
+    n = shape.numel()
     if out is None:
         out = torch.empty(n, dtype=out_dtype, device=A.device)
     elif out.numel() != n or out.dtype != out_dtype or not out.is_contiguous():
@@ -95,6 +102,19 @@ def dequantize_nf4_triton(A: torch.Tensor, quant_state, out: torch.Tensor | None
                                 blocksize, bs2, L.dtype_id(out_dtype), L.stream_of(A))
     L.check(rc, "lf_nf4_dequant")
     return out.view(shape)
+
+
+class NF4WeightRef:
+    """``struct lf_nf4_weight`` for a packed weight + quant state; keeps the tensors it points to alive."""
+
+    def __init__(self, A: torch.Tensor, quant_state):
+        tensors = _checked_state(A, quant_state)
+        A, absmax, code, absmax2, offset, blocksize, bs2, shape, out_dtype = tensors
+        if len(shape) != 2:
+            raise ValueError(f"the quantised weight must be 2-D [N, K], got shape {tuple(shape)}.")
+        self.keep = (A, absmax, code, absmax2, offset)
+        self.shape, self.dtype = shape, out_dtype
+        self.c = L.NF4Weight(L.ptr(A), L.ptr(absmax), L.ptr(code), L.ptr(absmax2), L.ptr(offset), blocksize, bs2)
 
 
 dequantize_nf4 = dequantize_nf4_triton
@@ -153,16 +173,15 @@ def quantize_nf4(w: torch.Tensor, blocksize: int = 64, compress_statistics: bool
 class FusedLinearLoRANF4(torch.autograd.Function):
     """QLoRA linear: NF4 base weight dequantised on the fly, bf16/fp16 adapters.
 
-    Forward and backward each dequantise the weight into a transient buffer with the HIP
-    kernel and run the fused LoRA GEMMs on it; only the packed weight stays resident.
+    Forward and backward each dequantise the weight into the call's workspace
+    (``lf_nf4_lora_fwd`` / ``lf_nf4_lora_bwd``) and run the fused LoRA GEMMs on it; only the
+    packed weight stays resident.
     """
 
     @staticmethod
     def forward(ctx, x, packed_w, quant_state, lora_a, lora_b, alpha, dropout_p, seed, linear_bias, dropout_mask):
-        import random
-
         from lorafusion_amd.ops import hip_ops
-        from lorafusion_amd.ops.lora_v1 import _validate
+        from lorafusion_amd.ops.lora_v1 import _validate_shapes
 
         if x.ndim == 3:
             lead = x.shape[:2]
@@ -174,25 +193,18 @@ class FusedLinearLoRANF4(torch.autograd.Function):
         x2d = x2d.contiguous()
         if quant_state.dtype != x2d.dtype:
             raise ValueError(f"quant_state.dtype {quant_state.dtype} must match x.dtype {x2d.dtype}.")
-        w = dequantize_nf4_triton(packed_w, quant_state)
-        if w.ndim != 2:
-            raise ValueError(f"the quantised weight must be 2-D [N, K], got shape {tuple(w.shape)}.")
+        wref = NF4WeightRef(packed_w, quant_state)
         lora_a, lora_b = lora_a.contiguous(), lora_b.contiguous()
-        M, N, K, r = _validate(x2d, w, lora_a, lora_b, linear_bias, dropout_p)
+        M, N, K, r = _validate_shapes(x2d, tuple(wref.shape), x2d.dtype, lora_a, lora_b, linear_bias, dropout_p)
         mask = None
         bias = linear_bias.contiguous() if linear_bias is not None else None
-        if dropout_p > 0 and dropout_mask is None:
-            if seed is None:
-                seed = random.randrange(int(1e6))  # noqa: S311
-            p_eff = dropout_p
-            routing = L.single_routing(r, alpha, p_eff)
-            y, s, mask = hip_ops.lora_forward_seeded(x2d, w, [lora_a], [lora_b], routing, L.round_rank(r), seed, bias)
-        else:
-            if dropout_p > 0:
-                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
-            p_eff = dropout_p if mask is not None else 0.0
-            routing = L.single_routing(r, alpha, p_eff)
-            y, s = hip_ops.lora_forward(x2d, w, [lora_a], [lora_b], routing, L.round_rank(r), mask, bias)
+        if dropout_p > 0:
+            if dropout_mask is None:
+                dropout_mask = hip_ops.make_dropout_mask((M, K), dropout_p, seed, x2d.device)
+            mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+        p_eff = dropout_p if mask is not None else 0.0
+        routing = L.single_routing(r, alpha, p_eff)
+        y, s = hip_ops.nf4_lora_forward(x2d, wref, [lora_a], [lora_b], routing, L.round_rank(r), mask, bias)
         ctx.save_for_backward(x2d, packed_w, lora_a, lora_b, mask, s)
         ctx.quant_state, ctx.alpha, ctx.p, ctx.lead = quant_state, alpha, p_eff, lead
         return y if lead is None else y.reshape(*lead, N)
@@ -204,11 +216,11 @@ class FusedLinearLoRANF4(torch.autograd.Function):
         x2d, packed_w, lora_a, lora_b, mask, s = ctx.saved_tensors
         dy2d = dy.reshape(-1, dy.shape[-1]).contiguous()
         r = lora_a.shape[0]
-        w = dequantize_nf4_triton(packed_w, ctx.quant_state) if ctx.needs_input_grad[0] else None
+        wref = NF4WeightRef(packed_w, ctx.quant_state)
         routing = L.single_routing(r, ctx.alpha, ctx.p)
-        w_arg = w if w is not None else x2d  # unused by the kernels when dx is not requested
-        dx, da_list, db_list = hip_ops.lora_backward(dy2d, x2d, w_arg, [lora_a], [lora_b], s, routing,
-                                                     L.round_rank(r), mask, [r], requires_dx=w is not None)
+        dx, da_list, db_list = hip_ops.nf4_lora_backward(dy2d, x2d, wref, [lora_a], [lora_b], s, routing,
+                                                         L.round_rank(r), mask, [r],
+                                                         requires_dx=ctx.needs_input_grad[0])
         if dx is not None and ctx.lead is not None:
             dx = dx.reshape(*ctx.lead, -1)
         return dx, None, None, da_list[0], db_list[0], None, None, None, None, None

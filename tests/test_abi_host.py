@@ -59,6 +59,15 @@ def test_argument_validation_without_gpu():
     # bad routing: rank not a multiple of 8, too many segments
     bad = _lib.single_routing(12, 1.0, 0.0)
     assert lib.lf_workspace_bytes(_lib.LF_OP_FWD, 256, 256, 256, 16, bad) == 0
+    # NF4 entry points: the workspace holds the dequantised weight ahead of the op's own scratch
+    wbytes = 256 * 256 * 2
+    assert lib.lf_workspace_bytes(_lib.LF_OP_NF4_FWD, 256, 256, 256, 16, r) == wbytes + lib.lf_workspace_bytes(_lib.LF_OP_FWD, 256, 256, 256, 16, r)
+    assert lib.lf_workspace_bytes(_lib.LF_OP_NF4_BWD, 256, 256, 256, 16, r) == wbytes + small
+    wq = _lib.NF4Weight(16, 16, None, None, None, 64, 0)
+    args_fwd = (one, ctypes.byref(wq), None, None, ptrs, ptrs, one, one)
+    assert lib.lf_nf4_lora_fwd(*args_fwd, None, 0, 256, 256, 256, 16, r, 0, None) == -3           # no workspace
+    assert lib.lf_nf4_lora_fwd(*args_fwd, ctypes.c_void_p(256), 100, 256, 256, 256, 16, r, 0, None) == -3   # too small
+    assert lib.lf_nf4_lora_fwd(one, None, None, None, ptrs, ptrs, one, one, ctypes.c_void_p(256), 1 << 20, 256, 256, 256, 16, r, 0, None) == -1
     bad2 = _lib.single_routing(16, 1.0, 0.0)
     bad2.n_seg = 64
     assert lib.lf_lora_xa(one, None, ptrs, one, one, 1 << 20, 128, 128, 16, bad2, 0, None) == -5

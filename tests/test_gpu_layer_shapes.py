@@ -51,7 +51,7 @@ def _nf4_weight(w_gpu):
     w_oracle = torch.from_numpy(onf4.dequantize(st).view(np.int16)).view(torch.bfloat16).reshape(w_gpu.shape)
     w_dev = dequantize_nf4_triton(packed, qs).reshape(w_gpu.shape)
     assert torch.equal(w_dev.cpu().view(torch.int16), w_oracle.view(torch.int16)), "NF4 dequant is not bit-exact"
-    return w_dev, w_oracle
+    return packed, qs, w_oracle
 
 
 def _run_multi(tokens, K, N, ranks, p_list, scale_list, nf4=False, seed=0):
@@ -71,8 +71,10 @@ def _run_multi(tokens, K, N, ranks, p_list, scale_list, nf4=False, seed=0):
     gm = torch.Generator(device="cuda").manual_seed(seed + 4)
     row_p = torch.cat([torch.full((pl,), float(p)) for pl, p in zip(padded, p_list)]).cuda()
     mask = torch.rand((Mp, K), generator=gm, device="cuda") >= row_p[:, None]
+    qs = None
     if nf4:
-        w, w_cpu = _nf4_weight(w)
+        # the op takes the packed codes + quant state and dequantises inside lf_nf4_lora_fwd / _bwd
+        w, qs, w_cpu = _nf4_weight(w)
     else:
         w_cpu = w.cpu()
 
@@ -80,7 +82,7 @@ def _run_multi(tokens, K, N, ranks, p_list, scale_list, nf4=False, seed=0):
         x.unsqueeze(0), w, lora_a_list=a_list, lora_b_list=b_list, seq_len_list=seq, padded_seq_len_list=padded,
         block_to_lookup_table=info.block_to_lookup_table, block_to_dropout_p=info.block_to_dropout_p,
         block_to_alpha=info.block_to_alpha, enable_dropout=info.enable_dropout,
-        same_dropout_p_value=info.same_dropout_p_value, max_r=info.max_r, dropout_mask=mask)
+        same_dropout_p_value=info.same_dropout_p_value, max_r=info.max_r, dropout_mask=mask, quant_state=qs)
     y.backward(dy.unsqueeze(0))
     torch.cuda.synchronize()
     y, dx = y[0].detach(), x.grad
@@ -127,7 +129,7 @@ def test_70b_layer_projections_nf4(K, N):
 
 def test_nf4_linear_4096_to_14336():
     """Single adapter, NF4 base weight [14336, 4096], 4096 tokens, r=16, p=0.1, scale 2."""
-    from lorafusion_amd.ops.nf4 import fused_linear_lora_nf4, quantize_nf4
+    from lorafusion_amd.ops.nf4 import fused_linear_lora_nf4
 
     M, K, N, r, p, scale = 4096, 4096, 14336, 16, 0.1, 2.0
     x = _gpu_randn((M, K), 1).requires_grad_(True)
@@ -137,8 +139,7 @@ def test_nf4_linear_4096_to_14336():
     b = _gpu_randn((N, r), 30, 0.01).requires_grad_(True)
     gm = torch.Generator(device="cuda").manual_seed(4)
     mask = torch.rand((M, K), generator=gm, device="cuda") >= p
-    _, w_cpu = _nf4_weight(w0)
-    packed, qs = quantize_nf4(w0.float())
+    packed, qs, w_cpu = _nf4_weight(w0)
     y = fused_linear_lora_nf4(x, packed, qs, a, b, scale, dropout_p=p, dropout_mask=mask)
     y.backward(dy)
     torch.cuda.synchronize()

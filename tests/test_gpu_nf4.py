@@ -121,3 +121,26 @@ def test_qlora_linear_parity():
     for got, exp, name in ((y, ye, "y"), (x.grad, dxe, "dx"), (a.grad, dae, "da"), (b.grad, dbe, "db")):
         ok, rel, excess = lora_ref.check_close(got.detach().float().cpu(), exp, rtol=1e-2)
         assert ok, f"{name}: rel {rel:.3e} excess {excess:.3e}"
+
+
+def test_qlora_linear_adapter_grads_only_and_seeded_mask():
+    """x without grad: the backward call gets dX = NULL and dequantises nothing; dropout mask from a seed."""
+    from lorafusion_amd.ops.hip_ops import make_dropout_mask
+    from lorafusion_amd.ops.nf4 import fused_linear_lora_nf4
+
+    M, K, N, r, p, scale = 256, 512, 384, 32, 0.25, 0.5
+    d = single_inputs(M, K, N, r, p=p, seed=11)
+    st = onf4.quantize_nf4(d["w"].float().numpy())
+    wq = torch.from_numpy(onf4.dequantize(st).view(np.int16)).view(torch.bfloat16).reshape(N, K)
+    packed, qs = _to_state(st)
+    x = d["x"].cuda()
+    a = d["a"].cuda().requires_grad_(True)
+    b = d["b"].cuda().requires_grad_(True)
+    y = fused_linear_lora_nf4(x, packed, qs, a, b, scale, seed=77, dropout_p=p)
+    y.backward(d["dy"].cuda())
+    mask = make_dropout_mask((M, K), p, 77, "cuda").cpu()
+    ye, _ = lora_ref.linear_lora_fwd_fp32(d["x"], wq, d["a"], d["b"], scale, mask, p)
+    _, dae, dbe, _ = lora_ref.linear_lora_bwd_fp32(d["dy"], d["x"], None, d["a"], d["b"], scale, mask, p)
+    for got, exp, name in ((y, ye, "y"), (a.grad, dae, "da"), (b.grad, dbe, "db")):
+        ok, rel, excess = lora_ref.check_close(got.detach().float().cpu(), exp, rtol=1e-2)
+        assert ok, f"{name}: rel {rel:.3e} excess {excess:.3e}"
