@@ -6,6 +6,11 @@ multi-adapter op depending on the ``MultiLoRAManager`` and falls back to the unf
 expressions when ``use_fused=False``.  The layer is duck-typed (``base_layer.weight/.bias``,
 ``lora_A/lora_B[name].weight``, ``lora_dropout[name].p``, ``scaling[name]``, ``training``), so
 any module with those attributes works when peft is not installed.
+
+Extension: a base layer whose weight is stored as NF4 the way bitsandbytes' ``Linear4bit`` holds it
+(a packed ``uint8`` tensor carrying a ``quant_state`` attribute) goes through the QLoRA ops
+(``fused_linear_lora_nf4`` / ``fused_linear_multi_lora(quant_state=...)``), which the reference's
+patch does not cover.
 """
 
 from __future__ import annotations
@@ -35,14 +40,37 @@ def _cast_input(model, x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return cast(x, dtype) if cast is not None else x.to(dtype)
 
 
+def _nf4_state(weight):
+    """The quant state of an NF4-packed base weight, or None for an ordinary 16-bit weight."""
+    qs = getattr(weight, "quant_state", None)
+    if qs is None or weight.dtype != torch.uint8:
+        return None
+    if getattr(qs, "quant_type", "nf4") != "nf4":
+        raise ValueError(f"only NF4 4-bit base weights are supported, got quant_type={qs.quant_type!r}")
+    return qs
+
+
+def _dense_weight(weight, qs):
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
+
+    return weight if qs is None else dequantize_nf4_triton(weight.detach().reshape(-1), qs)
+
+
 def _single(model, x, adapter_key, linear_bias, use_fused):
     lora_a = model.lora_A[adapter_key].weight
     lora_b = model.lora_B[adapter_key].weight
     p = float(getattr(model.lora_dropout[adapter_key], "p", 0.0)) if model.training else 0.0
     scaling = model.scaling[adapter_key]
     x = _cast_input(model, x, lora_a.dtype)
+    weight = model.base_layer.weight
+    qs = _nf4_state(weight)
+    if use_fused and qs is not None:
+        from lorafusion_amd.ops.nf4 import fused_linear_lora_nf4
+
+        return fused_linear_lora_nf4(x, weight.detach().reshape(-1), qs, lora_a, lora_b, scaling, dropout_p=p,
+                                     linear_bias=linear_bias)
     fn = fused_linear_lora if use_fused else torch_ref_linear_lora
-    return fn(x=x, linear_w=model.base_layer.weight, lora_a=lora_a, lora_b=lora_b, alpha=scaling,
+    return fn(x=x, linear_w=_dense_weight(weight, qs), lora_a=lora_a, lora_b=lora_b, alpha=scaling,
               dropout_p=p, linear_bias=linear_bias)
 
 
@@ -71,10 +99,13 @@ def lora_forward(model, x: torch.Tensor, *args, use_fused: bool = True, **kwargs
     lora_a_list = [model.lora_A[f"lora_{i}"].weight for i in info.lora_idx_list]
     lora_b_list = [model.lora_B[f"lora_{i}"].weight for i in info.lora_idx_list]
     x = _cast_input(model, x, lora_a_list[0].dtype)
+    weight = model.base_layer.weight
+    qs = _nf4_state(weight)
     if use_fused:
         result = fused_linear_multi_lora(
             padded_x=x,
-            linear_w=model.base_layer.weight,
+            linear_w=weight if qs is None else weight.detach().reshape(-1),
+            quant_state=qs,
             lora_a_list=lora_a_list,
             lora_b_list=lora_b_list,
             seq_len_list=info.seq_len_list,
@@ -90,7 +121,7 @@ def lora_forward(model, x: torch.Tensor, *args, use_fused: bool = True, **kwargs
     else:
         result = torch_ref_linear_multi_lora(
             padded_x=x,
-            linear_w=model.base_layer.weight,
+            linear_w=_dense_weight(weight, qs),
             lora_a_list=lora_a_list,
             lora_b_list=lora_b_list,
             seq_len_list=info.seq_len_list,
