@@ -222,13 +222,20 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // PFLOP/s at 8192x4096x4096, at a higher clock: the kernel is power limited).  PAIR0 = steps
   // issued before the loop.
   constexpr int PAIR0 = (NSTAGE - 1) & ~1;
+  auto issue_first_tiles = [&]() {
 #pragma unroll
-  for (int t = 0; t < PAIR0; t++)
-    if (t < nk) issue_loads(t, t);
+    for (int t = 0; t < PAIR0; t++)
+      if (t < nk) issue_loads(t, t);
+  };
 
-  // ---- LoRA term seeds the accumulator (overlaps with the first tile's loads)
+  // ---- LoRA term seeds the accumulator.  Its loads go out ahead of the first tile loads: the
+  // term needs two dependent round trips (routing table, then the operands) where the tiles need
+  // one, and behind PAIR0 stages of tile loads in the texture addresser it would start a
+  // microsecond late; the seeding MFMAs then run while the tiles land.
   const int wrow0 = m0 + wm * WM;  // first row of this wave's sub-tile
-  if (p.L != nullptr && wrow0 < p.M) {
+  if (p.L == nullptr || wrow0 >= p.M) {
+    issue_first_tiles();
+  } else {
     const T* __restrict__ L = (const T*)p.L;
     const T* rp = (const T*)seg.ptr[0];
     int rank = seg.rank[0];
@@ -300,22 +307,23 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         }
         rf[j] = v;
       }
-      constexpr int LCH = TM < 4 ? TM : 4;  // L fragments in flight (register budget)
+      lf_u32x4 lf[TM];
 #pragma unroll
-      for (int i0 = 0; i0 < TM; i0 += LCH) {
-        lf_u32x4 lf[LCH];
-#pragma unroll
-        for (int i = 0; i < LCH; i++) {
-          int gm = min(wrow0 + (i0 + i) * 16 + l16, p.M - 1);
-          lf_u32x4 v = {0, 0, 0, 0};
-          if (r0 < p.R) v = *(const lf_u32x4*)(L + (int64_t)gm * p.R + r0);
-          lf[i] = v;
-        }
-#pragma unroll
-        for (int i = 0; i < LCH; i++)
-#pragma unroll
-          for (int j = 0; j < TN; j++) acc[i0 + i][j] = MfmaOp<T>::run(rf[j], lf[i], acc[i0 + i][j]);
+      for (int i = 0; i < TM; i++) {
+        int gm = min(wrow0 + i * 16 + l16, p.M - 1);
+        lf_u32x4 v = {0, 0, 0, 0};
+        if (r0 < p.R) v = *(const lf_u32x4*)(L + (int64_t)gm * p.R + r0);
+        lf[i] = v;
       }
+      if (t == 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue_first_tiles();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = MfmaOp<T>::run(rf[j], lf[i], acc[i][j]);
     }
 #pragma unroll
     for (int i = 0; i < TM; i++) {

@@ -276,27 +276,40 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
 }
 
 // S[row][col] = cast( mult * sum_p part[p][row][col] ), zero for padded rows / rank columns.
+// Sum of `n` fp32x4 partials `stride` floats apart, in index order (deterministic), four loads in flight.
+__device__ __forceinline__ lf_f32x4 sum_parts(const float* __restrict__ p, int64_t stride, int n) {
+  lf_f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  int i = 0;
+  for (; i + 4 <= n; i += 4) {
+    const lf_f32x4 a = *(const lf_f32x4*)(p + (int64_t)i * stride), b = *(const lf_f32x4*)(p + (int64_t)(i + 1) * stride);
+    const lf_f32x4 c = *(const lf_f32x4*)(p + (int64_t)(i + 2) * stride), d = *(const lf_f32x4*)(p + (int64_t)(i + 3) * stride);
+    v += a; v += b; v += c; v += d;
+  }
+  for (; i < n; i++) v += *(const lf_f32x4*)(p + (int64_t)i * stride);
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ lf_u32x2 pack4(lf_f32x4 v) {
+  return lf_u32x2{(uint32_t)Mfma16<T>::cvt(v[0]) | ((uint32_t)Mfma16<T>::cvt(v[1]) << 16),
+                  (uint32_t)Mfma16<T>::cvt(v[2]) | ((uint32_t)Mfma16<T>::cvt(v[3]) << 16)};
+}
+
 template <typename T>
 __device__ __forceinline__ void reduce_rows_body(int bx, const float* __restrict__ part, T* __restrict__ out, int nparts, int M, int R,
                    int mode /*0: times 1/(1-p); 1: times scale*/, const LfSegTable seg) {
+  // four consecutive columns per thread (R and every rank are multiples of 8): 16-byte loads
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
-  const int64_t idx = (int64_t)bx * 256 + threadIdx.x;
+  const int64_t idx = ((int64_t)bx * 256 + threadIdx.x) * 4;
   if (idx >= (int64_t)Mrows * R) return;
   const int row = (int)(idx / R), col = (int)(idx % R);
   const int blk = row / ROWS;
   const BlockInfo bi = block_info(seg, blk, M);
-  float v = 0.f;
+  lf_f32x4 v = {0.f, 0.f, 0.f, 0.f};
   if (row - blk * ROWS < bi.valid && col < bi.rank) {
-    for (int p = 0; p < nparts; p++) v += part[(int64_t)p * Mrows * R + idx];
+    v = sum_parts(part + idx, (int64_t)Mrows * R, nparts);
     v *= (mode == 0) ? (bi.p > 0.f ? 1.f / (1.f - bi.p) : 1.f) : bi.scale;
   }
-  ((uint16_t*)out)[idx] = Mfma16<T>::cvt(v);
-}
-
-template <typename T>
-__global__ void __launch_bounds__(256)
-reduce_rows_kernel(const float* __restrict__ part, T* __restrict__ out, int nparts, int M, int R, int mode, const LfSegTable seg) {
-  reduce_rows_body<T>((int)blockIdx.x, part, out, nparts, M, R, mode, seg);
+  *(lf_u32x2*)((uint16_t*)out + idx) = pack4<T>(v);
 }
 
 // ------------------------------------------------------------------------------- dys_dyb
@@ -444,7 +457,7 @@ template <typename T>
 __device__ __forceinline__ void reduce_segments_body(int bx, int s, const float* __restrict__ part, int rows, int R, int transposed, int mult_mode, int M,
                        int group, int max_chunks, const LfSegTable seg) {
   const int rank = seg.rank[s];
-  const int64_t idx = (int64_t)bx * 256 + threadIdx.x;  // index into the output [rows, rank] or [rank, rows]
+  const int64_t idx = ((int64_t)bx * 256 + threadIdx.x) * 4;  // four consecutive outputs of [rows, rank] or [rank, rows]
   if (idx >= (int64_t)rows * rank) return;
   int b0, b1;
   segment_blocks(seg, s, M, b0, b1);
@@ -455,18 +468,16 @@ __device__ __forceinline__ void reduce_segments_body(int bx, int s, const float*
     mult = mult_mode == 0 ? (seg.block_scale ? seg.block_scale[b0] : 1.f)
                           : ((seg.block_p && seg.block_p[b0] > 0.f) ? 1.f / (1.f - seg.block_p[b0]) : 1.f);
   }
-  float v = 0.f;
+  lf_f32x4 v;
   if (!transposed) {
     const int n = (int)(idx / rank), r = (int)(idx % rank);
-    const int64_t pidx = (int64_t)n * R + r;
-    for (int b = b0; b < b1; b++) v += part[(int64_t)b * rows * R + pidx];
+    v = sum_parts(part + (int64_t)b0 * rows * R + (int64_t)n * R + r, (int64_t)rows * R, b1 - b0);
   } else {
     const int r = (int)(idx / rows), k = (int)(idx % rows);
-    const int64_t pidx = (int64_t)r * rows + k;
     const int nch = (b1 - b0 + group - 1) / group;
-    for (int ch = 0; ch < nch; ch++) v += part[((int64_t)s * max_chunks + ch) * R * rows + pidx];
+    v = sum_parts(part + (int64_t)s * max_chunks * R * rows + (int64_t)r * rows + k, (int64_t)R * rows, nch);
   }
-  ((uint16_t*)seg.out[s])[idx] = Mfma16<T>::cvt(v * mult);
+  *(lf_u32x2*)((uint16_t*)seg.out[s] + idx) = pack4<T>(v * mult);
 }
 
 template <typename T>
@@ -700,7 +711,7 @@ static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M
   int maxrank = 0;
   for (int s = 0; s < nseg; s++) maxrank = seg.rank[s] > maxrank ? seg.rank[s] : maxrank;
   const int64_t nout = (int64_t)N * maxrank;
-  const int nb_rows = (int)((n + 255) / 256), nb_seg = (int)((nout + 255) / 256);
+  const int nb_rows = (int)((n + 1023) / 1024), nb_seg = (int)((nout + 1023) / 1024);  // four outputs per thread
   hipLaunchKernelGGL((reduce_ds_db_kernel<T>), dim3((unsigned)(nb_rows + nb_seg * nseg)), dim3(256), 0, st, (const float*)ds_part,
                      (T*)dS, split, M, R, nb_rows, (const float*)db_part, N, nb_seg, seg);
   return lf_check_launch();
@@ -778,7 +789,7 @@ static int da_impl(const void* X, const uint8_t* mask, const void* dS, void* ws,
   int maxrank = 0;
   for (int s = 0; s < nseg; s++) maxrank = seg.rank[s] > maxrank ? seg.rank[s] : maxrank;
   const int64_t nout = (int64_t)K * maxrank;
-  hipLaunchKernelGGL((reduce_segments_kernel<T>), dim3((unsigned)((nout + 255) / 256), nseg), dim3(256), 0, st, (const float*)part, K, R, 1, 1, M, group, max_chunks, seg);
+  hipLaunchKernelGGL((reduce_segments_kernel<T>), dim3((unsigned)((nout + 1023) / 1024), nseg), dim3(256), 0, st, (const float*)part, K, R, 1, 1, M, group, max_chunks, seg);
   return lf_check_launch();
 }
 
