@@ -201,6 +201,34 @@ def main():
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
     value = step_flops(TOKENS) / (ms * 1e-3) / 1e12
 
+    # ---- the same forward + backward captured once as a HIP graph and replayed (what a training loop
+    # that captures its step gets: no host launch work, shorter gaps between the kernels)
+    routing_g = hip_ops.MultiRouting(info.padded_seq_len_list, [RANK] * 4, info.block_to_lookup_table,
+                                     info.block_to_alpha, info.block_to_dropout_p)
+    xg, ag, bg = x.detach(), [a.detach() for a in a_list], [b.detach() for b in b_list]
+
+    def raw_step():
+        y, s_ = hip_ops.lora_forward(xg, t["w"], ag, bg, routing_g.c, routing_g.R, t["mask"], None)
+        return y, hip_ops.lora_backward(t["dy"], xg, t["w"], ag, bg, s_, routing_g.c, routing_g.R, t["mask"], [RANK] * 4)
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        raw_step()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            graph_out = raw_step()
+    torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms_graph = (time.perf_counter() - t0) * 1e3 / args.steps
+    del graph_out
+
     # ---- per-kernel timings with HIP events (kernel launches only, outputs preallocated by the wrappers)
     routing = hip_ops.MultiRouting(info.padded_seq_len_list, [RANK] * 4, info.block_to_lookup_table,
                                    info.block_to_alpha, info.block_to_dropout_p)
@@ -285,6 +313,8 @@ def main():
             "xa": round(t_xa, 4), "gemm_fwd": round(t_fwd, 4), "dys_dyb": round(t_dys, 4), "da": round(t_da, 4),
             "gemm_bwd": round(t_bwd, 4), "seeded_mask": round(t_mask, 4), "fwd_seeded_xa_plus_gemm": round(t_fwd_seeded, 4), "plain_gemm_nt": round(t_plain_nt, 4), "plain_gemm_nn": round(t_plain_nn, 4),
         },
+        "hipgraph_replay": {"ms_per_step": round(ms_graph, 4),
+                            "TFLOP/s": round(step_flops(TOKENS) / (ms_graph * 1e-3) / 1e12, 2)},
         "lora_overhead_vs_plain_gemms": round((t_xa + t_fwd + t_dys + t_da + t_bwd) / (t_plain_nt + t_plain_nn) - 1.0, 4),
         "nf4_dequant": {
             "GB/s": round(nf4_gbs, 1), "frac_of_hbm_peak": round(nf4_gbs / HBM_PEAK_GBS, 4),

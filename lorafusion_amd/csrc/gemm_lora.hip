@@ -605,11 +605,8 @@ int launch_cfg(LfGemmParams p, const LfSegTable& seg, hipStream_t st) {
   p.grid_m = (p.M + BM - 1) / BM;
   p.grid_n = (p.N + BN - 1) / BN;
   auto kern = gemm_lora_kernel<T, BM, BN, WM, WN, NN, NSTAGE>;
-  static bool attr_set = false;  // idempotent; a race only repeats the same call
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess) return LF_ELAUNCH;
-    attr_set = true;
-  }
+  static bool lds_ok[64] = {};
+  if (!lf_allow_lds(kern, SMEM, lds_ok)) return LF_ELAUNCH;
   hipLaunchKernelGGL(kern, dim3(p.grid_m * p.grid_n), dim3(NTHREADS), SMEM, st, p, seg);
   return lf_check_launch();
 }

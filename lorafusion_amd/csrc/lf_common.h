@@ -54,6 +54,19 @@ struct LfGemmParams {
 // launchers (one per translation unit)
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st);
 
+// Raise a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's copy of
+// the function; the flag array is per kernel instantiation, a race only repeats the same call).
+template <typename Kern>
+static inline bool lf_allow_lds(Kern kern, int bytes, bool (&done)[64]) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+  if (!done[dev]) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+    done[dev] = true;
+  }
+  return true;
+}
+
 static inline int lf_check_launch() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? LF_OK : LF_ELAUNCH;

@@ -684,7 +684,8 @@ static int dys_launch(const void* dY, const void* S, float* ds_part, float* db_p
   constexpr int RP = RT * 32 + 32;
   const int smem = dys_smem(RT);
   static_assert(RP == RT * 32 + 32, "");
-  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return LF_ELAUNCH;
+  static bool lds_ok[64] = {};
+  if (!lf_allow_lds(kern, smem, lds_ok)) return LF_ELAUNCH;
   hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, tiles_per_wg, seg);
   return lf_check_launch();
 }
@@ -766,7 +767,8 @@ static int da_launch(const void* X, const uint8_t* mask, const void* dS, float* 
   auto kern = lora_da_kernel<T, RT>;
   constexpr int RP = RT * 32 + 32;
   const int smem = 2 * TILE_BYTES + 2 * ROWS * RP;
-  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return LF_ELAUNCH;
+  static bool lds_ok[64] = {};
+  if (!lf_allow_lds(kern, smem, lds_ok)) return LF_ELAUNCH;
   hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)X, mask, (const T*)dS, part, M, K, R, group, max_chunks, seg);
   return lf_check_launch();
 }
