@@ -36,6 +36,8 @@ def test_routing_struct_layout_matches_header():
     assert ctypes.sizeof(_lib.Routing) == 16 + 24 + 8 + 2 * 4 * _lib.LF_MAX_SEG
     r = _lib.single_routing(16, 2.0, 0.1)
     assert r.n_seg == 1 and r.seg_rank[0] == 16 and abs(r.p - 0.1) < 1e-7
+    # struct lf_nf4_weight: 5 pointers + 2 int32
+    assert ctypes.sizeof(_lib.NF4Weight) == 5 * 8 + 2 * 4
 
 
 def test_argument_validation_without_gpu():
