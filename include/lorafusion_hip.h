@@ -178,9 +178,10 @@ int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const
                     const lf_routing* routing, int dtype, void* stream);
 
 /* Seeded dropout keep-mask (1 = keep), uint8 [M, K], K % 16 == 0.  Stands in for the mask output of
- * seeded_dropout (lorafusion/ops/triton_ops/dropout.py:71-93) and, with `routing` carrying a block
- * table, of blocked_seeded_dropout with one p per 128-row block
- * (lorafusion/ops/triton_ops/blocked_dropout.py:78-135); routing == NULL uses `p` for every row.
+ * seeded_dropout (lorafusion/ops/triton_ops/dropout.py:71-93) and, with `routing` carrying
+ * block_p (n_blocks entries, one per block_size_m rows; the block table itself is not read), of
+ * blocked_seeded_dropout (lorafusion/ops/triton_ops/blocked_dropout.py:78-135); routing == NULL
+ * uses `p` for every row.
  * Philox4x32-10 keyed by `seed`, one 32-bit word per element (element e: counter e/4, word e%4),
  * kept when word >= floor(p * 2^32): a function of (seed, element index) only. */
 int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream);

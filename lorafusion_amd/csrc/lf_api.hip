@@ -246,7 +246,7 @@ int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const
 int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream) {
   const float* block_p = nullptr;
   int bs = 0;
-  if (routing != nullptr && routing->block_table != nullptr) {
+  if (routing != nullptr && (routing->block_table != nullptr || routing->block_p != nullptr)) {
     if (!routing->block_p || routing->block_size_m <= 0) return LF_EINVAL;
     if ((int64_t)routing->n_blocks * routing->block_size_m != M) return LF_ESHAPE;
     block_p = routing->block_p;

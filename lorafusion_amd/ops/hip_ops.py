@@ -172,6 +172,39 @@ def seeded_dropout(x: torch.Tensor, p: float, seed: int, *, store_mask: bool = T
     return out, (mask if store_mask else None)
 
 
+def blocked_seeded_dropout(x: torch.Tensor, block_to_dropout_p: torch.Tensor, block_size_m: int, seed: int | None = None,
+                           *, store_mask: bool = True):
+    """Dropout with one p per ``block_size_m`` rows -- lorafusion/ops/triton_ops/blocked_dropout.py:78-135.
+
+    Returns ``(where(mask, x / (1 - p_block), 0), mask)``; the mask comes from the HIP Philox kernel
+    keyed by ``seed`` (the same bytes ``make_dropout_mask`` gives a packed batch with these p).
+    """
+    if x.ndim != 2:
+        raise ValueError("x must be a 2D tensor")
+    L.require_gpu(x, "x")
+    M, K = x.shape
+    if block_size_m <= 0 or M % block_size_m != 0:
+        raise ValueError(f"x has {M} rows, not a multiple of block_size_m = {block_size_m}.")
+    if K % 16 != 0:
+        raise ValueError(f"the mask kernel needs K % 16 == 0, got K={K}.")
+    nb = M // block_size_m
+    p = block_to_dropout_p.to(device=x.device, dtype=torch.float32).contiguous()
+    if p.numel() != nb:
+        raise ValueError(f"block_to_dropout_p must have {nb} entries, got {p.numel()}.")
+    if seed is None:
+        seed = random.randrange(int(1e6))  # noqa: S311
+    r = L.Routing()
+    r.n_seg, r.block_size_m, r.n_blocks = 1, int(block_size_m), nb
+    r.block_table, r.block_scale, r.block_p = None, None, p.data_ptr()
+    mask = torch.empty((M, K), dtype=torch.bool, device=x.device)
+    with torch.cuda.device(x.device):
+        L.check(L.lib().lf_dropout_mask(L.ptr(mask), M, K, ctypes.c_float(0.0), ctypes.byref(r),
+                                        ctypes.c_uint64(int(seed) & 0xFFFFFFFFFFFFFFFF), L.stream_of(mask)), "lf_dropout_mask")
+    scale = (1.0 / (1.0 - p)).repeat_interleave(block_size_m).unsqueeze(1)
+    out = torch.where(mask, (x.float() * scale).to(x.dtype), torch.zeros((), dtype=x.dtype, device=x.device))
+    return out, (mask if store_mask else None)
+
+
 def fused_dropout_matmul(x: torch.Tensor, a: torch.Tensor, dropout_p: float, seed: int | None = None, *,
                          store_mask: bool = True, store_masked_scaled_x: bool = False,
                          dropout_mask: torch.Tensor | None = None):

@@ -154,3 +154,34 @@ def test_torch_ref_path_matches_oracle_on_cpu():
     yme, _ = lora_ref.linear_multi_lora_fwd_fp32(m["x"], m["w"], m["a_list"], m["b_list"], seq, m["padded"],
                                                  [1.0, 2.0], [0.0, 0.0])
     assert torch.allclose(ym[0], yme, atol=1e-5)
+
+
+def test_reference_module_and_function_names_resolve():
+    """A user of the reference swaps the package prefix: every module of lorafusion.ops on the hot path
+    and its public entry points exist under lorafusion_amd.ops with the same names."""
+    import importlib
+
+    names = {
+        "lora_v1": ["fused_linear_lora", "FusedLinearLoRA"],
+        "multi_lora": ["fused_linear_multi_lora", "FusedLinearMultiLoRA", "prepare_multi_lora_batch_info",
+                       "MultiLoRABatchInfo", "MultiLoRAManager", "init_multi_lora_manager", "get_multi_lora_manager"],
+        "lora_torch_ref": ["torch_ref_linear_lora", "torch_ref_linear_multi_lora"],
+        "triton_ops.dropout": ["seeded_dropout"],
+        "triton_ops.blocked_dropout": ["blocked_seeded_dropout"],
+        "triton_ops.fused_dropout_matmul": ["fused_dropout_matmul"],
+        "triton_ops.fused_lora_xw_sb": ["fused_lora_xw_sb"],
+        "triton_ops.fused_lora_xw_sb_tma": ["fused_lora_xw_sb_tma"],
+        "triton_ops.fused_lora_dys_dyb": ["fused_lora_dys_dyb"],
+        "triton_ops.fused_lora_dyw_dsa": ["fused_lora_dyw_dsa"],
+        "triton_ops.fused_lora_dyw_dsa_tma": ["fused_lora_dyw_dsa_tma"],
+        "triton_ops.fused_multi_lora_xw_sb": ["fused_multi_lora_xw_sb", "construct_s_and_b_ptrs_list"],
+        "triton_ops.fused_multi_lora_dys_dyb": ["fused_multi_lora_dys_dyb", "construct_s_and_b_ptrs_list"],
+        "triton_ops.fused_multi_lora_dyw_dsa": ["fused_multi_lora_dyw_dsa", "construct_ds_and_a_ptrs_list"],
+        "triton_ops.dequantize_nf4": ["dequantize_nf4_triton", "NF4_LUT"],
+        "triton_ops.config": ["get_lora_kernel_config", "LoRATritonConfig"],
+    }
+    for mod, syms in names.items():
+        m = importlib.import_module("lorafusion_amd.ops." + mod)
+        for s in syms:
+            assert hasattr(m, s), f"lorafusion_amd.ops.{mod}.{s} is missing"
+    assert importlib.import_module("lorafusion_amd.patch.patch_lora").apply_lora
