@@ -46,6 +46,9 @@ constexpr int BK = 32;
 #ifndef LF_NSTAGE
 #define LF_NSTAGE 5
 #endif
+#ifndef LF_MEMPHASE_LOADS
+#define LF_MEMPHASE_LOADS 1
+#endif
 
 template <typename T> struct MfmaOp;
 template <> struct MfmaOp<__bf16> {
@@ -484,12 +487,15 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   //   phase 2k+1 : group 0 computes tile k     | group 1 reads tile k
   // Tile k is read in phases 2k and 2k+1; every wave waits for its own share of it in a memory
   // phase that ends no later than phase 2k-1, so the barrier closing that phase publishes the tile.
-  // Tile loads are issued from the compute phase of every odd step kt, spread between the MFMAs
-  // (the texture addresser takes 16 cycles per 64-lane 16-byte load: a burst of loads at the head
-  // of a memory phase would hold the LDS reads of four waves back behind it, and behind the reads
-  // they measured no faster): the pair (kt+3, kt+4) goes into the stages of steps kt-2 and kt-1
-  // (last read in phase 2kt-1).  At the end of the memory phase of an odd step the pair
-  // (kt+1, kt+2), issued two steps earlier, must have landed.
+  // Tile loads are issued in every odd step kt: the pair (kt+3, kt+4) goes into the stages of steps
+  // kt-2 and kt-1 (last read in phase 2kt-1).  The texture addresser takes 16 cycles per 64-lane
+  // 16-byte load, and a wave whose load has to wait for it cannot issue the MFMAs behind it: with
+  // all loads of a step between the MFMAs of the compute phase that phase grows from 570 to 715
+  // cycles.  The memory phase has some slack behind its fragment reads, enough for one of the four
+  // loads of a step (LF_MEMPHASE_LOADS; measured per value at 8192x4096x4096: 0: 196 us, 1: 190,
+  // 2: 192, 3: 194, 4: 196); the others stay in the compute phase, spread between the MFMAs.  At
+  // the end of the memory phase of an odd step the pair (kt+1, kt+2), issued two steps earlier,
+  // must have landed.
   const int grp = wave >= NWAVES / 2 ? 1 : 0;
   auto phase_barrier = [&]() {
     __builtin_amdgcn_sched_barrier(0);
@@ -499,27 +505,28 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   int stage = 0, kt = 0;
   static_assert(NSTAGE == 5, "the anti-phase loop is written for a ring of five stages");
   constexpr int NM = TM * TN;
+  constexpr int ML = LF_MEMPHASE_LOADS < NL ? LF_MEMPHASE_LOADS : NL;  // loads of a step issued from the memory phase
   auto compute_phase = [&](auto LOADC) {
     __builtin_amdgcn_s_setprio(1);
     if constexpr (LOADC.value) {
       const int s3 = stage + 3 >= NSTAGE ? stage + 3 - NSTAGE : stage + 3;
       const int s4 = stage + 4 >= NSTAGE ? stage + 4 - NSTAGE : stage + 4;
 #pragma unroll
-      for (int i = 0; i < NL; i++) {
+      for (int i = ML; i < NL; i++) {
         issue_load_one(s3, kt + 3, i);
         issue_load_one(s4, kt + 4, i);
       }
     }
     join_b(0);
     mfma_range(0, 0, NM);
-    if constexpr (LOADC.value) {
-      constexpr int PER = NM / (2 * NL);
+    if constexpr (LOADC.value && NL > ML) {
+      constexpr int NLC = NL - ML > 0 ? NL - ML : 1, PER = NM / (2 * NLC);
 #pragma unroll
-      for (int r = 0; r < 2 * NL; r++) {
+      for (int r = 0; r < 2 * NLC; r++) {
         __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * 2 * NL, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * 2 * NLC, 0);
     }
     __builtin_amdgcn_s_setprio(0);
     phase_barrier();
@@ -535,6 +542,17 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     // odd step: the pair (kt+1, kt+2) must have landed; issue the pair (kt+3, kt+4)
     read_frags(0, stage);
     wait_loads(Steps0{});
+    if constexpr (LOAD.value && ML > 0) {
+      __builtin_amdgcn_sched_barrier(0);
+      const int s3 = stage + 3 >= NSTAGE ? stage + 3 - NSTAGE : stage + 3;
+      const int s4 = stage + 4 >= NSTAGE ? stage + 4 - NSTAGE : stage + 4;
+#pragma unroll
+      for (int i = 0; i < ML; i++) {
+        issue_load_one(s3, kt + 3, i);
+        issue_load_one(s4, kt + 4, i);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
     __builtin_amdgcn_s_waitcnt(0xc07f);
     phase_barrier();
     compute_phase(LOAD);
