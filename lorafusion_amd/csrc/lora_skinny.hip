@@ -725,6 +725,8 @@ int lf_launch_dys_dyb(const void* dY, const void* S, void* dS, void* ws, size_t 
   if (seg.table && seg.block_size_m != ROWS) return LF_ESHAPE;
   const int nseg = seg.table ? seg.n_seg : 1;
   for (int s = 0; s < nseg; s++) if (!seg.out[s] || !seg.ptr[s] || seg.rank[s] % 8 != 0 || seg.rank[s] > R) return LF_EINVAL;
+  for (int s = 0; s < nseg; s++) if (((uintptr_t)seg.out[s] & 7) != 0) return LF_ESHAPE;  // 8-byte stores of dB
+  if (((uintptr_t)dS & 7) != 0) return LF_ESHAPE;
   if (!ws || ws_bytes < lf_dys_dyb_workspace(M, N, R, seg)) return LF_EWORKSPACE;
   if (dtype == LF_BF16) return dys_dyb_impl<__bf16>(dY, S, dS, ws, M, N, R, seg, st);
   if (dtype == LF_F16) return dys_dyb_impl<_Float16>(dY, S, dS, ws, M, N, R, seg, st);
@@ -802,6 +804,7 @@ int lf_launch_da(const void* X, const uint8_t* mask, const void* dS, void* ws, s
   if (seg.table && seg.block_size_m != ROWS) return LF_ESHAPE;
   const int nseg = seg.table ? seg.n_seg : 1;
   for (int s = 0; s < nseg; s++) if (!seg.out[s] || seg.rank[s] % 8 != 0 || seg.rank[s] > R) return LF_EINVAL;
+  for (int s = 0; s < nseg; s++) if (((uintptr_t)seg.out[s] & 7) != 0) return LF_ESHAPE;  // 8-byte stores of dA
   if (!ws || ws_bytes < lf_da_workspace(M, K, R, seg)) return LF_EWORKSPACE;
   if (dtype == LF_BF16) return da_impl<__bf16>(X, mask, dS, ws, M, K, R, seg, st);
   if (dtype == LF_F16) return da_impl<_Float16>(X, mask, dS, ws, M, K, R, seg, st);
