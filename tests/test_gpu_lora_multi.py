@@ -83,7 +83,7 @@ def test_multi_bias_and_bf16_tables():
 
 
 def test_multi_config1_shape():
-    """BASELINE configs[1]: 4 adapters r=16, scales {16,32,32,64}/16, p {0,.05,.1,.1}, lognormal
+    """The headline multi-adapter configuration: 4 adapters r=16, scales {16,32,32,64}/16, p {0,.05,.1,.1}, lognormal
     segments packed to 8192 tokens, K=N=4096."""
     seq = lognormal_segments(8192, 4, seed=0)
     assert sum(seq) == 8192

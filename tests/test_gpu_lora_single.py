@@ -73,7 +73,7 @@ def test_single_fp16():
 
 
 def test_single_config0_full_size():
-    """BASELINE configs[0]: M=2048, K=N=4096, r=16, s=2, p=0.1."""
+    """The single-adapter configuration the reference runs on CPU too: M=2048, K=N=4096, r=16, s=2, p=0.1."""
     _run_case(2048, 4096, 4096, 16, 0.1, 2.0)
 
 

@@ -74,7 +74,7 @@ def test_dequant_fp16_output():
 
 
 def test_dequant_config2_shape_and_roundtrip():
-    """BASELINE configs[2] weight: [14336, 4096], blocksize 64, double quantised.  Bit-exact vs the
+    """The NF4 linear configuration's weight: [14336, 4096], blocksize 64, double quantised.  Bit-exact vs the
     oracle, and the size-independent property |dequant(quant(w)) - w| <= half the widest code gap * absmax."""
     from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
 
