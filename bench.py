@@ -94,6 +94,31 @@ def event_time_ms(fn, reps: int) -> float:
     return e0.elapsed_time(e1) / reps
 
 
+def graph_time_ms(fn, reps: int, inner: int = 10) -> float:
+    """Average duration of `fn`'s launches with no host work between them: `inner` calls captured once
+    as a HIP graph, replayed between two HIP events.  For kernels of a few tens of microseconds, whose
+    Python wrapper takes longer than the kernel runs (the GPU would otherwise wait for the host)."""
+    side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        fn()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            keep = [fn() for _ in range(inner)]
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    n = max(1, reps // inner)
+    st = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(st)
+    for _ in range(n):
+        graph.replay()
+    e1.record(st)
+    torch.cuda.synchronize()
+    del keep
+    return e0.elapsed_time(e1) / (n * inner)
+
+
 def cpu_baseline(seq, budget_s: float = 15.0):
     """Oracle (bf16 op-by-op, autograd backward) on the host cores: the whole 8192-token batch when one
     run takes under a second (it does on the GPU box's host), else the first 256 tokens of every
@@ -229,7 +254,8 @@ def main():
     ms_graph = (time.perf_counter() - t0) * 1e3 / args.steps
     del graph_out
 
-    # ---- per-kernel timings with HIP events (kernel launches only, outputs preallocated by the wrappers)
+    # ---- per-kernel timings with HIP events: the GEMMs as plain back-to-back launches, the short rank-r,
+    # mask and dequant kernels replayed from a graph (their wrappers take longer than they run)
     routing = hip_ops.MultiRouting(info.padded_seq_len_list, [RANK] * 4, info.block_to_lookup_table,
                                    info.block_to_alpha, info.block_to_dropout_p)
     xd, wd, dyd, mask = x.detach(), t["w"], t["dy"], t["mask"]
@@ -243,10 +269,10 @@ def main():
     t_bwd = event_time_ms(lambda: hip_ops.fused_multi_lora_dyw_dsa(dyd, wd, ds, ad, routing, mask), reps)
     t_plain_nt = event_time_ms(lambda: hip_ops.gemm(xd, wd, trans_b=True), reps)
     t_plain_nn = event_time_ms(lambda: hip_ops.gemm(dyd, wd, trans_b=False), reps)
-    t_xa = event_time_ms(lambda: hip_ops.fused_multi_lora_xa(xd, ad, routing, mask), reps)
-    t_dys = event_time_ms(lambda: hip_ops.fused_multi_lora_dys_dyb(dyd, s, bd, routing), reps)
-    t_da = event_time_ms(lambda: hip_ops.fused_multi_lora_da(xd, ds, routing, mask), reps)
-    t_mask = event_time_ms(lambda: hip_ops.make_dropout_mask(xd.shape, None, 1234, dev, routing=routing), reps)
+    t_xa = graph_time_ms(lambda: hip_ops.fused_multi_lora_xa(xd, ad, routing, mask), reps)
+    t_dys = graph_time_ms(lambda: hip_ops.fused_multi_lora_dys_dyb(dyd, s, bd, routing), reps)
+    t_da = graph_time_ms(lambda: hip_ops.fused_multi_lora_da(xd, ds, routing, mask), reps)
+    t_mask = graph_time_ms(lambda: hip_ops.make_dropout_mask(xd.shape, None, 1234, dev, routing=routing), reps)
     t_fwd_seeded = event_time_ms(lambda: hip_ops.lora_forward_seeded(xd, wd, ad, bd, routing.c, routing.R, 1234, None), reps)
     # ---- dominant kernel: the 256x256-tile MFMA GEMM of the dX path.  The library runs rows
     # [0, 8192) of the 8448 in whole rounds of that tile and the last 256 rows as a second, small
@@ -274,7 +300,8 @@ def main():
     wq = torch.randn(14336, 4096, device=dev) * 0.02
     packed, qs = quantize_nf4(wq)
     out = torch.empty(14336 * 4096, dtype=torch.bfloat16, device=dev)
-    t_nf4 = event_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), reps)
+    t_nf4_op = event_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), reps)   # as called from Python
+    t_nf4 = graph_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), 5 * reps)   # the kernel alone
     n = 14336 * 4096
     nf4_bytes = n / 2 + n / 64 + 4 * n / 16384 + 1028 + 2 * n
     nf4_gbs = nf4_bytes / (t_nf4 * 1e-3) / 1e9
@@ -318,7 +345,8 @@ def main():
         "lora_overhead_vs_plain_gemms": round((t_xa + t_fwd + t_dys + t_da + t_bwd) / (t_plain_nt + t_plain_nn) - 1.0, 4),
         "nf4_dequant": {
             "GB/s": round(nf4_gbs, 1), "frac_of_hbm_peak": round(nf4_gbs / HBM_PEAK_GBS, 4),
-            "launch_ms": round(t_nf4, 4), "bytes_per_launch": nf4_bytes, "shape": [14336, 4096],
+            "launch_ms": round(t_nf4, 4), "op_ms_from_python": round(t_nf4_op, 4), "bytes_per_launch": nf4_bytes,
+            "shape": [14336, 4096],
         },
     }
     if not args.no_cpu_baseline:
