@@ -460,7 +460,9 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     };
     using T_ = integral_constant<bool, true>;
     using F_ = integral_constant<bool, false>;
-    if (nk > 2) wait_loads(integral_constant<int, PAIR0 - 2>{});  // tiles 0 and 1
+    // tiles 0 and 1 must have landed.  PAIR0 steps are in flight only when the K loop has that many;
+    // a shorter loop has fewer loads outstanding than the count allows, so it waits for all of them
+    if (nk >= PAIR0) wait_loads(integral_constant<int, PAIR0 - 2>{});
     else wait_loads(Steps0{});
     __syncthreads();
     read_frags(0, 0);
