@@ -99,7 +99,7 @@ nf4_dequant_kernel(const uint32_t* __restrict__ packed, const void* __restrict__
         const float lo = lut[byte & 15u] * am[s];
         o[b] = pack2<T>(hi, lo);
       }
-      __builtin_nontemporal_store(o, out + i);
+      out[i] = o;  // a plain store: the non-temporal kind fills 117 MB at 5.6 TB/s, this one at 6.45
     }
   }
 }
