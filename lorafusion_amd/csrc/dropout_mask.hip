@@ -24,7 +24,7 @@ dropout_mask_kernel(uint8_t* __restrict__ mask, int64_t n16, int K, uint32_t thr
   lf_u32x4 o;
 #pragma unroll
   for (int c = 0; c < 4; c++) o[c] = lf_keep4((uint64_t)(e0 >> 2) + c, thr, seed_lo, seed_hi);
-  __builtin_nontemporal_store(o, (lf_u32x4*)(mask + e0));
+  *(lf_u32x4*)(mask + e0) = o;
 }
 
 }  // namespace

@@ -113,8 +113,8 @@ __device__ __forceinline__ void tile_load(TileRegs& r, const T* __restrict__ src
   for (int i = 0; i < 4; i++) {
     const int row = min(row0 + i * 32 + (tid >> 3), max_row - 1);
     const int64_t off = (int64_t)row * ld + col0 + srcg * 8;
-    r.x[i] = __builtin_nontemporal_load((const lf_u32x4*)(src + off));
-    if (use_mask) r.m[i] = __builtin_nontemporal_load((const lf_u32x2*)(mask + off));
+    r.x[i] = *((const lf_u32x4*)(src + off));
+    if (use_mask) r.m[i] = *((const lf_u32x2*)(mask + off));
   }
 }
 
@@ -209,9 +209,9 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
       if (s < nsteps) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-          xv[b][u][i] = __builtin_nontemporal_load((const lf_u32x4*)(xrow[i] + s * 64));
+          xv[b][u][i] = *((const lf_u32x4*)(xrow[i] + s * 64));
           if constexpr (!GEN) {
-            if (use_mask) mv[b][u][i] = __builtin_nontemporal_load((const lf_u32x2*)(mrow[i] + s * 64));
+            if (use_mask) mv[b][u][i] = *((const lf_u32x2*)(mrow[i] + s * 64));
           }
 #pragma unroll
           for (int c = 0; c < RT; c++) {
@@ -233,7 +233,7 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
           if constexpr (GEN) {
             const uint64_t ctr = (uint64_t)(erow[i] + s * 64) >> 2;
             mv[b][u][i] = lf_u32x2{lf_keep4(ctr, thr, seed_lo, seed_hi), lf_keep4(ctr + 1, thr, seed_lo, seed_hi)};
-            if (row_real[i]) __builtin_nontemporal_store(mv[b][u][i], (lf_u32x2*)(mask_out + erow[i] + s * 64));
+            if (row_real[i]) *(lf_u32x2*)(mask_out + erow[i] + s * 64) = mv[b][u][i];
           }
           *(lf_u32x4*)(patch + wr_off[i]) = use_mask ? apply_mask8(xv[b][u][i], mv[b][u][i]) : xv[b][u][i];
 #pragma unroll

@@ -58,7 +58,7 @@ nf4_dequant_kernel(const uint32_t* __restrict__ packed, const void* __restrict__
 #pragma unroll
   for (int s = 0; s < NF4_STEPS; s++) {
     const int64_t i = base + (int64_t)s * NF4_THREADS;
-    w[s] = i < n_words ? __builtin_nontemporal_load(packed + i) : 0u;
+        w[s] = i < n_words ? packed[i] : 0u;
   }
   if (NESTED) __syncthreads();  // lut2 is complete
   // One scale per quantisation block of the span, computed once (a lane-per-dword lookup would
