@@ -182,8 +182,9 @@ int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const
  * block_p (n_blocks entries, one per block_size_m rows; the block table itself is not read), of
  * blocked_seeded_dropout (lorafusion/ops/triton_ops/blocked_dropout.py:78-135); routing == NULL
  * uses `p` for every row.
- * Philox4x32-10 keyed by `seed`, one 32-bit word per element (element e: counter e/4, word e%4),
- * kept when word >= floor(p * 2^32): a function of (seed, element index) only. */
+ * Philox4x32-10 keyed by `seed`, sixteen bits per element (element e: counter e/8, 16-bit draw e%8 of
+ * the 128 output bits, low half of a word first), kept when draw >= floor(p * 2^16): a function of
+ * (seed, element index) only. */
 int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream);
 
 #ifdef __cplusplus

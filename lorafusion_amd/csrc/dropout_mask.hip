@@ -4,8 +4,8 @@
 // is never materialised here: the rank-r kernels rebuild it from X and this mask.
 //
 // Generator: Philox4x32 with 10 rounds (Salmon et al., SC'11), key = the 64-bit seed, counter =
-// (element index / 4, 0, 0); output word (element index % 4) belongs to the element, which is kept
-// when word >= floor(p * 2^32).  The stream is a function of (seed, element index) only, so it is
+// (element index / 8, 0, 0); the 16-bit draw (element index % 8) of the 128 output bits belongs to
+// the element, which is kept when draw >= floor(p * 2^16).  The stream is a function of (seed, element index) only, so it is
 // independent of the launch shape; it is not the reference's stream (Triton's rand4x with 7
 // rounds and a float compare).  HBM bound: one byte written per element.
 #include "lf_common.h"
@@ -13,7 +13,7 @@
 
 namespace {
 
-// Each thread writes 16 consecutive mask bytes (four Philox calls); K % 16 == 0 keeps them in one row.
+// Each thread writes 16 consecutive mask bytes (two Philox calls); K % 16 == 0 keeps them in one row.
 __global__ void __launch_bounds__(256)
 dropout_mask_kernel(uint8_t* __restrict__ mask, int64_t n16, int K, uint32_t thr, const float* __restrict__ block_p,
                     int block_size_m, uint32_t seed_lo, uint32_t seed_hi) {
@@ -23,7 +23,12 @@ dropout_mask_kernel(uint8_t* __restrict__ mask, int64_t n16, int K, uint32_t thr
   if (block_p != nullptr) thr = lf_keep_threshold(block_p[(e0 / K) / block_size_m]);
   lf_u32x4 o;
 #pragma unroll
-  for (int c = 0; c < 4; c++) o[c] = lf_keep4((uint64_t)(e0 >> 2) + c, thr, seed_lo, seed_hi);
+  for (int c = 0; c < 2; c++) {
+    uint32_t lo, hi;
+    lf_keep8((uint64_t)(e0 >> 3) + c, thr, seed_lo, seed_hi, lo, hi);
+    o[2 * c] = lo;
+    o[2 * c + 1] = hi;
+  }
   *(lf_u32x4*)(mask + e0) = o;
 }
 

@@ -231,8 +231,9 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
 #pragma unroll
         for (int i = 0; i < 2; i++) {
           if constexpr (GEN) {
-            const uint64_t ctr = (uint64_t)(erow[i] + s * 64) >> 2;
-            mv[b][u][i] = lf_u32x2{lf_keep4(ctr, thr, seed_lo, seed_hi), lf_keep4(ctr + 1, thr, seed_lo, seed_hi)};
+            uint32_t klo, khi;
+            lf_keep8((uint64_t)(erow[i] + s * 64) >> 3, thr, seed_lo, seed_hi, klo, khi);
+            mv[b][u][i] = lf_u32x2{klo, khi};
             if (row_real[i]) *(lf_u32x2*)(mask_out + erow[i] + s * 64) = mv[b][u][i];
           }
           *(lf_u32x4*)(patch + wr_off[i]) = use_mask ? apply_mask8(xv[b][u][i], mv[b][u][i]) : xv[b][u][i];

@@ -1,7 +1,10 @@
 // Philox4x32-10 (Salmon et al., SC'11) and the keep rule of the seeded dropout mask, shared by the
 // standalone mask kernel and the rank-r forward pass that draws its mask on the fly.
-// Element e of the [M, K] mask uses counter (e / 4, 0, 0), key = the 64-bit seed, output word
-// e % 4, and is kept when word >= floor(p * 2^32).
+// Element e of the [M, K] mask uses counter (e / 8, 0, 0), key = the 64-bit seed, and the 16-bit
+// draw e % 8 of the call's 128 output bits (word (e % 8) / 2, low half for even e, high half for odd
+// e); it is kept when draw >= floor(p * 2^16).  Sixteen bits per element resolve p to 1.5e-5 and halve
+// the integer multiplies per element, which are what bounds the generation (20 quarter-rate 32x32
+// multiplies per call).
 #pragma once
 #include <stdint.h>
 
@@ -19,13 +22,17 @@ __device__ __forceinline__ void lf_philox4x32_10(uint32_t c0, uint32_t c1, uint3
 }
 
 __host__ __device__ __forceinline__ uint32_t lf_keep_threshold(float p) {
-  const double s = (double)p * 4294967296.0;
-  return s >= 4294967295.0 ? 0xffffffffu : (uint32_t)s;
+  const double s = (double)p * 65536.0;
+  return s >= 65535.0 ? 65535u : (uint32_t)s;
 }
 
-// Keep bytes (0/1) of the four elements 4*ctr .. 4*ctr+3, packed into one dword in memory order.
-__device__ __forceinline__ uint32_t lf_keep4(uint64_t ctr, uint32_t thr, uint32_t seed_lo, uint32_t seed_hi) {
+// Keep bytes (0/1) of the eight elements 8*ctr .. 8*ctr+7 in memory order: `lo` holds the first four.
+__device__ __forceinline__ void lf_keep8(uint64_t ctr, uint32_t thr, uint32_t seed_lo, uint32_t seed_hi, uint32_t& lo,
+                                         uint32_t& hi) {
   uint32_t w[4];
   lf_philox4x32_10((uint32_t)ctr, (uint32_t)(ctr >> 32), 0u, 0u, seed_lo, seed_hi, w);
-  return (w[0] >= thr ? 1u : 0u) | (w[1] >= thr ? 0x100u : 0u) | (w[2] >= thr ? 0x10000u : 0u) | (w[3] >= thr ? 0x1000000u : 0u);
+  lo = ((w[0] & 0xffffu) >= thr ? 1u : 0u) | ((w[0] >> 16) >= thr ? 0x100u : 0u) | ((w[1] & 0xffffu) >= thr ? 0x10000u : 0u) |
+       ((w[1] >> 16) >= thr ? 0x1000000u : 0u);
+  hi = ((w[2] & 0xffffu) >= thr ? 1u : 0u) | ((w[2] >> 16) >= thr ? 0x100u : 0u) | ((w[3] & 0xffffu) >= thr ? 0x10000u : 0u) |
+       ((w[3] >> 16) >= thr ? 0x1000000u : 0u);
 }

@@ -2,7 +2,7 @@
  * product).  The reference draws its mask with Triton's rand4x (Philox, 7 rounds, float compare;
  * lorafusion/ops/triton_ops/dropout.py:49-50, blocked_dropout.py:57-60); the build defines its own
  * stream -- Philox4x32 with the standard 10 rounds (Salmon, Moraes, Dror, Shaw: "Parallel random
- * numbers: as easy as 1, 2, 3", SC'11), one 32-bit word per element, integer compare -- and this
+ * numbers: as easy as 1, 2, 3", SC'11), sixteen bits per element, integer compare -- and this
  * file is its scalar definition.  Pinned by the published known-answer vectors of Philox4x32-10. */
 #include <stdint.h>
 
@@ -18,22 +18,24 @@ void philox4x32_10_ref(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
 }
 
 uint32_t keep_threshold_ref(float p) {
-  const double s = (double)p * 4294967296.0;
-  return s >= 4294967295.0 ? 0xffffffffu : (uint32_t)s;
+  const double s = (double)p * 65536.0;
+  return s >= 65535.0 ? 65535u : (uint32_t)s;
 }
 
-/* mask[m][k] = word(e % 4) of philox(counter = (e / 4, 0, 0), key = seed) >= floor(p_row[m] * 2^32),
- * e = m * K + k. */
+/* mask[m][k] = draw(e % 8) of philox(counter = (e / 8, 0, 0), key = seed) >= floor(p_row[m] * 2^16),
+ * e = m * K + k; draw j is the low (even j) or high (odd j) 16 bits of output word j / 2. */
 void keep_mask_ref(uint8_t* mask, int64_t M, int64_t K, const float* row_p, uint64_t seed) {
   const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
   for (int64_t m = 0; m < M; m++) {
     const uint32_t thr = keep_threshold_ref(row_p[m]);
     for (int64_t k = 0; k < K; k++) {
-      const uint64_t e = (uint64_t)(m * K + k), c = e >> 2;
+      const uint64_t e = (uint64_t)(m * K + k), c = e >> 3;
       const uint32_t ctr[4] = {(uint32_t)c, (uint32_t)(c >> 32), 0u, 0u};
       uint32_t w[4];
       philox4x32_10_ref(ctr, key, w);
-      mask[m * K + k] = w[e & 3] >= thr ? 1 : 0;
+      const uint32_t word = w[(e & 7) >> 1];
+      const uint32_t draw = (e & 1) ? word >> 16 : word & 0xffffu;
+      mask[m * K + k] = draw >= thr ? 1 : 0;
     }
   }
 }

@@ -28,7 +28,7 @@ def test_mask_bit_exact(M, K, p, seed):
 
 
 def test_mask_counter_beyond_32_bits():
-    """Element indices above 2^32 (counter index above 2^30): a tall mask checked on its last rows."""
+    """Element indices above 2^32 (64-bit index arithmetic in the kernel): a tall mask checked on its last rows."""
     from lorafusion_amd.ops import hip_ops
 
     M, K, p, seed = 270_000, 16_384, 0.25, 77     # 4.4e9 elements, 4.4 GB of mask
@@ -39,10 +39,11 @@ def test_mask_counter_beyond_32_bits():
     for r, g in zip(rows, got):
         e0 = r * K
         exp = np.empty(K, dtype=np.uint8)
-        for c in range(K // 4):
-            ctr = (e0 >> 2) + c
+        for c in range(K // 8):
+            ctr = (e0 >> 3) + c
             w = od.philox4x32_10([ctr & 0xFFFFFFFF, ctr >> 32, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
-            exp[4 * c:4 * c + 4] = w >= thr
+            draws = np.stack([w & 0xFFFF, w >> 16], axis=1).reshape(-1)    # low half first
+            exp[8 * c:8 * c + 8] = draws >= thr
         assert np.array_equal(g, exp), f"row {r}"
     del m
 

@@ -47,21 +47,24 @@ def test_philox_against_second_implementation():
 
 def test_threshold():
     assert od.keep_threshold(0.0) == 0
-    assert od.keep_threshold(0.5) == 2**31
-    assert od.keep_threshold(0.25) == 2**30
-    # float32(0.1) * 2^32, floored
-    assert od.keep_threshold(0.1) == int(float(np.float32(0.1)) * 2**32)
-    assert od.keep_threshold(float(np.nextafter(np.float32(1.0), np.float32(0.0)))) == 0xFFFFFF00
+    assert od.keep_threshold(0.5) == 2**15
+    assert od.keep_threshold(0.25) == 2**14
+    # float32(0.1) * 2^16, floored
+    assert od.keep_threshold(0.1) == int(float(np.float32(0.1)) * 2**16) == 6553
+    assert od.keep_threshold(float(np.nextafter(np.float32(1.0), np.float32(0.0)))) == 0xFFFF
 
 
 def test_mask_definition_elementwise():
-    """Element e uses counter (e // 4, 0, 0, 0), key = (seed low, seed high), word e % 4."""
+    """Element e uses counter (e // 8, 0, 0, 0), key = (seed low, seed high) and the 16-bit draw e % 8 of the
+    four output words: word (e % 8) // 2, low half for even e, high half for odd e."""
     M, K, seed, p = 3, 16, 0x1234567890ABCDEF, 0.3
     mask = od.keep_mask(M, K, p, seed)
     thr = od.keep_threshold(p)
     for e in range(M * K):
-        w = _philox_numpy([e // 4, 0, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
-        assert mask.reshape(-1)[e] == (1 if w[e % 4] >= thr else 0)
+        w = _philox_numpy([e // 8, 0, 0, 0], [seed & 0xFFFFFFFF, seed >> 32])
+        word = w[(e % 8) // 2]
+        draw = (word >> 16) if e % 2 else (word & 0xFFFF)
+        assert mask.reshape(-1)[e] == (1 if draw >= thr else 0)
 
 
 def test_mask_properties():
