@@ -1,6 +1,6 @@
 """Seeded dropout keep-mask oracle (test infrastructure): ctypes front end of dropout_oracle.c.
 
-The mask stream is the build's own definition (Philox4x32-10, one word per element, integer
+The mask stream is the build's own definition (Philox4x32-10, sixteen bits per element, integer
 compare), not the reference's Triton stream (dropout.py:49-50): the reference's stream could only
 be reproduced by running Triton on a GPU, and nothing downstream depends on which Bernoulli
 stream is drawn.  What is pinned here is that the device kernel implements exactly this
