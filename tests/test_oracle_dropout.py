@@ -1,7 +1,7 @@
 """CPU checks that pin the keep-mask oracle (oracle/dropout_oracle.c).
 
 * Philox4x32-10 against the three published known-answer vectors of the Random123 distribution
-  (zero, all-ones and the pi/e digits input);
+  (zero, all-ones and the pi digits input; tests/golden/philox4x32_10_kat.json);
 * against a second, independently written numpy implementation on random inputs;
 * the mask definition: which counter / word / threshold an element uses, p = 0 keeps everything,
   per-row p, and the keep rate.
@@ -13,11 +13,10 @@ import pytest
 from oracle import dropout as od
 
 
-KAT = [
-    ([0, 0, 0, 0], [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
-    ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
-    ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0], [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
-]
+from tests.util import golden
+
+KAT = [([int(x, 16) for x in v["counter"]], [int(x, 16) for x in v["key"]], [int(x, 16) for x in v["output"]])
+       for v in golden("philox4x32_10_kat.json")["vectors"]]
 
 
 @pytest.mark.parametrize("ctr,key,expect", KAT)

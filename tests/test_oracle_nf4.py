@@ -11,13 +11,11 @@
 import numpy as np
 
 from oracle import nf4
+from tests.util import golden
 
 
 def test_code_table_bits():
-    expect = [-1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453, -0.28444138169288635,
-              -0.18477343022823334, -0.09105003625154495, 0.0, 0.07958029955625534, 0.16093020141124725,
-              0.24611230194568634, 0.33791524171829224, 0.44070982933044434, 0.5626170039176941,
-              0.7229568362236023, 1.0]
+    expect = [float(v) for v in golden("nf4_code_table.json")["values"]]
     assert nf4.NF4_CODE.dtype == np.float32
     assert np.array_equal(nf4.NF4_CODE, np.asarray(expect, dtype=np.float32))
     lib_table = np.ctypeslib.as_array(nf4._lib().nf4_code_table(), shape=(16,))

@@ -13,13 +13,17 @@ from hypothesis import given, settings, strategies as st
 
 from oracle import nf4 as onf4
 from oracle import routing
+from tests.util import golden
 
 
 def test_reference_worked_example():
-    padded, lookup, bp, ba, max_r, en, same = routing.block_tables([129, 130, 128], [16, 16, 16], [0.1] * 3, [2.0] * 3, 128)
-    assert padded == [256, 256, 128]
-    assert lookup[:, 1].tolist() == [128, 1, 128, 2, 128]
-    assert lookup[:, 2].tolist() == [0, 0, 2, 2, 4]
+    ex = golden("routing_worked_example.json")
+    n = len(ex["seq_len_list"])
+    padded, lookup, bp, ba, max_r, en, same = routing.block_tables(ex["seq_len_list"], [16] * n, [0.1] * n, [2.0] * n,
+                                                                   ex["block_size_m"])
+    assert padded == ex["padded_seq_len_list"]
+    assert lookup[:, 1].tolist() == ex["valid_rows_per_block"]
+    assert lookup[:, 2].tolist() == ex["first_block_per_block"]
     assert lookup[:, 0].tolist() == [16] * 5
     assert max_r == 16 and en and same == 0.1
     assert bp.tolist() == [0.1] * 5 and ba.tolist() == [2.0] * 5

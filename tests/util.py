@@ -57,3 +57,12 @@ def multi_inputs(seq_len_list, K, N, ranks, p_list, seed=0, dtype=torch.bfloat16
     mask = u >= row_p[:, None] if any(p > 0 for p in p_list) else None
     bias_t = (torch.randn(N, generator=g) * 0.1).to(dtype) if bias else None
     return dict(x=x, w=w, dy=dy, a_list=a_list, b_list=b_list, mask=mask, padded=padded, bias=bias_t)
+
+
+def golden(name: str):
+    """A fixture of tests/golden (JSON data)."""
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name)) as f:
+        return json.load(f)
