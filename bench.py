@@ -39,11 +39,11 @@ DROPOUT = [0.0, 0.05, 0.1, 0.1]
 BLOCK = 128
 
 
-def segments(total_tokens: int, n_adapters: int, seed: int = 0):
+def segments(total_tokens: int, n_adapters: int, seed: int = 0, longest: int = 4096):
     rng = np.random.default_rng(seed)
     lens, tot = [], 0
     while tot < total_tokens:
-        n = int(np.clip(rng.lognormal(6.5, 0.8), 64, 4096))
+        n = int(np.clip(rng.lognormal(6.5, 0.8), 64, longest))
         n = min(n, total_tokens - tot)
         lens.append(n)
         tot += n
@@ -119,6 +119,90 @@ def graph_time_ms(fn, reps: int, inner: int = 10) -> float:
     return e0.elapsed_time(e1) / (n * inner)
 
 
+# The other benchmark configurations of the reference, as linear layers of the same fused path:
+# (tokens, adapters, rank, scales, dropout, NF4 base weight, longest segment, [(projection, K, N)]).
+LAYER_WORKLOADS = {
+    "c1": (2048, 1, 16, [2.0], [0.1], False, 4096, [("linear", 4096, 4096)]),
+    "c3": (4096, 1, 16, [2.0], [0.0], True, 4096, [("linear", 4096, 14336)]),
+    "c4": (16384, 4, 16, [1.0, 2.0, 2.0, 4.0], [0.0, 0.05, 0.1, 0.1], False, 8192,
+           [("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024), ("o", 4096, 4096),
+            ("gate", 4096, 14336), ("up", 4096, 14336), ("down", 14336, 4096)]),
+    "c5": (8192, 8, 64, [1.0, 2.0, 2.0, 4.0] * 2, [0.0, 0.05, 0.1, 0.1] * 2, True, 4096,
+           [("q", 8192, 8192), ("k", 8192, 1024), ("v", 8192, 1024), ("o", 8192, 8192),
+            ("gate", 8192, 28672), ("up", 8192, 28672), ("down", 28672, 8192)]),
+}
+LAYER_NAMES = {
+    "c1": "single LoRA linear, 2048 tokens, K=N=4096, r=16, p=0.1, explicit mask, fwd+bwd",
+    "c3": "NF4 QLoRA linear 4096 -> 14336, 4096 tokens, r=16, dequantisation inside the call, fwd+bwd",
+    "c4": "the seven LoRA linears of an 8B-class decoder layer (hidden 4096, kv 1024, MLP 14336), 16384 packed "
+          "tokens, 4 adapters r=16, fwd+bwd; attention, norms and activation are not part of the path",
+    "c5": "the seven LoRA linears of a 70B-class decoder layer (hidden 8192, kv 1024, MLP 28672) with NF4 base "
+          "weights, 8192 packed tokens, 8 adapters r=64, fwd+bwd; attention, norms and activation are not part of the path",
+}
+
+
+def layer_workload(args, name: str) -> None:
+    """One of the reference's other configurations: every projection timed on its own (inputs of one
+    projection resident at a time), `value` = algorithmic flops of all projections / the sum of their times."""
+    from lorafusion_amd.ops import hip_ops
+    from lorafusion_amd.ops.multi_lora import prepare_multi_lora_batch_info
+    from lorafusion_amd.ops.nf4 import NF4WeightRef, quantize_nf4
+
+    tokens, n_ad, rank, scales, drops, nf4, longest, projs = LAYER_WORKLOADS[name]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    seq = segments(tokens, n_ad, longest=longest) if n_ad > 1 else [tokens]
+    info = prepare_multi_lora_batch_info(seq, list(range(n_ad)), [rank] * n_ad, drops, scales, BLOCK)
+    padded = info.padded_seq_len_list
+    Mp = sum(padded)
+    routing = hip_ops.MultiRouting(padded, [rank] * n_ad, info.block_to_lookup_table, info.block_to_alpha, info.block_to_dropout_p)
+    row_p = torch.cat([torch.full((pl,), float(p)) for pl, p in zip(padded, drops)]).to(dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    per_proj, total_ms, total_flops = {}, 0.0, 0.0
+    for pname, k, n in projs:
+        x = torch.randn(Mp, k, generator=g, device=dev).to(torch.bfloat16)
+        dy = torch.randn(Mp, n, generator=g, device=dev).to(torch.bfloat16)
+        w = (torch.randn(n, k, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        a_l = [((torch.rand(rank, k, generator=g, device=dev) * 2 - 1) / k ** 0.5).to(torch.bfloat16) for _ in range(n_ad)]
+        b_l = [(torch.randn(n, rank, generator=g, device=dev) * 0.01).to(torch.bfloat16) for _ in range(n_ad)]
+        mask = (torch.rand(Mp, k, generator=g, device=dev) >= row_p[:, None]) if any(p > 0 for p in drops) else None
+        if nf4:
+            packed, qs = quantize_nf4(w.float())
+            wref = NF4WeightRef(packed, qs)
+            del w
+
+            def step():
+                y, s_ = hip_ops.nf4_lora_forward(x, wref, a_l, b_l, routing.c, routing.R, mask, None)
+                return y, hip_ops.nf4_lora_backward(dy, x, wref, a_l, b_l, s_, routing.c, routing.R, mask, [rank] * n_ad)
+        else:
+            def step():
+                y, s_ = hip_ops.lora_forward(x, w, a_l, b_l, routing.c, routing.R, mask, None)
+                return y, hip_ops.lora_backward(dy, x, w, a_l, b_l, s_, routing.c, routing.R, mask, [rank] * n_ad)
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        flops = 2 * (2.0 * tokens * k * n) + 6.0 * tokens * rank * (k + n)
+        per_proj[pname] = {"K": k, "N": n, "ms": round(ms, 4), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1)}
+        total_ms += ms
+        total_flops += flops
+        del x, dy, mask, a_l, b_l, step
+        torch.cuda.empty_cache()
+    print(json.dumps({
+        "metric": "fused LoRA fwd+bwd TFLOP/s (8B layer, r=16); NF4 dequant GB/s; % roofline",
+        "value": round(total_flops / (total_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(total_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": LAYER_NAMES[name], "tokens": tokens, "rows_launched": Mp, "rank": rank, "adapters": n_ad,
+                   "nf4_base": nf4, "seq_len_list": seq},
+        "projections": per_proj, "roofline": None, "cpu_baseline": None,
+    }))
+
+
 def cpu_baseline(seq, budget_s: float = 15.0):
     """Oracle (bf16 op-by-op, autograd backward) on the host cores: the whole 8192-token batch when one
     run takes under a second (it does on the GPU box's host), else the first 256 tokens of every
@@ -176,6 +260,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", choices=["c2", *LAYER_WORKLOADS], default="c2",
+                    help="c2 (default): the multi-LoRA packed batch the metric is quoted on; c1, c3, c4, c5: the "
+                         "reference's other configurations, one line with a per-projection breakdown and no roofline entry")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -183,6 +270,9 @@ def main():
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (MI355X); none is visible.")
+
+    if args.workload != "c2":
+        return layer_workload(args, args.workload)
 
     from lorafusion_amd.ops import hip_ops
     from lorafusion_amd.ops.multi_lora import fused_linear_multi_lora, prepare_multi_lora_batch_info
