@@ -164,8 +164,11 @@ __global__ void __launch_bounds__(xa_waves(RT) * 64)
 lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_t* __restrict__ mask_out,
                uint32_t seed_lo, uint32_t seed_hi, T* __restrict__ S, int M, int K, int R, const LfSegTable seg) {
   constexpr int XA_WAVES = xa_waves(RT), XA_U = xa_unroll(RT);
-  __shared__ __attribute__((aligned(16))) char patch_all[XA_WAVES * 2048 * (1 + RT)];
-  __shared__ float red[XA_WAVES][XA_ROWS][RT * 16];
+  // the partial accumulators of the final sum reuse the patches (a barrier separates the two uses): at
+  // rank 64 the separate 16 KB pushed the workgroup over 40 KB, and a CU then holds two workgroups, not four
+  constexpr int PATCH_BYTES = XA_WAVES * 2048 * (1 + RT), RED_BYTES = XA_WAVES * XA_ROWS * RT * 16 * 4;
+  __shared__ __attribute__((aligned(16))) char patch_all[PATCH_BYTES > RED_BYTES ? PATCH_BYTES : RED_BYTES];
+  float (*red)[XA_ROWS][RT * 16] = (float (*)[XA_ROWS][RT * 16])patch_all;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, qq = lane >> 4;
   const int row0 = blockIdx.x * XA_ROWS;
@@ -254,6 +257,7 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
     load_batch(0, s0);
     use_batch(0, s0);
   }
+  __syncthreads();  // every wave is done with its patches
   // C layout: lane holds column (lane & 15), rows 4*(lane >> 4) + e
 #pragma unroll
   for (int c = 0; c < RT; c++)
