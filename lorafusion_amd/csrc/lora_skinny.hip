@@ -368,7 +368,8 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
   for (int g = tid; g < ROWS * RT * 2; g += 256) {
     const int row = g / (RT * 2), gc = g % (RT * 2);
     lf_u32x4 v = {0, 0, 0, 0};
-    if (row < bi.valid) v = *(const lf_u32x4*)(S + (int64_t)(blk * ROWS + row) * R + gc * 8);
+    // S has R columns; R may be smaller than the RT * 16 columns of the register tiling (R = 48, 80, 96, 112)
+    if (row < bi.valid && gc * 8 < R) v = *(const lf_u32x4*)(S + (int64_t)(blk * ROWS + row) * R + gc * 8);
     *(lf_u32x4*)(ss + row * RP + gc * 16) = v;
   }
   tile_store(tr, ys, tid, false);
@@ -419,7 +420,8 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
 #pragma unroll
     for (int c = 0; c < RT; c++)
 #pragma unroll
-      for (int e = 0; e < 4; e++) dbo[(int64_t)(wave * 16 + qq * 4 + e) * R + c * 16 + li] = acc_db[c][e];
+      for (int e = 0; e < 4; e++)
+        if (c * 16 < R) dbo[(int64_t)(wave * 16 + qq * 4 + e) * R + c * 16 + li] = acc_db[c][e];
 
     if (t + 1 < ntiles) {
       tile_store(tr, ys + ((t + 1) & 1) * TILE_BYTES, tid, false);
@@ -439,7 +441,7 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         const int row = blk * ROWS + wave * 32 + rt * 16 + qq * 4 + e;
-        if (row < Mrows) dso[(int64_t)row * R + c * 16 + li] = acc_ds[rt][c][e];
+        if (row < Mrows && c * 16 < R) dso[(int64_t)row * R + c * 16 + li] = acc_ds[rt][c][e];
       }
 }
 
@@ -540,7 +542,7 @@ lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const 
       const int g = i * 256 + tid;
       const int row = g / (RT * 2), gc = g % (RT * 2);
       lf_u32x4 v = {0, 0, 0, 0};
-      if (row < valid) v = *(const lf_u32x4*)(dS + (int64_t)(b * ROWS + row) * R + gc * 8);
+      if (row < valid && gc * 8 < R) v = *(const lf_u32x4*)(dS + (int64_t)(b * ROWS + row) * R + gc * 8);
       dr[i] = v;
     }
   };
@@ -597,7 +599,8 @@ lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const 
 #pragma unroll
   for (int c = 0; c < RT; c++)
 #pragma unroll
-    for (int e = 0; e < 4; e++) po[(int64_t)(c * 16 + qq * 4 + e) * K + kt * 64 + wave * 16 + li] = acc[c][e];
+    for (int e = 0; e < 4; e++)
+      if (c * 16 < R) po[(int64_t)(c * 16 + qq * 4 + e) * K + kt * 64 + wave * 16 + li] = acc[c][e];  // the partial has R rows
 }
 
 int rt_of(int R) { return R <= 16 ? 1 : R <= 32 ? 2 : R <= 64 ? 4 : 8; }

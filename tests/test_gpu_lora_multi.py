@@ -70,6 +70,8 @@ def _run(seq_len_list, K, N, ranks, p_list, scale_list, seed=0, bias=False, expl
         ([200, 50], [16, 64], [0.0, 0.0], [2.0, 0.5]),                               # mixed ranks, no dropout
         ([1, 127, 128, 129, 5, 300, 77, 64], [16, 32, 16, 8, 64, 16, 16, 32], [0.1] * 8, [1.0] * 8),  # 8 adapters
         ([640], [16], [0.1], [2.0]),                                                 # one segment through the multi path
+        ([200, 130, 300], [16, 48, 8], [0.1, 0.0, 0.25], [1.0, 2.0, 0.5]),          # S/dS of 48 columns: not a power of two
+        ([150, 260], [96, 40], [0.1, 0.1], [0.5, 2.0]),                              # 96 columns; rank 40 inside them
     ],
 )
 def test_multi_parity(seq, ranks, p_list, scales):

@@ -58,6 +58,10 @@ def _run_case(M, K, N, r, p, scale, dtype=torch.bfloat16, bias=False, seed=0, th
         (1, 128, 128, 16, 0.1, 2.0),     # single token
         (130, 384, 256, 8, 0.2, 4.0),    # rank 8 (padded to 16 inside)
         (300, 256, 256, 128, 0.1, 1.0),  # largest supported rank
+        (511, 1024, 384, 48, 0.0, 2.0),  # 48 columns of S/dS: fewer than the 64 of the kernels' register tiling
+        (257, 256, 384, 40, 0.3, 0.5),   # rank 40 in 48 columns
+        (300, 512, 640, 96, 0.1, 1.0),   # 96 columns (tiling of 128)
+        (130, 384, 256, 112, 0.1, 2.0),
     ],
 )
 def test_single_parity(M, K, N, r, p, scale):
