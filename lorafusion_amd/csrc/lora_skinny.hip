@@ -142,7 +142,7 @@ __device__ __forceinline__ lf_u32x4 tile_tr_frag(const char* tile, int row, int 
 }
 
 // ------------------------------------------------------------------------------------ xa
-// One workgroup of 8 waves (fewer for ranks above 32) per 16 rows; no partial sums leave the workgroup.  The K range is dealt
+// One workgroup of 8 waves (fewer for ranks above 32) per 16 rows (32 from rank 48 on); no partial sums leave the workgroup.  The K range is dealt
 // to the waves in 64-column steps (step s goes to wave s % waves), each wave streams its steps of the
 // 16 rows with coalesced 16-byte loads (8 lanes cover one 128-byte line), all loads of a batch
 // of steps in flight at once, applies the keep-mask in registers and turns the row-major
@@ -151,7 +151,10 @@ __device__ __forceinline__ lf_u32x4 tile_tr_frag(const char* tile, int row, int 
 // loads would put the four lanes of every quad on four different rows, a quarter of the
 // coalesced rate in the texture addresser.  The eight partial [16, R] accumulators are added in a fixed order through LDS,
 // scaled by 1/(1-p), zeroed in padded rows and beyond the adapter's rank, and stored as S.
-constexpr int XA_ROWS = 16;
+// Rows per workgroup: 16, or 32 from rank 48 on -- every workgroup reads the whole adapter matrix (from L2),
+// which at rank 64 is four times the bytes of its 16 rows of X; two row blocks share one set of A fragments.
+constexpr int xa_nb(int rt) { return rt >= 4 ? 2 : 1; }
+constexpr int xa_rows(int rt) { return 16 * xa_nb(rt); }
 // waves per workgroup and steps in flight per wave, by rank tiles (LDS: 2 KB * (1+RT) per wave; registers: 8 * RT per step)
 constexpr int xa_waves(int rt) { return rt <= 2 ? 8 : rt <= 4 ? 4 : 2; }
 constexpr int xa_unroll(int rt) { return rt <= 1 ? 4 : rt <= 2 ? 2 : 1; }
@@ -163,10 +166,10 @@ template <typename T, int RT, bool GEN>
 __global__ void __launch_bounds__(xa_waves(RT) * 64)
 lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_t* __restrict__ mask_out,
                uint32_t seed_lo, uint32_t seed_hi, T* __restrict__ S, int M, int K, int R, const LfSegTable seg) {
-  constexpr int XA_WAVES = xa_waves(RT), XA_U = xa_unroll(RT);
+  constexpr int XA_WAVES = xa_waves(RT), XA_U = xa_unroll(RT), NB = xa_nb(RT), XA_ROWS = xa_rows(RT);
   // the partial accumulators of the final sum reuse the patches (a barrier separates the two uses): at
   // rank 64 the separate 16 KB pushed the workgroup over 40 KB, and a CU then holds two workgroups, not four
-  constexpr int PATCH_BYTES = XA_WAVES * 2048 * (1 + RT), RED_BYTES = XA_WAVES * XA_ROWS * RT * 16 * 4;
+  constexpr int PATCH_BYTES = XA_WAVES * 2048 * (NB + RT), RED_BYTES = XA_WAVES * XA_ROWS * RT * 16 * 4;
   __shared__ __attribute__((aligned(16))) char patch_all[PATCH_BYTES > RED_BYTES ? PATCH_BYTES : RED_BYTES];
   float (*red)[XA_ROWS][RT * 16] = (float (*)[XA_ROWS][RT * 16])patch_all;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -179,16 +182,16 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
   const uint32_t thr = lf_keep_threshold(bi.p);
   const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
   const int nsteps = K / 64;
-  char* patch = patch_all + wave * 2048 * (1 + RT);  // X patch, then one patch per 16 rank rows of A
+  char* patch = patch_all + wave * 2048 * (NB + RT);  // one X patch per 16-row block, then one patch per 16 rank rows of A
 
   // loader mapping: lane -> (row lane>>3 (+8), granule lane&7); fragment mapping: (row li, granule 4h+qq)
   const int lrow = lane >> 3, lg = lane & 7;
-  const T* xrow[2];
-  const uint8_t* mrow[2];
-  int64_t erow[2];    // GEN: element index of this lane's first column in each of its two rows
-  bool row_real[2];   // GEN: the row exists (is not a clamped duplicate): its mask bytes are written
+  const T* xrow[2 * NB];
+  const uint8_t* mrow[2 * NB];
+  int64_t erow[2 * NB];    // GEN: element index of this lane's first column in each of its rows (two per 16-row block)
+  bool row_real[2 * NB];   // GEN: the row exists (is not a clamped duplicate): its mask bytes are written
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < 2 * NB; i++) {
     const int r = min(row0 + i * 8 + lrow, Mrows - 1);
     xrow[i] = X + (int64_t)r * K + lg * 8;
     mrow[i] = mask + (int64_t)r * K + lg * 8;
@@ -198,24 +201,29 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
   const int wr_off[2] = {lrow * 128 + ((lg ^ ((lrow >> 1) & 7)) << 4), (8 + lrow) * 128 + ((lg ^ (((8 + lrow) >> 1) & 7)) << 4)};
   const int rd_row = li * 128, rd_key = (li >> 1) & 7;
 
-  lf_f32x4 acc[RT];
+  lf_f32x4 acc[NB][RT];
 #pragma unroll
-  for (int c = 0; c < RT; c++) acc[c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+    for (int c = 0; c < RT; c++) acc[nb][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
 
   // (a second register set to overlap the next batch's loads costs occupancy and measured slower)
-  lf_u32x4 xv[1][XA_U][2], av[1][XA_U][RT][2];
-  lf_u32x2 mv[1][XA_U][2];
+  lf_u32x4 xv[1][XA_U][2 * NB], av[1][XA_U][RT][2];
+  lf_u32x2 mv[1][XA_U][2 * NB];
   auto load_batch = [&](int b, int s0) {
 #pragma unroll
     for (int u = 0; u < XA_U; u++) {
       const int s = s0 + u * XA_WAVES;
       if (s < nsteps) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < 2 * NB; i++) {
           xv[b][u][i] = *((const lf_u32x4*)(xrow[i] + s * 64));
           if constexpr (!GEN) {
             if (use_mask) mv[b][u][i] = *((const lf_u32x2*)(mrow[i] + s * 64));
           }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
 #pragma unroll
           for (int c = 0; c < RT; c++) {
             const int ar = c * 16 + i * 8 + lrow;
@@ -232,23 +240,31 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
       const int s = s0 + u * XA_WAVES;
       if (s < nsteps) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < 2 * NB; i++) {
           if constexpr (GEN) {
             uint32_t klo, khi;
             lf_keep8((uint64_t)(erow[i] + s * 64) >> 3, thr, seed_lo, seed_hi, klo, khi);
             mv[b][u][i] = lf_u32x2{klo, khi};
             if (row_real[i]) *(lf_u32x2*)(mask_out + erow[i] + s * 64) = mv[b][u][i];
           }
-          *(lf_u32x4*)(patch + wr_off[i]) = use_mask ? apply_mask8(xv[b][u][i], mv[b][u][i]) : xv[b][u][i];
-#pragma unroll
-          for (int c = 0; c < RT; c++) *(lf_u32x4*)(patch + (1 + c) * 2048 + wr_off[i]) = av[b][u][c][i];
+          *(lf_u32x4*)(patch + (i >> 1) * 2048 + wr_off[i & 1]) = use_mask ? apply_mask8(xv[b][u][i], mv[b][u][i]) : xv[b][u][i];
         }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int c = 0; c < RT; c++) *(lf_u32x4*)(patch + (NB + c) * 2048 + wr_off[i]) = av[b][u][c][i];
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           const int fo = rd_row + (((h * 4 + qq) ^ rd_key) << 4);
-          const lf_u32x4 xf = *(const lf_u32x4*)(patch + fo);
+          lf_u32x4 af[RT];
 #pragma unroll
-          for (int c = 0; c < RT; c++) acc[c] = Mfma16<T>::run(xf, *(const lf_u32x4*)(patch + (1 + c) * 2048 + fo), acc[c]);
+          for (int c = 0; c < RT; c++) af[c] = *(const lf_u32x4*)(patch + (NB + c) * 2048 + fo);
+#pragma unroll
+          for (int nb = 0; nb < NB; nb++) {
+            const lf_u32x4 xf = *(const lf_u32x4*)(patch + nb * 2048 + fo);
+#pragma unroll
+            for (int c = 0; c < RT; c++) acc[nb][c] = Mfma16<T>::run(xf, af[c], acc[nb][c]);
+          }
         }
       }
     }
@@ -260,9 +276,11 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
   __syncthreads();  // every wave is done with its patches
   // C layout: lane holds column (lane & 15), rows 4*(lane >> 4) + e
 #pragma unroll
-  for (int c = 0; c < RT; c++)
+  for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-    for (int e = 0; e < 4; e++) red[wave][qq * 4 + e][c * 16 + li] = acc[c][e];
+    for (int c = 0; c < RT; c++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) red[wave][nb * 16 + qq * 4 + e][c * 16 + li] = acc[nb][c][e];
   __syncthreads();
   const float mult = bi.p > 0.f ? 1.f / (1.f - bi.p) : 1.f;
   for (int o = tid; o < XA_ROWS * RT * 16; o += XA_WAVES * 64) {
@@ -642,7 +660,7 @@ size_t lf_xa_workspace(int, int, int, const LfSegTable&) { return 0; }
 template <typename T, int RT>
 static int xa_launch(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t seed, void* S, int M, int K, int R,
                      int64_t rows, const LfSegTable& seg, hipStream_t st) {
-  const unsigned grid = (unsigned)((rows + XA_ROWS - 1) / XA_ROWS);
+  const unsigned grid = (unsigned)((rows + xa_rows(RT) - 1) / xa_rows(RT));
   if (mask_out != nullptr)
     hipLaunchKernelGGL((lora_xa_kernel<T, RT, true>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
                        (uint32_t)seed, (uint32_t)(seed >> 32), (T*)S, M, K, R, seg);
