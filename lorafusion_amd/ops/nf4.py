@@ -159,14 +159,14 @@ def quantize_nf4(w: torch.Tensor, blocksize: int = 64, compress_statistics: bool
     out_dtype = dtype or (w.dtype if w.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16)
     if not compress_statistics:
         return packed, QuantState(shape, out_dtype, blocksize, absmax)
-    if absmax.numel() % blocksize2:
-        raise ValueError("number of blocks must be a multiple of the second-level blocksize")
     offset = absmax.double().mean().float().reshape(1)
-    centred = (absmax - offset).reshape(-1, blocksize2)
+    nb = absmax.numel()
+    pad = (-nb) % blocksize2          # a short last second-level block is padded with zeros, which change no maximum
+    centred = torch.nn.functional.pad(absmax - offset, (0, pad)).reshape(-1, blocksize2)
     absmax2 = centred.abs().amax(dim=1)
     safe2 = torch.where(absmax2 > 0, absmax2, torch.ones_like(absmax2))
     code = dynamic_code_table(w.device)
-    absq = _nearest((centred / safe2[:, None]).reshape(-1), code)
+    absq = _nearest((centred / safe2[:, None]).reshape(-1), code)[:nb].contiguous()
     return packed, QuantState(shape, out_dtype, blocksize, absq, offset, QuantState2(absmax2, code, blocksize2))
 
 

@@ -90,6 +90,26 @@ def test_dequant_config2_shape_and_roundtrip():
     assert (err <= (0.1520 + 0.03) * absmax_true + 1e-6).all()
 
 
+def test_quantiser_short_last_second_level_block():
+    """A weight whose block count is not a multiple of the second-level block size (896 x 896 at block size
+    128: 6272 blocks, 24.5 groups of 256): the product quantiser pads the last group, the state it returns
+    dequantises bit-exactly against the oracle, and the round trip stays within the code's resolution."""
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton, quantize_nf4
+
+    g = torch.Generator(device="cuda").manual_seed(5)
+    w = torch.randn(896, 896, generator=g, device="cuda") * 0.02
+    packed, qs = quantize_nf4(w, blocksize=128)
+    assert qs.absmax.numel() == 6272 and qs.state2.absmax.numel() == 25
+    st = onf4.NF4State(packed=packed.cpu().numpy().reshape(-1), shape=(896, 896), blocksize=128, absmax=qs.absmax.cpu().numpy(),
+                       code2=qs.state2.code.cpu().numpy(), absmax2=qs.state2.absmax.cpu().numpy(),
+                       offset=qs.offset.cpu().numpy().reshape(1).astype(np.float32), blocksize2=256)
+    got = dequantize_nf4_triton(packed, qs)
+    assert np.array_equal(_bits(got), onf4.dequantize(st))
+    blocks = w.reshape(-1, 128)
+    err = (got.float().reshape(-1, 128) - blocks).abs().amax(dim=1)
+    assert bool((err <= (0.1520 + 0.03) * blocks.abs().amax(dim=1) + 1e-6).all())
+
+
 def test_dequant_errors():
     from lorafusion_amd.ops.nf4 import QuantState, dequantize_nf4_triton
 
