@@ -396,11 +396,14 @@ def main():
     nf4_bytes = n / 2 + n / 64 + 4 * n / 16384 + 1028 + 2 * n
     nf4_gbs = nf4_bytes / (t_nf4 * 1e-3) / 1e9
 
+    # HBM-side bytes per launch of the dominant kernel: the figure of the committed counter summary
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "gemm_traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "bench_c2_hbm_traffic.txt")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get("dx_gemm_bytes_per_launch")
+            for line in f:
+                if line.startswith("dominant_kernel_bytes_per_launch"):
+                    traffic = int(line.split()[1])
 
     res = {
         "metric": "fused LoRA fwd+bwd TFLOP/s (8B layer, r=16); NF4 dequant GB/s; % roofline",
