@@ -142,8 +142,12 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 
   // ---- direct-to-LDS buffer loads: per thread one 32-bit byte offset per 16-byte granule (row part,
   // clamped at the matrix edge); the K position of a tile is a scalar offset shared by the wave.
-  const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, 0x7fffffff, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, 0x7fffffff, 0x00020000);
+  // The buffer of an operand with K-contiguous rows starts at the tile's first row, so the 32-bit
+  // offsets span one panel of the tile and the operand itself may exceed 2 GiB.
+  const char* a_base = (const char*)p.A + (int64_t)m0 * p.lda * 2;
+  const char* b_base = NN ? (const char*)p.B : (const char*)p.B + (int64_t)n0 * p.ldb * 2;
+  const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)b_base, 0, 0x7fffffff, 0x00020000);
   uint32_t avoff[NLA], bvoff[NLB];
   {
     // LDS slot (tid&3) of row r holds source granule slot ^ ((r>>1)&3); r>>1 = tid>>3 (mod 4)
@@ -151,14 +155,14 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
     for (int i = 0; i < NLA; i++) {
       int row = i * (NTHREADS / 4) + (tid >> 2);
-      int gm = min(m0 + row, p.M - 1);
+      int gm = min(m0 + row, p.M - 1) - m0;  // row within the tile, clamped at the matrix edge
       avoff[i] = (uint32_t)((int64_t)gm * p.lda * 2 + srcg * 16);
     }
     if constexpr (!NN) {
 #pragma unroll
       for (int i = 0; i < NLB; i++) {
         int row = i * (NTHREADS / 4) + (tid >> 2);
-        int gn = min(n0 + row, p.N - 1);
+        int gn = min(n0 + row, p.N - 1) - n0;
         bvoff[i] = (uint32_t)((int64_t)gn * p.ldb * 2 + srcg * 16);
       }
     } else {
@@ -707,8 +711,8 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
   if (p.L != nullptr && (p.R % 16 != 0 || p.R <= 0 || p.R > LF_MAX_RANK)) return LF_ESHAPE;
   // the keep-mask is read 16 bytes at a time
   if (p.mask != nullptr && (p.N % 16 != 0 || p.ldmask % 16 != 0 || ((uintptr_t)p.mask & 15) != 0)) return LF_ESHAPE;
-  // tile loads address the operands with 32-bit byte offsets
-  if ((int64_t)p.M * p.lda * 2 >= 0x7fffffffLL || (int64_t)(nn ? p.K : p.N) * p.ldb * 2 >= 0x7fffffffLL) return LF_ESHAPE;
+  // tile loads address a panel of 256 rows (the K-major operand of the NN product: all of it) with 32-bit byte offsets
+  if (256 * p.lda * 2 >= 0x7fffffffLL || (int64_t)(nn ? p.K : 256) * p.ldb * 2 >= 0x7fffffffLL) return LF_ESHAPE;
   if (seg.table != nullptr && (seg.block_size_m % 64 != 0)) return LF_ESHAPE;
   auto launch = [&](const LfGemmParams& q, int cfg) {
     if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1)) cfg = 2;

@@ -46,6 +46,23 @@ def test_gemm_row_split_plan(trans_b, M, N):
     _close(auto, e, f"gemm auto plan M={M} N={N} trans_b={trans_b}")
 
 
+@pytest.mark.parametrize("trans_b", [True, False])
+def test_gemm_row_operand_above_2_gib(trans_b):
+    """A row operand of 2.46 GB (300000 x 4096): the tile loads address one 256-row panel at a time, so only the
+    panel has to fit 32-bit offsets.  Checked on the first, last and some middle rows against fp32 torch."""
+    from lorafusion_amd.ops import hip_ops
+
+    M, K, N = 300_000, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(3)
+    a = torch.randn(M, K, generator=g, device="cuda").bfloat16()
+    b = (torch.randn(N, K, generator=g, device="cuda") if trans_b else torch.randn(K, N, generator=g, device="cuda")).bfloat16()
+    c = hip_ops.gemm(a, b, trans_b=trans_b)
+    rows = torch.tensor([0, 1, 255, 256, 131_071, 131_072, 262_143, 262_144, 262_145, M - 257, M - 2, M - 1], device="cuda")
+    e = a[rows].float() @ (b.float().T if trans_b else b.float())
+    _close(c[rows], e.cpu(), f"gemm rows of a 2.46 GB operand, trans_b={trans_b}")
+    del a, c
+
+
 def test_gemm_identity_exact():
     """A @ I^T reproduces A bit for bit in every layout (catches operand / index transpositions)."""
     from lorafusion_amd.ops import hip_ops

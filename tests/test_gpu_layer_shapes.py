@@ -152,3 +152,32 @@ def test_nf4_linear_4096_to_14336():
     dxe, *_ = lora_ref.linear_lora_bwd_fp32(dys[ti], xs[ti], w_cpu, ac, bc, scale, ms[ti], p)
     _close(y.detach()[ti.cuda()], ye, "y rows")
     _close(x.grad[ti.cuda()], dxe, "dx rows")
+
+
+def test_activation_above_2_gib():
+    """270000 tokens x 4096 (2.2 GB of X, 1.1 GB of mask) through the single-adapter op: 32-bit offsets inside the
+    kernels must not span the whole operand.  dA and dB (sums over all rows) against the oracle in full, Y and dX
+    on sampled rows including the last ones."""
+    from lorafusion_amd.ops.lora_v1 import fused_linear_lora
+
+    M, K, N, r, p, scale = 270_000, 4096, 128, 16, 0.1, 2.0
+    x = _gpu_randn((M, K), 1).requires_grad_(True)
+    w = _gpu_randn((N, K), 2, 0.02)
+    dy = _gpu_randn((M, N), 3)
+    a = (_gpu_randn((r, K), 4) / math.sqrt(K)).requires_grad_(True)
+    b = _gpu_randn((N, r), 5, 0.01).requires_grad_(True)
+    mask = torch.rand((M, K), generator=torch.Generator(device="cuda").manual_seed(6), device="cuda") >= p
+    y = fused_linear_lora(x, w, a, b, scale, dropout_p=p, dropout_mask=mask)
+    y.backward(dy)
+    torch.cuda.synchronize()
+    xs, dys, ms = x.detach().cpu(), dy.cpu(), mask.cpu()
+    ac, bc, wc = a.detach().cpu(), b.detach().cpu(), w.cpu()
+    _, dae, dbe, _ = lora_ref.linear_lora_bwd_fp32(dys, xs, None, ac, bc, scale, ms, p)
+    _close(a.grad, dae, "da over 270000 rows")
+    _close(b.grad, dbe, "db over 270000 rows")
+    ti = torch.tensor([0, 1, 127, 128, 131_071, 131_072, 262_143, 262_144, 262_145, M - 129, M - 2, M - 1])
+    ye, _ = lora_ref.linear_lora_fwd_fp32(xs[ti], wc, ac, bc, scale, ms[ti], p)
+    dxe, *_ = lora_ref.linear_lora_bwd_fp32(dys[ti], xs[ti], wc, ac, bc, scale, ms[ti], p)
+    _close(y.detach()[ti.cuda()], ye, "y rows")
+    _close(x.grad[ti.cuda()], dxe, "dx rows")
+
