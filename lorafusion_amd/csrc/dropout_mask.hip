@@ -44,7 +44,6 @@ int lf_launch_dropout_mask(uint8_t* mask, int M, int K, float p, const float* bl
   const int64_t n16 = (int64_t)M * K / 16;
   const int64_t blocks = (n16 + 255) / 256;
   if (blocks > 0x7fffffffLL) return LF_ELIMIT;
-  hipLaunchKernelGGL(dropout_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, st, mask, n16, K, thr, block_p, block_size_m,
+  return lf_launch(dropout_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, st, mask, n16, K, thr, block_p, block_size_m,
                      (uint32_t)seed, (uint32_t)(seed >> 32));
-  return lf_check_launch();
 }

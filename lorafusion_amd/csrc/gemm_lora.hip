@@ -249,8 +249,9 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     const T* __restrict__ L = (const T*)p.L;
     const T* rp = (const T*)seg.ptr[0];
     int rank = seg.rank[0];
-    float mult = p.mult_mode == 0 ? seg.scale : (seg.p > 0.f ? 1.f / (1.f - seg.p) : 1.f);
+    // mult_mode 1 without a keep-mask means no dropout, whatever p says: the term is not rescaled
     bool use_mask = p.mask != nullptr && p.mult_mode == 1 && seg.p > 0.f;
+    float mult = p.mult_mode == 0 ? seg.scale : (use_mask ? 1.f / (1.f - seg.p) : 1.f);
     if (seg.table != nullptr) {
       int blk = (p.row0 + wrow0) / seg.block_size_m;
       blk = min(blk, seg.n_blocks - 1);
@@ -263,8 +264,8 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         mult = seg.block_scale[blk];
       } else {
         float pb = seg.block_p[blk];
-        mult = pb > 0.f ? 1.f / (1.f - pb) : 1.f;
         use_mask = p.mask != nullptr && pb > 0.f;
+        mult = use_mask ? 1.f / (1.f - pb) : 1.f;
       }
     }
     // Keep-mask of this wave's sub-tile: 16-byte loads that cover whole rows of the sub-tile (issued
@@ -632,10 +633,9 @@ int launch_cfg(LfGemmParams p, const LfSegTable& seg, hipStream_t st) {
   p.grid_m = (p.M + BM - 1) / BM;
   p.grid_n = (p.N + BN - 1) / BN;
   auto kern = gemm_lora_kernel<T, BM, BN, WM, WN, NN, NSTAGE>;
-  static bool lds_ok[64] = {};
+  static LfLdsFlags lds_ok;
   if (!lf_allow_lds(kern, SMEM, lds_ok)) return LF_ELAUNCH;
-  hipLaunchKernelGGL(kern, dim3(p.grid_m * p.grid_n), dim3(NTHREADS), SMEM, st, p, seg);
-  return lf_check_launch();
+  return lf_launch(kern, dim3(p.grid_m * p.grid_n), dim3(NTHREADS), SMEM, st, p, seg);
 }
 
 template <typename T, bool NN>

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <atomic>
 #include "../../include/lorafusion_hip.h"  // error codes, dtype ids, LF_MAX_SEG
 
 #define LF_MAX_RANK 128
@@ -55,19 +56,26 @@ struct LfGemmParams {
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st);
 
 // Raise a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's copy of
-// the function; the flag array is per kernel instantiation, a race only repeats the same call).
+// the function; one flag array per kernel instantiation; threads that race here repeat the same call).
+struct LfLdsFlags { std::atomic<bool> done[64]; };
 template <typename Kern>
-static inline bool lf_allow_lds(Kern kern, int bytes, bool (&done)[64]) {
+static inline bool lf_allow_lds(Kern kern, int bytes, LfLdsFlags& flags) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-  if (!done[dev]) {
+  if (!flags.done[dev].load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
-    done[dev] = true;
+    flags.done[dev].store(true, std::memory_order_release);
   }
   return true;
 }
 
-static inline int lf_check_launch() {
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? LF_OK : LF_ELAUNCH;
+// Launch `kern` and report this launch's own status: the return code of hipLaunchKernel, not the
+// thread's last-error slot, which may hold (and would lose) an error of the caller's earlier HIP calls.
+template <typename... KArgs, typename... Args>
+static inline int lf_launch(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t smem, hipStream_t st, Args&&... args) {
+  auto go = [&](KArgs... ka) {
+    void* argv[] = {(void*)&ka...};
+    return hipLaunchKernel((const void*)kern, grid, block, argv, smem, st);
+  };
+  return go(args...) == hipSuccess ? LF_OK : LF_ELAUNCH;
 }

@@ -282,7 +282,7 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
 #pragma unroll
       for (int e = 0; e < 4; e++) red[wave][nb * 16 + qq * 4 + e][c * 16 + li] = acc[nb][c][e];
   __syncthreads();
-  const float mult = bi.p > 0.f ? 1.f / (1.f - bi.p) : 1.f;
+  const float mult = (use_mask && bi.p > 0.f) ? 1.f / (1.f - bi.p) : 1.f;  // no mask given: no dropout, whatever p says
   for (int o = tid; o < XA_ROWS * RT * 16; o += XA_WAVES * 64) {
     const int r = o / (RT * 16), c = o % (RT * 16);
     const int row = row0 + r;
@@ -477,7 +477,7 @@ __device__ __forceinline__ void segment_blocks(const LfSegTable& seg, int s, int
 // out_s = cast( mult * sum over parts of part[...] ) for segment s = blockIdx.y.
 //   transposed == 0 (dB): parts are the segment's blocks, part[b][n][R] -> out [rows, rank]
 //   transposed == 1 (dA): parts are the segment's chunks, part[(s*max_chunks + ch)][R][rows] -> out [rank, rows]
-//   mult_mode 0: segment scale ; 1: 1/(1-p) of the segment.
+//   mult_mode 0: segment scale ; 1: 1/(1-p) of the segment ; 2: none (no keep-mask was given: no dropout).
 template <typename T>
 __device__ __forceinline__ void reduce_segments_body(int bx, int s, const float* __restrict__ part, int rows, int R, int transposed, int mult_mode, int M,
                        int group, int max_chunks, const LfSegTable seg) {
@@ -487,7 +487,9 @@ __device__ __forceinline__ void reduce_segments_body(int bx, int s, const float*
   int b0, b1;
   segment_blocks(seg, s, M, b0, b1);
   float mult;
-  if (seg.table == nullptr) {
+  if (mult_mode == 2) {
+    mult = 1.f;
+  } else if (seg.table == nullptr) {
     mult = mult_mode == 0 ? seg.scale : (seg.p > 0.f ? 1.f / (1.f - seg.p) : 1.f);
   } else {
     mult = mult_mode == 0 ? (seg.block_scale ? seg.block_scale[b0] : 1.f)
@@ -662,12 +664,10 @@ static int xa_launch(const void* X, const uint8_t* mask, uint8_t* mask_out, uint
                      int64_t rows, const LfSegTable& seg, hipStream_t st) {
   const unsigned grid = (unsigned)((rows + xa_rows(RT) - 1) / xa_rows(RT));
   if (mask_out != nullptr)
-    hipLaunchKernelGGL((lora_xa_kernel<T, RT, true>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
+    return lf_launch((lora_xa_kernel<T, RT, true>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
                        (uint32_t)seed, (uint32_t)(seed >> 32), (T*)S, M, K, R, seg);
-  else
-    hipLaunchKernelGGL((lora_xa_kernel<T, RT, false>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
+  return lf_launch((lora_xa_kernel<T, RT, false>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
                        0u, 0u, (T*)S, M, K, R, seg);
-  return lf_check_launch();
 }
 
 template <typename T>
@@ -710,10 +710,9 @@ static int dys_launch(const void* dY, const void* S, float* ds_part, float* db_p
   constexpr int RP = RT * 32 + 32;
   const int smem = dys_smem(RT);
   static_assert(RP == RT * 32 + 32, "");
-  static bool lds_ok[64] = {};
+  static LfLdsFlags lds_ok;
   if (!lf_allow_lds(kern, smem, lds_ok)) return LF_ELAUNCH;
-  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, tiles_per_wg, seg);
-  return lf_check_launch();
+  return lf_launch(kern, grid, dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, tiles_per_wg, seg);
 }
 
 template <typename T>
@@ -739,9 +738,8 @@ static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M
   for (int s = 0; s < nseg; s++) maxrank = seg.rank[s] > maxrank ? seg.rank[s] : maxrank;
   const int64_t nout = (int64_t)N * maxrank;
   const int nb_rows = (int)((n + 1023) / 1024), nb_seg = (int)((nout + 1023) / 1024);  // four outputs per thread
-  hipLaunchKernelGGL((reduce_ds_db_kernel<T>), dim3((unsigned)(nb_rows + nb_seg * nseg)), dim3(256), 0, st, (const float*)ds_part,
+  return lf_launch((reduce_ds_db_kernel<T>), dim3((unsigned)(nb_rows + nb_seg * nseg)), dim3(256), 0, st, (const float*)ds_part,
                      (T*)dS, split, M, R, nb_rows, (const float*)db_part, N, nb_seg, seg);
-  return lf_check_launch();
 }
 
 int lf_launch_dys_dyb(const void* dY, const void* S, void* dS, void* ws, size_t ws_bytes, int M, int N, int R,
@@ -795,10 +793,9 @@ static int da_launch(const void* X, const uint8_t* mask, const void* dS, float* 
   auto kern = lora_da_kernel<T, RT>;
   constexpr int RP = RT * 32 + 32;
   const int smem = 2 * TILE_BYTES + 2 * ROWS * RP;
-  static bool lds_ok[64] = {};
+  static LfLdsFlags lds_ok;
   if (!lf_allow_lds(kern, smem, lds_ok)) return LF_ELAUNCH;
-  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)X, mask, (const T*)dS, part, M, K, R, group, max_chunks, seg);
-  return lf_check_launch();
+  return lf_launch(kern, grid, dim3(256), smem, st, (const T*)X, mask, (const T*)dS, part, M, K, R, group, max_chunks, seg);
 }
 
 template <typename T>
@@ -819,8 +816,7 @@ static int da_impl(const void* X, const uint8_t* mask, const void* dS, void* ws,
   int maxrank = 0;
   for (int s = 0; s < nseg; s++) maxrank = seg.rank[s] > maxrank ? seg.rank[s] : maxrank;
   const int64_t nout = (int64_t)K * maxrank;
-  hipLaunchKernelGGL((reduce_segments_kernel<T>), dim3((unsigned)((nout + 1023) / 1024), nseg), dim3(256), 0, st, (const float*)part, K, R, 1, 1, M, group, max_chunks, seg);
-  return lf_check_launch();
+  return lf_launch((reduce_segments_kernel<T>), dim3((unsigned)((nout + 1023) / 1024), nseg), dim3(256), 0, st, (const float*)part, K, R, 1, mask != nullptr ? 1 : 2, M, group, max_chunks, seg);
 }
 
 int lf_launch_da(const void* X, const uint8_t* mask, const void* dS, void* ws, size_t ws_bytes, int M, int K, int R,

@@ -123,7 +123,7 @@ int lf_launch_nf4_dequant(const uint8_t* packed, const void* absmax, const float
   const int64_t grid = (n_words + per_wg - 1) / per_wg;
   if (grid > 0x7fffffffLL) return LF_ESHAPE;
 #define LF_NF4_LAUNCH(T, NESTED)                                                                         \
-  hipLaunchKernelGGL((nf4_dequant_kernel<T, NESTED>), dim3((unsigned)grid), dim3(NF4_THREADS), 0, st,    \
+  return lf_launch((nf4_dequant_kernel<T, NESTED>), dim3((unsigned)grid), dim3(NF4_THREADS), 0, st,      \
                      (const uint32_t*)packed, absmax, code2, absmax2, offset, (lf_u32x4*)out, n_words, shift, shift2)
   if (out_dtype == LF_BF16) {
     if (nested) LF_NF4_LAUNCH(__bf16, true); else LF_NF4_LAUNCH(__bf16, false);
@@ -133,5 +133,4 @@ int lf_launch_nf4_dequant(const uint8_t* packed, const void* absmax, const float
     return LF_EINVAL;
   }
 #undef LF_NF4_LAUNCH
-  return lf_check_launch();
 }

@@ -308,8 +308,11 @@ def fused_lora_da(x: torch.Tensor, ds: torch.Tensor, r: int, dropout_p: float = 
     if ds.shape[0] != M or ds.shape[1] not in (r, R):
         raise ValueError(f"ds must have shape [{M}, {r}], but got {tuple(ds.shape)}.")
     _check_dims(M, None, K)
+    _check_p(dropout_p)
+    if dropout_p > 0 and dropout_mask is None:
+        raise ValueError("dropout_mask must be provided if dropout_p != 0")
     mask = _check_mask(dropout_mask, x.shape) if dropout_p > 0 else None
-    routing = _routing_single(r, 1.0, dropout_p if mask is not None else 0.0)
+    routing = _routing_single(r, 1.0, dropout_p)
     da = torch.empty((r, K), dtype=x.dtype, device=x.device)
     ws, nbytes = _ws(L.LF_OP_DA, M, 0, K, R, routing, x.device)
     ds_p = _pad_cols(ds, R)
@@ -334,8 +337,11 @@ def fused_lora_dyw_dsa(dy: torch.Tensor, w: torch.Tensor, ds: torch.Tensor, a: t
     if ds.shape[0] != M or ds.shape[1] not in (r, R):
         raise ValueError(f"ds must have shape [{M}, {r}], but got {tuple(ds.shape)}.")
     _check_dims(M, N, K)
+    _check_p(dropout_p)
+    if dropout_p > 0 and dropout_mask is None:  # as fused_lora_dyw_dsa.py:184-297 does
+        raise ValueError("dropout_mask must be provided if dropout_p != 0")
     mask = _check_mask(dropout_mask, (M, K)) if dropout_p > 0 else None
-    routing = _routing_single(r, 1.0, dropout_p if mask is not None else 0.0)
+    routing = _routing_single(r, 1.0, dropout_p)
     dx = torch.empty((M, K), dtype=dy.dtype, device=dy.device)
     ds_p = _pad_cols(ds, R)
     rc = L.lib().lf_lora_dyw_dsa(L.ptr(dy), L.ptr(w), L.ptr(ds_p), L.ptr_array([a]), L.ptr(mask), L.ptr(dx),

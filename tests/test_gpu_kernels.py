@@ -115,6 +115,45 @@ def test_tier2_wrappers():
         T.fused_lora_xw_sb(x, w, s[:-1].contiguous(), b, alpha)
     with pytest.raises(ValueError):
         T.fused_lora_dyw_dsa(dy, w.t(), ds, a, p, mask)
+    # dropout asked for but no mask given: an error, as in the reference (fused_lora_dyw_dsa.py:234-236)
+    with pytest.raises(ValueError, match="dropout_mask must be provided"):
+        T.fused_lora_dyw_dsa(dy, w, ds, a, p, None)
+    with pytest.raises(ValueError, match="dropout_mask must be provided"):
+        T.fused_lora_da(x, ds, r, p, None)
+
+
+def test_null_mask_means_no_dropout_at_the_c_abi():
+    """At the C ABI a NULL keep-mask switches dropout off for the call: p of the routing is ignored and
+    nothing is rescaled by 1/(1-p) (xa, da, dyw_dsa), single routing and block tables alike."""
+    from lorafusion_amd import _lib as L
+    from lorafusion_amd.ops import hip_ops
+    from lorafusion_amd.ops.multi_lora import prepare_multi_lora_batch_info
+
+    M, K, N, r = 256, 512, 384, 16
+    d = single_inputs(M, K, N, r, p=0.0, seed=6)
+    x, w, a, b, dy = (d[k].cuda() for k in ("x", "w", "a", "b", "dy"))
+    lib = L.lib()
+    info = prepare_multi_lora_batch_info([M], [0], [r], [0.25], [2.0], 128)
+    multi = hip_ops.MultiRouting(info.padded_seq_len_list, [r], info.block_to_lookup_table, info.block_to_alpha,
+                                 info.block_to_dropout_p)
+    for what, rt in (("single", L.single_routing(r, 1.0, 0.25)), ("table", multi.c)):
+        s = torch.empty((M, 16), dtype=x.dtype, device="cuda")
+        rc = lib.lf_lora_xa(L.ptr(x), None, L.ptr_array([a]), L.ptr(s), None, 0, M, K, 16, rt, L.LF_BF16, L.stream_of(x))
+        assert rc == 0
+        _close(s, d["x"].float() @ d["a"].float().T, f"{what}: S without a mask")
+        ds = (torch.randn(M, 16) * 0.1).to(torch.bfloat16).cuda()
+        da = torch.empty((r, K), dtype=x.dtype, device="cuda")
+        need = lib.lf_workspace_bytes(L.LF_OP_DA, M, 0, K, 16, rt)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        rc = lib.lf_lora_da(L.ptr(x), None, L.ptr(ds), L.ptr_array([da]), L.ptr(ws), need, M, K, 16, rt, L.LF_BF16,
+                            L.stream_of(x))
+        assert rc == 0
+        _close(da, ds.float().cpu().T @ d["x"].float(), f"{what}: dA without a mask")
+        dx = torch.empty((M, K), dtype=x.dtype, device="cuda")
+        rc = lib.lf_lora_dyw_dsa(L.ptr(dy), L.ptr(w), L.ptr(ds), L.ptr_array([a]), None, L.ptr(dx), M, N, K, 16, rt,
+                                 L.LF_BF16, L.stream_of(x))
+        assert rc == 0
+        _close(dx, d["dy"].float() @ d["w"].float() + ds.float().cpu() @ d["a"].float(), f"{what}: dX without a mask")
 
 
 def test_seeded_mask_statistics_and_reproducibility():
