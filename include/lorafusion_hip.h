@@ -10,7 +10,9 @@
  *    `lf_routing` and the `*_ptrs` arrays are HOST memory, read during the call only.
  *  - dtype: LF_BF16 or LF_F16 for all 16-bit tensors of a call; accumulation is fp32.
  *  - Return 0 on success, a negative LF_E* code otherwise (lf_strerror gives the text).  The
- *    library keeps no global mutable state and may be called from several host threads.
+ *    library may be called from several host threads: the only state it keeps is set once per
+ *    device and then only read (per-kernel LDS limits, the address of the static scratch buffer);
+ *    lf_lora_bwd_static is the one entry point whose calls share memory (see there).
  *  - Work is enqueued on `stream` (a hipStream_t, passed as void*); nothing synchronises.
  *  - The library allocates nothing: scratch memory comes in through `workspace`
  *    (size from lf_workspace_bytes), 256-byte aligned.
@@ -19,7 +21,9 @@
  *
  * Notation: X [M,K], W [N,K], A_i [r_i,K], B_i [N,r_i], S [M,R] = drop(X) A^T (1/(1-p) applied,
  * zero beyond rank_i and in padded rows), dS [M,R] = scale dY B, mask uint8 [M,K] keep-mask
- * (non-zero = keep), R = max rank rounded up to 16.
+ * (non-zero = keep), R = max rank rounded up to 16.  Wherever an entry point takes a keep-mask,
+ * mask == NULL means "no dropout" for the whole call: p of the routing is then ignored and
+ * nothing is rescaled by 1/(1-p).
  */
 #ifndef LORAFUSION_HIP_H
 #define LORAFUSION_HIP_H
@@ -37,6 +41,7 @@ extern "C" {
 #define LF_EWORKSPACE (-3)
 #define LF_ELAUNCH (-4)
 #define LF_ELIMIT (-5)
+#define LF_ESTATIC (-6)
 
 #define LF_BF16 0
 #define LF_F16 1
@@ -135,6 +140,24 @@ int lf_lora_bwd(const void* dY, const void* X, const void* W, const uint8_t* mas
                 const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
                 void* const* db_ptrs, void* dS_out, void* workspace, size_t ws_bytes, int M, int N, int K, int R,
                 const lf_routing* routing, int dtype, void* stream);
+
+/* lf_lora_bwd without a workspace argument, for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The fp32 partial sums of the rank-r passes go to a buffer of
+ * LF_STATIC_SCRATCH_BYTES that is part of the library's device image (one copy per GPU, held until
+ * the process ends); the call allocates and frees nothing.  A call that needs more than the buffer
+ * holds (lf_workspace_bytes(LF_OP_BWD, ...) > LF_STATIC_SCRATCH_BYTES) returns LF_ESTATIC and
+ * enqueues nothing.  All calls on one GPU share the buffer: calls that may overlap on one GPU
+ * (different streams, or several host threads) race -- serialise them.  Nothing in the buffer has
+ * to start at zero (every partial sum is written before it is read within the call), and its
+ * contents after a call are unspecified.  The first call on a device looks up the buffer's
+ * address, which loads the library's device code if no kernel of it has run there yet; make that
+ * call outside a graph capture.  Outputs are bit-identical to lf_lora_bwd's. */
+#define LF_STATIC_SCRATCH_BYTES (32u << 20)
+int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8_t* mask, const void* S,
+                       const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
+                       void* const* db_ptrs, void* dS_out, int M, int N, int K, int R, const lf_routing* routing,
+                       int dtype, void* stream);
 
 /* C = A op(B) (+bias): trans_b = 1: B is [N,K] (C = A B^T); trans_b = 0: B is [K,N].  The same
  * MFMA kernel as above without the LoRA term; used to time the plain base GEMMs.  tile_cfg

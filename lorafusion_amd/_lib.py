@@ -17,12 +17,13 @@ LIB_PATH = os.path.join(_HERE, "liblorafusion_hip.so")
 LF_BF16, LF_F16 = 0, 1
 LF_MAX_SEG = 32
 LF_OP_XA, LF_OP_DYS_DYB, LF_OP_DA, LF_OP_FWD, LF_OP_BWD, LF_OP_NF4_FWD, LF_OP_NF4_BWD = range(7)
-LF_OK, LF_EINVAL, LF_ESHAPE, LF_EWORKSPACE, LF_ELAUNCH, LF_ELIMIT = 0, -1, -2, -3, -4, -5
+LF_OK, LF_EINVAL, LF_ESHAPE, LF_EWORKSPACE, LF_ELAUNCH, LF_ELIMIT, LF_ESTATIC = 0, -1, -2, -3, -4, -5, -6
+LF_STATIC_SCRATCH_BYTES = 32 << 20
 
 EXPORTS = (
     "lf_version", "lf_strerror", "lf_workspace_bytes", "lf_lora_xa", "lf_lora_xw_sb", "lf_lora_dys_dyb",
     "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant", "lf_dropout_mask",
-    "lf_lora_xa_seeded", "lf_lora_fwd_seeded", "lf_nf4_lora_fwd", "lf_nf4_lora_bwd",
+    "lf_lora_xa_seeded", "lf_lora_fwd_seeded", "lf_nf4_lora_fwd", "lf_nf4_lora_bwd", "lf_lora_bwd_static",
 )
 
 
@@ -86,6 +87,7 @@ def lib() -> ctypes.CDLL:
     l.lf_lora_dyw_dsa.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, rp, i, vp]
     l.lf_lora_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, rp, i, vp]
     l.lf_lora_bwd.argtypes = [vp] * 12 + [sz, i, i, i, i, rp, i, vp]
+    l.lf_lora_bwd_static.argtypes = [vp] * 11 + [i, i, i, i, rp, i, vp]
     l.lf_gemm.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, vp]
     l.lf_nf4_dequant.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, i, i, i, vp]
     l.lf_dropout_mask.argtypes = [vp, i, i, ctypes.c_float, rp, ctypes.c_uint64, vp]

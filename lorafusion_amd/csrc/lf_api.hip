@@ -1,5 +1,6 @@
 // extern "C" entry points of liblorafusion_hip.so: argument checks, workspace carving, launches.
 #include "lf_common.h"
+#include <atomic>
 
 int lf_launch_nf4_dequant(const uint8_t*, const void*, const float*, const float*, const float*, void*, int64_t,
                           int, int, int, hipStream_t);
@@ -10,6 +11,27 @@ int lf_launch_dropout_mask(uint8_t*, int, int, float, const float*, int, uint64_
 size_t lf_xa_workspace(int, int, int, const LfSegTable&);
 size_t lf_dys_dyb_workspace(int, int, int, const LfSegTable&);
 size_t lf_da_workspace(int, int, int, const LfSegTable&);
+
+// Scratch of lf_lora_bwd_static: part of the device image, one copy per GPU at its own address.  In
+// host code the array's name is only a handle for hipGetSymbolAddress; kernels and launch code
+// receive the looked-up device address.
+static __device__ __align__(256) unsigned char scratch[LF_STATIC_SCRATCH_BYTES];
+static constexpr int kMaxDevices = 64;
+static std::atomic<void*> scratch_addr[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device (two threads that
+// race here store the same value).
+static int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return LF_ELAUNCH;
+  void* p = scratch_addr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return LF_ELAUNCH;
+    scratch_addr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return LF_OK;
+}
 
 namespace {
 
@@ -64,6 +86,7 @@ const char* lf_strerror(int code) {
     case LF_EWORKSPACE: return "workspace missing or too small (see lf_workspace_bytes)";
     case LF_ELAUNCH: return "HIP reported an error at kernel launch";
     case LF_ELIMIT: return "too many adapter segments in one call";
+    case LF_ESTATIC: return "the call needs more scratch than the library's static buffer holds (LF_STATIC_SCRATCH_BYTES); use the entry point with a workspace argument";
     default: return "unknown error code";
   }
 }
@@ -194,6 +217,24 @@ int lf_lora_bwd(const void* dY, const void* X, const void* W, const uint8_t* mas
   if (rc != LF_OK) return rc;
   if (dX) rc = lf_lora_dyw_dsa(dY, W, dS_out, a_ptrs, mask, dX, M, N, K, R, routing, dtype, stream);
   return rc;
+}
+
+int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8_t* mask, const void* S,
+                       const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
+                       void* const* db_ptrs, void* dS_out, int M, int N, int K, int R, const lf_routing* routing,
+                       int dtype, void* stream) {
+  LfSegTable t;
+  int rc = make_seg(routing, M, nullptr, nullptr, t);
+  if (rc != LF_OK) return rc;
+  if (M <= 0 || N <= 0 || K <= 0 || R <= 0) return LF_EINVAL;
+  const size_t a = lf_dys_dyb_workspace(M, N, R, t), b = lf_da_workspace(M, K, R, t);
+  const size_t need = align256(a > b ? a : b);
+  if (need > (size_t)LF_STATIC_SCRATCH_BYTES) return LF_ESTATIC;
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != LF_OK) return rc;
+  return lf_lora_bwd(dY, X, W, mask, S, a_ptrs, b_ptrs, dX, da_ptrs, db_ptrs, dS_out, ws, LF_STATIC_SCRATCH_BYTES, M, N, K,
+                     R, routing, dtype, stream);
 }
 
 int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int N, int K, int trans_b, int dtype,
