@@ -165,6 +165,15 @@ int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8
 int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int N, int K, int trans_b, int dtype,
             int tile_cfg, void* stream);
 
+/* Tile configuration of every later MFMA GEMM launch of this process that does not name one itself
+ * (the fused entry points, lf_gemm with tile_cfg = -1): 0..7 pins it, -1 (the initial state)
+ * returns to the library's own choice.  A process-wide setting meant for tests and tuning runs --
+ * parity of every tile shape at small sizes; the reference has the same kind of knob in the
+ * Triton autotune configs of its kernels (lorafusion/ops/triton_ops/config.py).  A launch whose
+ * shape the pinned configuration cannot take fails with LF_ESHAPE (7, the persistent 256x256
+ * kernel, needs M, N >= 256).  Returns LF_EINVAL outside -1..7. */
+int lf_set_tile_cfg(int tile_cfg);
+
 /* NF4 block dequantisation.  Stands in for dequantize_nf4_triton
  * (lorafusion/ops/triton_ops/dequantize_nf4.py:271-346).  packed: uint8 [n/2] (element 2i in the
  * high nibble of byte i); absmax: uint8 [n/blocksize] when blocksize2 > 0 (double quantised:

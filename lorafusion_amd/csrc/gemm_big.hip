@@ -1,0 +1,587 @@
+// Persistent 256x256-tile MFMA GEMM with the LoRA term seeded into the accumulator, for gfx950 (MI355X).
+//
+//   C[M,N] = A[M,K] * op(B) + mult * (L[M,R] * Rop) (+ bias)        (operands as in gemm_lora.hip)
+//
+// The large-shape instance of the kernels that stand in for fused_lora_xw_sb / fused_multi_lora_xw_sb
+// (lorafusion/ops/triton_ops/fused_lora_xw_sb.py:74-206, fused_multi_lora_xw_sb.py:66-218; the reference's
+// persistent forward is fused_lora_xw_sb_tma.py:314,351-357) and fused_lora_dyw_dsa / fused_multi_lora_dyw_dsa
+// (fused_lora_dyw_dsa.py:69-181, fused_multi_lora_dyw_dsa.py:60-185).
+//
+// Structure
+//  * One workgroup per CU (at most), four 64-lane waves, each owning a 128x128 sub-tile (8x8 blocks of
+//    16x16x32 MFMA, 256 accumulator registers).  One wave per SIMD: a K step of 32 costs 16 LDS fragment
+//    reads per wave for 64 MFMAs, a third less LDS traffic than eight waves of 128x64.
+//  * Persistent: workgroup b walks tiles b, b+G, b+2G, ... (G = workgroups launched).  The K loops of
+//    successive tiles form one software pipeline: while a tile's last K steps run, the first stages of
+//    the next tile are already on their way into LDS, and they land during the epilogue.
+//  * K advances in stages of 64 (128-byte rows: every 16-byte lane of a load instruction belongs to a
+//    whole cache line) through two LDS stages of 64 KB, filled by 16-byte direct-to-LDS buffer loads.
+//    Stage s+1 is loaded while stage s is consumed; one workgroup barrier per stage, placed between
+//    the two MFMA sub-steps (k 0-31, k 32-63) of a stage:
+//        sub-step 0: MFMAs on fragment set 0; LDS reads of set 1 (same stage, k 32-63)
+//        wait for this wave's loads of the next stage, barrier  (next stage visible, current stage dead)
+//        sub-step 1: MFMAs on set 1; LDS reads of set 0 of the next stage; 16 tile loads of the stage
+//                    after next into the dead stage, one every four MFMAs (the texture addresser takes
+//                    16 cycles per 64-lane 16-byte load, and four waves issue in lockstep)
+//    All memory instructions of the loop carry hand-placed s_waitcnt: fragment reads are inline assembly,
+//    because the compiler's own counter bookkeeping gives up across the loop edge and waits for reads
+//    and loads that were issued a few cycles earlier.
+//  * LDS rows are 128 bytes (8 granules); granule g of row r sits at slot g ^ ((r>>1)&7), applied on the
+//    global side of the direct load.  Fragment reads (ds_read_b128) are conflict free with it.  The NN
+//    operand (W read as [K,N]) is stored untransposed and unpermuted in 512-byte rows (a permuted fetch order
+//    measured twice as slow), two rows per load instruction with 32 bytes of padding after each pair, and
+//    read with ds_read_b64_tr_b16: the rows that lanes read together sit in different pairs, hence on
+//    different banks.
+//  * The LoRA product seeds the accumulator before a tile's K loop (its operands are requested before
+//    the previous tile's epilogue); the forward scale is folded into the 16-bit L fragments (exact for
+//    powers of two), the backward 1/(1-p) is applied in fp32 together with the keep-mask select.
+//  * Epilogue: 16-row bands of a wave's sub-tile go through 4 KB of LDS per wave (beside the two stages) and
+//    leave as 16-byte stores that cover whole 256-byte rows of the sub-tile.
+#include "lf_common.h"
+#include <type_traits>
+#include <utility>
+
+namespace {
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int STAGE_A = BM * BK * 2;
+// NN operand B [64 k-rows, 256 columns]: rows of 512 bytes stored in pairs (k-rows r and r+4: the 1024 bytes one wave
+// instruction of the direct load fills), 32 bytes of padding after every pair
+constexpr int PAIR_NN = 1024 + 32;
+template <bool NN> struct Lds {
+  static constexpr int STAGE_B = NN ? 32 * PAIR_NN : BN * BK * 2;
+  static constexpr int STAGE = STAGE_A + STAGE_B;
+  static constexpr int EP_OFF = 2 * STAGE, EP_WAVE = 4096, BYTES = EP_OFF + 4 * EP_WAVE;
+  static_assert(BYTES <= 160 * 1024, "two stages and the epilogue bands fit the LDS of a CU");
+};
+
+template <typename T> struct BigOp;
+// The MFMAs are inline assembly with the accumulator block constrained to the accumulation registers ("+a"): all 256
+// of them hold the tile for the whole kernel, and the register allocator can neither park accumulator blocks in
+// ordinary vector registers nor use accumulation registers as spill space for other values (both happened with the
+// builtin: copies between the two files inside the K loop).  The compiler's hazard recogniser does not look inside
+// inline assembly: the wait states between these MFMAs and compiler-generated code that touches the accumulator
+// (v_accvgpr_write before, v_accvgpr_read after) are the explicit s_nop of mfma_fence() below.
+template <> struct BigOp<__bf16> {
+  static __device__ __forceinline__ void mfma(lf_f32x4& c, lf_u32x4 a, lf_u32x4 b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t bits) { return __builtin_bit_cast(float, (uint32_t)bits << 16); }
+};
+template <> struct BigOp<_Float16> {
+  static __device__ __forceinline__ void mfma(lf_f32x4& c, lf_u32x4 a, lf_u32x4 b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+};
+
+// 24 wait states: more than any MFMA-to-VALU / VALU-to-MFMA distance the hardware asks for on an accumulator register
+__device__ __forceinline__ void mfma_fence() { asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); }
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+template <int N, typename F>
+__device__ __forceinline__ void sfor(F&& f) {
+  [&]<int... I>(std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>{}), ...); }(std::make_integer_sequence<int, N>{});
+}
+
+#ifdef LF_BIG_TIMING
+__device__ unsigned long long lf_big_timing[8];  // cycles: seed, k loop, epilogue, wall (100 MHz), tiles
+#define LF_TICK(var) const long long var = __builtin_readcyclecounter()
+#else
+#define LF_TICK(var)
+#endif
+
+// LORA = false: the instance for calls without a LoRA term (the seed code is compiled out, which also keeps that
+// instance free of register spills: a kernel that needs scratch memory pays for it at every launch).
+template <typename T, bool NN, bool LORA>
+__global__ void __launch_bounds__(256, 1)
+gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (buffer-resource types are device-only)
+  using std::integral_constant;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int STAGE = Lds<NN>::STAGE, EP_OFF = Lds<NN>::EP_OFF, EP_WAVE = Lds<NN>::EP_WAVE;
+
+  const int total = p.grid_m * p.grid_n;
+  const int G = gridDim.x, wg = blockIdx.x;
+  const int n_my = (total - wg + G - 1) / G;
+  const int nk = p.K / BK;
+
+  // Tile `it` of this workgroup -> first row / column and the start of its K walk.  XCD-aware (workgroup ids that
+  // differ by a multiple of 8 share an XCD and its L2: they get neighbouring tiles), grouped 8 tile rows deep.  A tile
+  // that would cross the matrix edge is shifted inwards instead (M, N >= 256): it recomputes a few rows / columns of
+  // its neighbour -- identical values, since both walk K from the same start -- and no load or store needs a guard.
+  struct Tile { int m0, n0, kstart; };
+  auto tile_of = [&](int it) __attribute__((always_inline)) {
+    int pid = it * G + wg;
+    if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    constexpr int GROUP_M = 8;
+    const int width = GROUP_M * p.grid_n;
+    const int group = pid / width;
+    const int first_m = group * GROUP_M;
+    const int gsz = min(p.grid_m - first_m, GROUP_M);
+    const int pid_m = first_m + (pid % width) % gsz;
+    const int pid_n = (pid % width) / gsz;
+    Tile t;
+    t.m0 = min(pid_m * BM, p.M - BM);
+    t.n0 = min(pid_n * BN, p.N - BN);
+    // tile columns that run side by side start one 128-byte step apart, so their loads spread over the memory
+    // channels; the tiles of one column stay aligned and share the lines of their B panel in L2.  A shifted last
+    // column starts where the column it overlaps starts.
+    const int kcol = (pid_n == p.grid_n - 1 && p.N % BN != 0 && pid_n > 0) ? pid_n - 1 : pid_n;
+    t.kstart = (kcol & 15) % nk;
+    return t;
+  };
+
+  // ---------------------------------------------------------------- tile loads
+  // Direct-to-LDS loads: one wave instruction fills 1024 contiguous LDS bytes.  Operands with K-contiguous rows
+  // (A; B of the NT product): 8 rows of 128 B, lane -> (row tid>>3, slot tid&7) fetches granule slot ^ ((row>>1)&7);
+  // load i of an operand covers rows i*32 .. i*32+31 (a scalar offset).  NN operand B [K,N]: wave w, load i fills
+  // the pair of k-rows 8i+w (lanes 0-31) and 8i+w+4 (lanes 32-63), 512 contiguous bytes each, unpermuted.
+  uint32_t a_voff, b_voff;
+  {
+    const int lrow = tid >> 3, lg = tid & 7;
+    const int srcg = lg ^ ((lrow >> 1) & 7);
+    a_voff = (uint32_t)((int64_t)lrow * p.lda * 2 + srcg * 16);
+    if constexpr (!NN) {
+      b_voff = (uint32_t)((int64_t)lrow * p.ldb * 2 + srcg * 16);
+    } else {
+      b_voff = (uint32_t)((int64_t)(wave + 4 * (lane >> 5)) * p.ldb * 2 + (lane & 31) * 16);
+    }
+  }
+  const int a_istride = 32 * (int)p.lda * 2;
+  const int b_istride = NN ? 8 * (int)p.ldb * 2 : 32 * (int)p.ldb * 2;
+  // A wave issues one instruction per four cycles: behind every MFMA (16 cycles) there is room for three others.  The
+  // loop therefore keeps scalar work per load to one instruction where the loads are issued: the buffer descriptors
+  // of a tile sit in scalar registers, the scalar offsets of a stage's 16 loads are prepared one per MFMA during the
+  // previous sub-step, and M0 (the LDS destination of a direct load) is written one MFMA ahead of its load, which also
+  // covers the wait state between the two.
+  struct LoadSrc { lf_u32x4 ra, rb; int kstart; };
+  auto src_of = [&](const Tile& t) __attribute__((always_inline)) {
+    const char* a_base = (const char*)p.A + (int64_t)t.m0 * p.lda * 2;
+    const char* b_base = NN ? (const char*)p.B + (int64_t)t.n0 * 2 : (const char*)p.B + (int64_t)t.n0 * p.ldb * 2;
+    LoadSrc s;
+    s.ra = lf_u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)a_base),
+                    (uint32_t)__builtin_amdgcn_readfirstlane((int)((uintptr_t)a_base >> 32)) & 0xffffu, 0x7fffffffu, 0x00020000u};
+    s.rb = lf_u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)b_base),
+                    (uint32_t)__builtin_amdgcn_readfirstlane((int)((uintptr_t)b_base >> 32)) & 0xffffu, 0x7fffffffu, 0x00020000u};
+    s.kstart = t.kstart;
+    return s;
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+  // LDS destination of load idx in stage 0: m0a / m0b + a compile-time offset
+  const uint32_t m0a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + wave * 1024));
+  const uint32_t m0b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + STAGE_A + wave * (NN ? PAIR_NN : 1024)));
+  constexpr int M0B_STEP = NN ? 4 * PAIR_NN : 4096;
+  int istr[16];  // scalar offset of load idx relative to the stage's first byte of its operand
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    istr[i] = __builtin_amdgcn_readfirstlane(i * a_istride);
+    istr[8 + i] = __builtin_amdgcn_readfirstlane(i * b_istride);
+  }
+  // Scalars the K loop uses come through an empty asm: the compiler then waits for the kernel-argument loads behind
+  // them here, once, instead of keeping a "scalar load may be pending" wait inside the loop, where it would also wait
+  // for the fragment reads in flight (which it cannot see).
+  int nk_s = nk, kb_mul = BK * (int)p.ldb * 2;
+  asm volatile("" : "+s"(nk_s), "+s"(kb_mul));
+#pragma unroll
+  for (int i = 0; i < 16; i++) asm volatile("" : "+s"(istr[i]));
+  // byte offsets (operand A, operand B) of K step k of a tile whose walk starts at kstart
+  auto kbase = [&](int kstart, int k, int& ka, int& kb) __attribute__((always_inline)) {
+    int kp = kstart + k;
+    kp = kp >= nk_s ? kp - nk_s : kp;
+    ka = kp * (BK * 2);
+    kb = NN ? kp * kb_mul : ka;
+  };
+  auto set_m0 = [&](uint32_t base, auto OFF) __attribute__((always_inline)) {
+    asm volatile("s_add_u32 m0, %0, %1" ::"s"(base), "n"(OFF.value) : "memory", "scc");
+  };
+  auto issue_load = [&](lf_u32x4 rsrc, uint32_t voff, int soff) __attribute__((always_inline)) {
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  };
+  // all 16 loads of K step k of the tile behind `src` into stage `stage` (prologue only: no MFMAs to hide behind)
+  auto load_stage = [&](const LoadSrc& src, int k, int stage) __attribute__((always_inline)) {
+    int ka, kb;
+    kbase(src.kstart, k, ka, kb);
+    sfor<16>([&](auto I) {
+      constexpr int idx = I.value;
+      if constexpr (idx < 8) set_m0(m0a + stage * STAGE, std::integral_constant<int, idx * 4096>{});
+      else set_m0(m0b + stage * STAGE, std::integral_constant<int, (idx - 8) * M0B_STEP>{});
+      asm volatile("s_nop 0" ::: "memory");
+      issue_load(idx < 8 ? src.ra : src.rb, idx < 8 ? a_voff : b_voff, (idx < 8 ? ka : kb) + istr[idx]);
+    });
+  };
+
+  auto lgkm0 = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
+  auto barrier = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    lgkm0();
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using S0 = integral_constant<int, 0>;
+  using S1 = integral_constant<int, 1>;
+  constexpr int RDS = 3;   // a fragment read every RDS MFMAs
+  const T* __restrict__ Lp = (const T*)p.L;
+  T* __restrict__ C = (T*)p.C;
+  const uint16_t* bias16 = (const uint16_t*)p.bias;
+
+  // the first two stages of the first tile
+  Tile tile = tile_of(0);
+  LoadSrc src = src_of(tile);
+  load_stage(src, 0, 0);
+  load_stage(src, nk > 1 ? 1 : 0, 1);
+
+  int par = 0;  // LDS stage of the current tile's K step 0 (tiles follow each other through the two stages without a gap)
+  for (int it = 0; it < n_my; it++) {
+    // everything below is scoped to one tile: fragments, accumulators and seed operands do not live across tiles
+    const Tile nxt_tile = it + 1 < n_my ? tile_of(it + 1) : tile;
+    const LoadSrc nxt_src = src_of(nxt_tile);
+    const int m0 = tile.m0, n0 = tile.n0;
+    const int wrow0 = m0 + wm * 128;
+
+    LF_TICK(tk0);
+#ifdef LF_BIG_TIMING
+    const long long tw0 = wall_clock64();
+#endif
+    lf_u32x4 fa[2][8], fb[2][8];
+    lf_f32x4 acc[8][8];
+    uint32_t fa_off[2], fb_off[2];  // fragment addresses: set after the seed, so they are not live across it
+    // one fragment read of sub-step KS of the stage at LDS byte offset `st`: idx < 8: A fragment idx; else B fragment idx-8
+    auto read_one = [&](auto SET, auto KS, uint32_t st, auto IDX) __attribute__((always_inline)) {
+      constexpr int idx = IDX.value, set = SET.value, ks = KS.value;
+      if constexpr (idx < 8) {
+        const uint32_t ad = fa_off[ks] + st;
+        lf_u32x4 tmp;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(tmp) : "v"(ad), "n"(idx * 2048) : "memory");
+        fa[set][idx] = tmp;
+      } else if constexpr (!NN) {
+        const uint32_t ad = fb_off[ks] + st;
+        lf_u32x4 tmp;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(tmp) : "v"(ad), "n"((idx - 8) * 2048) : "memory");
+        fb[set][idx - 8] = tmp;
+      } else {
+        const uint32_t ad = fb_off[0] + st;
+        lf_u32x2 lo, hi;
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(ad), "n"(ks * 16 * PAIR_NN + (idx - 8) * 32) : "memory");
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(ad), "n"(ks * 16 * PAIR_NN + (idx - 8) * 32 + 512) : "memory");
+        fb[set][idx - 8] = lf_u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
+    };
+    auto mfma_one = [&](int set, int m) __attribute__((always_inline)) {
+      const int i = m >> 3, j = m & 7;
+      BigOp<T>::mfma(acc[i][j], fb[set][j], fa[set][i]);
+    };
+
+    // ------------------------------------------------------------ LoRA seed: acc = mult * L Rop (masked), or zero
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        acc[i][j] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+        asm volatile("" : "+a"(acc[i][j]));  // zeroed in the accumulation registers themselves
+      }
+    if (LORA && p.L != nullptr) {
+      int sl = lane;
+      asm volatile("" : "+v"(sl));   // as in the epilogue: keep the seed's address arithmetic inside the tile loop
+      const int l16 = sl & 15, kg = sl >> 4;
+      const T* rp = (const T*)seg.ptr[0];
+      int rank = seg.rank[0];
+      // mult_mode 1 without a keep-mask means no dropout, whatever p says: the term is not rescaled
+      bool use_mask = p.mask != nullptr && p.mult_mode == 1 && seg.p > 0.f;
+      float mult = p.mult_mode == 0 ? seg.scale : (use_mask ? 1.f / (1.f - seg.p) : 1.f);
+      if (seg.table != nullptr) {
+        int blk = (p.row0 + wrow0) / seg.block_size_m;
+        blk = min(blk, seg.n_blocks - 1);
+        rank = seg.table[3 * blk + 0];
+        const int fbk = seg.table[3 * blk + 2];
+        int sidx = 0;
+        for (int i = 1; i < seg.n_seg; i++) sidx = (seg.first_block[i] == fbk) ? i : sidx;
+        rp = (const T*)seg.ptr[sidx];
+        if (p.mult_mode == 0) {
+          mult = seg.block_scale[blk];
+        } else {
+          const float pb = seg.block_p[blk];
+          use_mask = p.mask != nullptr && pb > 0.f;
+          mult = use_mask ? 1.f / (1.f - pb) : 1.f;
+        }
+      }
+      const __amdgpu_buffer_rsrc_t rsrcR = __builtin_amdgcn_make_buffer_rsrc((void*)rp, 0, 0x7fffffff, 0x00020000);
+      // one MFMA k-step covers 32 rank columns; lanes whose 8 columns lie beyond R (or the rank) feed zeros.  The work
+      // goes one 16-row block row at a time, with scheduling fences in between: few values are live at any point (a
+      // register spill anywhere in this kernel puts scratch reloads, and their waits, into the K loop).
+      for (int t = 0; t < (p.R + 31) / 32; t++) {
+        const int r0 = t * 32 + kg * 8;
+        lf_u32x4 rf[8];
+        if (t == 0) mfma_fence();  // the accumulator was just zeroed by vector instructions
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const int gn = n0 + wn * 128 + j * 16 + l16;
+          // branch-free: lanes beyond the rank read the first columns again and are zeroed by a select
+          const bool in_r = r0 < rank;
+          const int rc = in_r ? r0 : 0;
+          lf_u32x4 v;
+          if constexpr (!NN) {
+            v = *(const lf_u32x4*)(rp + (int64_t)gn * rank + rc);
+          } else {
+            // eight rows of one column of Rop [rank, N]: 16-bit buffer loads that share a per-lane offset
+            const uint32_t voff = (uint32_t)(((rc - t * 32) * p.N + gn) * 2);
+            uint32_t e[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) e[k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcR, voff, (t * 32 + k) * p.N * 2, 0);
+            v[0] = e[0] | (e[1] << 16); v[1] = e[2] | (e[3] << 16);
+            v[2] = e[4] | (e[5] << 16); v[3] = e[6] | (e[7] << 16);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+#pragma unroll
+          for (int d = 0; d < 4; d++) v[d] = in_r ? v[d] : 0u;
+          rf[j] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const int gm = wrow0 + i * 16 + l16;
+          const bool in_R = r0 < p.R;
+          lf_u32x4 v = *(const lf_u32x4*)(Lp + (int64_t)gm * p.R + (in_R ? r0 : 0));
+#pragma unroll
+          for (int d = 0; d < 4; d++) v[d] = in_R ? v[d] : 0u;
+          if (p.mult_mode == 0 && mult != 1.f) {
+            // the forward scale goes into the 16-bit L fragment (fp32 product, one rounding; exact for powers of two)
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+              v[d] = BigOp<T>::pack2(BigOp<T>::to_float((uint16_t)(v[d] & 0xffffu)) * mult, BigOp<T>::to_float((uint16_t)(v[d] >> 16)) * mult);
+          }
+          // The MFMAs are inline assembly, which the compiler's hazard recogniser does not see: a vector ALU result
+          // (the selects and the scaling above) needs wait states before an MFMA reads it.  The empty-bodied nop takes
+          // the operands as in/outs, so every instruction that produces them stays in front of it.
+          if (i == 0) {
+            asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]), "+v"(v));
+          } else {
+            asm volatile("s_nop 3" : "+v"(v));
+          }
+#pragma unroll
+          for (int j = 0; j < 8; j++) BigOp<T>::mfma(acc[i][j], rf[j], v);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      mfma_fence();
+      if (p.mult_mode == 1 && use_mask) {
+        // keep-mask select and 1/(1-p) in fp32, one block row at a time: a lane reads the four mask bytes of its four
+        // accumulator columns of every block (one dword each)
+        const uint8_t* mrow = p.mask + (int64_t)(wrow0 + l16) * p.ldmask + n0 + wn * 128 + kg * 4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          uint32_t mk[8];
+#pragma unroll
+          for (int j = 0; j < 8; j++) mk[j] = *(const uint32_t*)(mrow + (int64_t)(i * 16) * p.ldmask + j * 16);
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[i][j][e] = ((mk[j] >> (8 * e)) & 0xffu) ? acc[i][j][e] * mult : 0.f;
+            asm volatile("" : "+a"(acc[i][j]));  // back into the accumulation registers now, not at the next use
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        mfma_fence();
+      }
+    }
+
+    // ------------------------------------------------------------ fragment addresses
+    // A (and NT B): lane reads granule ks*4+kg of row l16 of a 16-row block; blocks are 2048 bytes apart.  Derived
+    // from an opaque copy of the lane id, every tile: four registers fewer live across the seed
+    {
+      int fl = lane;
+      asm volatile("" : "+v"(fl));
+      const int l16 = fl & 15, kg = fl >> 4;
+      const int key = (l16 >> 1) & 7;
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) fa_off[ks] = lds0 + (wm * 128 + l16) * 128 + (((ks * 4 + kg) ^ key) << 4);
+      if constexpr (!NN) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) fb_off[ks] = lds0 + STAGE_A + (wn * 128 + l16) * 128 + (((ks * 4 + kg) ^ key) << 4);
+      } else {
+        // ds_read_b64_tr_b16: within a 16-lane group, lane 4j+c addresses row j, columns 4c..4c+3 and receives column
+        // (lane&15), rows 0..3.  Group kg takes k-rows kg*8 + j4 (and +4: the other row of the pair, 512 bytes on);
+        // sub-step ks: +32 rows.  k-row r = 32 ks + 16 b4 + 8 b3 + 4 hh + j4 lives in pair j4 + 4 b3 + 8 (b4 + 2 ks): the
+        // eight rows that 32 lanes read together sit in eight pairs, whose paddings put them on different banks
+        const int j4 = l16 >> 2, c = l16 & 3;
+        fb_off[0] = lds0 + STAGE_A + (j4 + 4 * (kg & 1) + 8 * (kg >> 1)) * PAIR_NN + (wn * 128 + 4 * c) * 2;
+        fb_off[1] = fb_off[0];
+      }
+    }
+
+    // ------------------------------------------------------------ K loop
+    LF_TICK(tk1);
+    mfma_fence();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // both stages requested so far (and the seed operands) have landed
+    barrier();
+    {
+      const uint32_t st = par * STAGE;
+      sfor<16>([&](auto I) { read_one(S0{}, S0{}, st, integral_constant<int, (I.value + 8) & 15>{}); });
+    }
+    lgkm0();
+    LF_TICK(tk1b);
+    // K step s lives in stage (par + s) & 1.  Sub-step 1 of step s refills that stage with step s+2 of this tile; the
+    // last two steps prefetch the first two steps of the next tile instead (of this tile again when none follows:
+    // loads that nothing consumes keep the step body uniform).  Gap schedule of a step (one MFMA = one gap of three
+    // issue slots): sub-step 0: a fragment read every third gap, the scalar offset of one load of the coming stage
+    // every fourth; sub-step 1: a fragment read every third gap, M0 in gap 4i, load i in gap 4i+1.
+    auto k_step = [&](int s, const LoadSrc& ld, int lk) __attribute__((always_inline)) {
+      const int cs = (par + s) & 1;
+      const uint32_t cur = cs * STAGE, nxt = STAGE - cur;
+      int ka, kb;
+      kbase(ld.kstart, lk, ka, kb);
+      const uint32_t ma = m0a + cur, mb = m0b + cur;
+      int soff[16];
+      sfor<64>([&](auto MM) {
+        constexpr int m = MM.value;
+        if constexpr (m % RDS == 0 && m / RDS < 16) read_one(S1{}, S1{}, cur, integral_constant<int, (m / RDS + 8) & 15>{});
+        if constexpr (m % 4 == 2) soff[m / 4] = (m / 4 < 8 ? ka : kb) + istr[m / 4];
+        mfma_one(0, m);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads of step s+1 (issued a sub-step ago) have landed
+      barrier();
+      sfor<64>([&](auto MM) {
+        constexpr int m = MM.value;
+        if constexpr (m % RDS == 0 && m / RDS < 16) read_one(S0{}, S0{}, nxt, integral_constant<int, (m / RDS + 8) & 15>{});
+        if constexpr (m % 4 == 0) {
+          if constexpr (m / 4 < 8) set_m0(ma, integral_constant<int, (m / 4) * 4096>{});
+          else set_m0(mb, integral_constant<int, (m / 4 - 8) * M0B_STEP>{});
+        }
+        if constexpr (m % 4 == 1) issue_load(m / 4 < 8 ? ld.ra : ld.rb, m / 4 < 8 ? a_voff : b_voff, soff[m / 4]);
+        mfma_one(1, m);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+      lgkm0();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    {
+      int s = 0;
+      for (; s + 2 < nk; s++) k_step(s, src, s + 2);
+      for (; s < nk; s++) k_step(s, nxt_src, s + 2 - nk < nk ? s + 2 - nk : 0);
+    }
+    par = (par + nk) & 1;
+    mfma_fence();
+    LF_TICK(tk2);
+
+    // ------------------------------------------------------------ epilogue: bias, convert, 16-row bands through LDS
+    {
+      // lane-dependent addresses are derived from an opaque copy of the lane id: computed here, every tile, in a few
+      // instructions -- otherwise the compiler hoists a hundred address registers out of the tile loop and spills them
+      int ln = lane;
+      asm volatile("" : "+v"(ln));
+      const int e16 = ln & 15, ekg = ln >> 4;
+      const uint32_t ep_lds = lds0 + EP_OFF + wave * EP_WAVE;
+      lf_u32x2 bvp[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) bvp[j] = lf_u32x2{0u, 0u};
+      if (bias16 != nullptr) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) bvp[j] = *(const lf_u32x2*)(bias16 + n0 + wn * 128 + j * 16 + ekg * 4);
+      }
+      const int orow = ln >> 4, og = ln & 15;  // on the way out: 16 lanes per 256-byte row, 4 rows per instruction
+      T* crow = C + (int64_t)(wrow0 + orow) * p.ldc + n0 + wn * 128 + og * 8;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        // band = the 16 rows of accumulator block row i; band row r, granule g (16 bytes = 8 columns) at slot g ^ r
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const lf_f32x4 a = acc[i][j];
+          const float b0 = BigOp<T>::to_float((uint16_t)(bvp[j][0] & 0xffffu)), b1 = BigOp<T>::to_float((uint16_t)(bvp[j][0] >> 16));
+          const float b2 = BigOp<T>::to_float((uint16_t)(bvp[j][1] & 0xffffu)), b3 = BigOp<T>::to_float((uint16_t)(bvp[j][1] >> 16));
+          const lf_u32x2 o = {BigOp<T>::pack2(a[0] + b0, a[1] + b1), BigOp<T>::pack2(a[2] + b2, a[3] + b3)};
+          const int g = j * 2 + (ekg >> 1);
+          const uint32_t ad = ep_lds + e16 * 256 + ((g ^ e16) << 4) + (ekg & 1) * 8;
+          asm volatile("ds_write_b64 %0, %1" ::"v"(ad), "v"(o) : "memory");
+        }
+        lf_u32x4 v[4];
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+          const int row = rr * 4 + orow;
+          const uint32_t ad = ep_lds + row * 256 + ((og ^ row) << 4);
+          asm volatile("ds_read_b128 %0, %1" : "=v"(v[rr]) : "v"(ad) : "memory");
+        }
+        lgkm0();
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) *(lf_u32x4*)(crow + (int64_t)(i * 16 + rr * 4) * p.ldc) = v[rr];
+        __builtin_amdgcn_sched_barrier(0);  // one band at a time: the scheduler otherwise reads all 256 accumulators up front
+      }
+    }
+#ifdef LF_BIG_TIMING
+    if (tid == 0) {
+      const long long tk3 = __builtin_readcyclecounter();
+      atomicAdd(&lf_big_timing[0], (unsigned long long)(tk1 - tk0));
+      atomicAdd(&lf_big_timing[it == 0 ? 5 : 6], (unsigned long long)(tk1b - tk1));
+      atomicAdd(&lf_big_timing[1], (unsigned long long)(tk2 - tk1b));
+      atomicAdd(&lf_big_timing[2], (unsigned long long)(tk3 - tk2));
+      atomicAdd(&lf_big_timing[3], (unsigned long long)(wall_clock64() - tw0));
+      atomicAdd(&lf_big_timing[4], 1ull);
+    }
+#endif
+    tile = nxt_tile;
+    src = nxt_src;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last, unconsumed prefetches
+#endif
+}
+
+template <typename T, bool NN, bool LORA>
+int launch_big(LfGemmParams p, const LfSegTable& seg, int max_wgs, hipStream_t st) {
+  p.grid_m = (p.M + BM - 1) / BM;
+  p.grid_n = (p.N + BN - 1) / BN;
+  auto kern = gemm_big_kernel<T, NN, LORA>;
+  static LfLdsFlags lds_ok;
+  constexpr int SMEM_BYTES = Lds<NN>::BYTES;
+  if (!lf_allow_lds(kern, SMEM_BYTES, lds_ok)) return LF_ELAUNCH;
+  const long total = (long)p.grid_m * p.grid_n;
+  const int grid = (int)(total < max_wgs ? total : max_wgs);
+  return lf_launch(kern, dim3(grid), dim3(256), SMEM_BYTES, st, p, seg);
+}
+
+std::atomic<int> cu_count[64];
+
+}  // namespace
+
+// Compute units of the current device (one persistent workgroup each), looked up once per device.
+int lf_cu_count() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cu_count[dev].load(std::memory_order_acquire);
+  if (n <= 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cu_count[dev].store(n, std::memory_order_release);
+  }
+  return n;
+}
+
+int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, hipStream_t st) {
+  if (p.K % BK != 0 || p.M < BM || p.N < BN || p.N % 8 != 0) return LF_ESHAPE;  // edge tiles are shifted inwards
+  // a wave's 128 rows lie in one routing block, also in a shifted edge tile
+  if (seg.table != nullptr && (seg.block_size_m % 128 != 0 || p.M % 128 != 0)) return LF_ESHAPE;
+  if (p.mask != nullptr && p.N % 16 != 0) return LF_ESHAPE;
+  const int wgs = lf_cu_count();
+  const bool lora = p.L != nullptr;
+  if (dtype == LF_BF16) {
+    if (lora) return nn ? launch_big<__bf16, true, true>(p, seg, wgs, st) : launch_big<__bf16, false, true>(p, seg, wgs, st);
+    return nn ? launch_big<__bf16, true, false>(p, seg, wgs, st) : launch_big<__bf16, false, false>(p, seg, wgs, st);
+  }
+  if (dtype == LF_F16) {
+    if (lora) return nn ? launch_big<_Float16, true, true>(p, seg, wgs, st) : launch_big<_Float16, false, true>(p, seg, wgs, st);
+    return nn ? launch_big<_Float16, true, false>(p, seg, wgs, st) : launch_big<_Float16, false, false>(p, seg, wgs, st);
+  }
+  return LF_EINVAL;
+}

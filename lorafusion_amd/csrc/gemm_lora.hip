@@ -662,6 +662,7 @@ int launch_dtype(const LfGemmParams& p, const LfSegTable& seg, int cfg, hipStrea
 // round next_a + next_b * fill, where fill is the occupied fraction of the round's slots.
 struct TileCand { int cfg, bm, bn, slots; double lat0, first_b, next_a, next_b; };
 static const TileCand kCands[] = {
+    {7, 256, 256, 256, 70.0, 40.0, 50.0, 30.0},   // persistent, 4 waves of 128x128 (gemm_big.hip): rounds = tiles per workgroup
     {1, 256, 256, 256, 66.0, 50.0, 44.0, 60.0},   // 8 waves, 128x64 per wave
     {3, 128, 256, 256, 48.0, 28.0, 28.0, 38.0},   // 8 waves, 64x64 per wave
     {4, 128, 128, 512, 38.0, 47.0, 5.0, 70.0},    // 4 waves, two workgroups per CU
@@ -676,10 +677,11 @@ static double launch_cost(const TileCand& c, int M, int N) {
   if (full == 0) return c.lat0 + c.first_b * fill * fill;
   return c.lat0 + c.first_b + (full - 1) * (c.next_a + c.next_b) + (fill > 0 ? c.next_a + c.next_b * fill : 0.0);
 }
-static int choose_cfg(int M, int N, double* cost_out = nullptr) {
+static int choose_cfg(int M, int N, bool allow_big, double* cost_out = nullptr) {
   int best = 1;
   double best_cost = 1e30;
   for (const TileCand& c : kCands) {
+    if (c.cfg == 7 && (!allow_big || M < 256 || N < 256)) continue;
     const double cost = launch_cost(c, M, N);
     if (cost < best_cost) { best_cost = cost; best = c.cfg; }
   }
@@ -689,7 +691,7 @@ static int choose_cfg(int M, int N, double* cost_out = nullptr) {
 // Rows [0, m_main) in whole rounds of 256x256 tiles, the rest as a second launch with the tile
 // that spreads it best, when that beats one launch (a nearly empty last round of big tiles
 // costs a full tile time).  Returns m_main (0: single launch).
-static int choose_split(int M, int N, int* cfg_tail) {
+static int choose_split(int M, int N, bool allow_big, int* cfg_head, int* cfg_tail) {
   constexpr double kLaunch = 4.0;  // a second launch
   const int grid_n = (N + 255) / 256;
   if (grid_n > 256) return 0;
@@ -697,13 +699,23 @@ static int choose_split(int M, int N, int* cfg_tail) {
   const int m_main = (M / rows_per_round) * rows_per_round;
   if (m_main <= 0 || m_main >= M) return 0;
   double single, tail;
-  choose_cfg(M, N, &single);
-  *cfg_tail = choose_cfg(M - m_main, N, &tail);
-  const double split = launch_cost(kCands[0], m_main, N) + tail + kLaunch;
+  choose_cfg(M, N, allow_big, &single);
+  *cfg_tail = choose_cfg(M - m_main, N, allow_big, &tail);
+  const bool big = allow_big && N >= 256;
+  *cfg_head = big ? 7 : 1;
+  const double split = launch_cost(kCands[big ? 0 : 1], m_main, N) + tail + kLaunch;
   return split < single ? m_main : 0;
 }
 
+static std::atomic<int> pinned_cfg{-1};
+int lf_pin_tile_cfg(int cfg) {
+  if (cfg < -1 || cfg > 7) return LF_EINVAL;
+  pinned_cfg.store(cfg, std::memory_order_relaxed);
+  return LF_OK;
+}
+
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st) {
+  if (force_cfg < 0) force_cfg = pinned_cfg.load(std::memory_order_relaxed);
   if (p.M <= 0 || p.N <= 0 || p.K <= 0) return LF_EINVAL;
   if (p.K % 64 != 0 || p.N % 8 != 0 || p.N < 8) return LF_ESHAPE;
   // 16-byte output stores
@@ -715,15 +727,18 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
   if (256 * p.lda * 2 >= 0x7fffffffLL || (int64_t)(nn ? p.K : 256) * p.ldb * 2 >= 0x7fffffffLL) return LF_ESHAPE;
   if (seg.table != nullptr && (seg.block_size_m % 64 != 0)) return LF_ESHAPE;
   auto launch = [&](const LfGemmParams& q, int cfg) {
-    if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1)) cfg = 2;
+    if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1 || cfg == 7)) cfg = 2;
+    if (cfg == 7) return lf_launch_gemm_big(q, seg, nn, dtype, st);
     if (dtype == LF_BF16) return nn ? launch_dtype<__bf16, true>(q, seg, cfg, st) : launch_dtype<__bf16, false>(q, seg, cfg, st);
     if (dtype == LF_F16) return nn ? launch_dtype<_Float16, true>(q, seg, cfg, st) : launch_dtype<_Float16, false>(q, seg, cfg, st);
     return (int)LF_EINVAL;
   };
   if (force_cfg >= 0) return launch(p, force_cfg);
-  int cfg_tail = 1;
-  const int m_main = choose_split(p.M, p.N, &cfg_tail);
-  if (m_main == 0) return launch(p, choose_cfg(p.M, p.N));
+  // the persistent kernel shifts edge tiles inwards: a wave's 128 rows must stay inside one routing block
+  const bool allow_big = seg.table == nullptr || (seg.block_size_m % 128 == 0 && p.M % 128 == 0);
+  int cfg_head = 1, cfg_tail = 1;
+  const int m_main = choose_split(p.M, p.N, allow_big, &cfg_head, &cfg_tail);
+  if (m_main == 0) return launch(p, choose_cfg(p.M, p.N, allow_big));
   LfGemmParams head = p, tail = p;
   head.M = m_main;
   tail.M = p.M - m_main;
@@ -732,6 +747,6 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
   tail.C = (char*)p.C + (int64_t)m_main * p.ldc * 2;
   if (p.L != nullptr) tail.L = (const char*)p.L + (int64_t)m_main * p.R * 2;
   if (p.mask != nullptr) tail.mask = p.mask + (int64_t)m_main * p.ldmask;
-  const int rc = launch(head, 1);
+  const int rc = launch(head, cfg_head);
   return rc != LF_OK ? rc : launch(tail, cfg_tail);
 }

@@ -237,6 +237,8 @@ int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8
                      R, routing, dtype, stream);
 }
 
+int lf_set_tile_cfg(int tile_cfg) { return lf_pin_tile_cfg(tile_cfg); }
+
 int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int N, int K, int trans_b, int dtype,
             int tile_cfg, void* stream) {
   if (bad_dtype(dtype) || !A || !B || !C) return LF_EINVAL;

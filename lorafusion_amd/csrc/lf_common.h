@@ -54,6 +54,9 @@ struct LfGemmParams {
 
 // launchers (one per translation unit)
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st);
+int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, hipStream_t st);  // persistent 256x256 tiles
+int lf_cu_count();
+int lf_pin_tile_cfg(int cfg);  // -1: automatic choice
 
 // Raise a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's copy of
 // the function; one flag array per kernel instantiation; threads that race here repeat the same call).
