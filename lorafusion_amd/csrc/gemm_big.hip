@@ -320,82 +320,96 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         }
       }
       const __amdgpu_buffer_rsrc_t rsrcR = __builtin_amdgcn_make_buffer_rsrc((void*)rp, 0, 0x7fffffff, 0x00020000);
-      // one MFMA k-step covers 32 rank columns; lanes whose 8 columns lie beyond R (or the rank) feed zeros.  The work
-      // goes one 16-row block row at a time, with scheduling fences in between: few values are live at any point (a
-      // register spill anywhere in this kernel puts scratch reloads, and their waits, into the K loop).
-      for (int t = 0; t < (p.R + 31) / 32; t++) {
+      // Everything the seed reads is requested up front -- per chunk of 32 rank columns the 8 + 8 operand fragments
+      // and, together with the last chunk's, the keep-mask bytes of the wave's 128x128 block (one dword per
+      // accumulator block and lane) -- so that a tile pays the memory latency once per chunk, not once per block row.
+      // The K loop's fragment registers are still dead here, which is where the room comes from.
+      const bool sel = p.mult_mode == 1 && use_mask;
+      const int n_chunks = (p.R + 31) / 32;
+      // one MFMA k-step covers 32 rank columns; lanes whose 8 columns lie beyond R (or the rank) read the first
+      // columns again and are zeroed by a select (branch-free)
+      mfma_fence();  // the accumulator was just zeroed by vector instructions
+      auto chunk = [&](int t) __attribute__((always_inline)) {
         const int r0 = t * 32 + kg * 8;
-        lf_u32x4 rf[8];
-        if (t == 0) mfma_fence();  // the accumulator was just zeroed by vector instructions
+        const bool in_r = r0 < rank, in_R = r0 < p.R;
+        lf_u32x4 rf[8], lv[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
           const int gn = n0 + wn * 128 + j * 16 + l16;
-          // branch-free: lanes beyond the rank read the first columns again and are zeroed by a select
-          const bool in_r = r0 < rank;
           const int rc = in_r ? r0 : 0;
-          lf_u32x4 v;
           if constexpr (!NN) {
-            v = *(const lf_u32x4*)(rp + (int64_t)gn * rank + rc);
+            rf[j] = *(const lf_u32x4*)(rp + (int64_t)gn * rank + rc);
           } else {
             // eight rows of one column of Rop [rank, N]: 16-bit buffer loads that share a per-lane offset
             const uint32_t voff = (uint32_t)(((rc - t * 32) * p.N + gn) * 2);
             uint32_t e[8];
 #pragma unroll
             for (int k = 0; k < 8; k++) e[k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcR, voff, (t * 32 + k) * p.N * 2, 0);
-            v[0] = e[0] | (e[1] << 16); v[1] = e[2] | (e[3] << 16);
-            v[2] = e[4] | (e[5] << 16); v[3] = e[6] | (e[7] << 16);
-            __builtin_amdgcn_sched_barrier(0);
+            rf[j] = lf_u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
           }
-#pragma unroll
-          for (int d = 0; d < 4; d++) v[d] = in_r ? v[d] : 0u;
-          rf[j] = v;
         }
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-          const int gm = wrow0 + i * 16 + l16;
-          const bool in_R = r0 < p.R;
-          lf_u32x4 v = *(const lf_u32x4*)(Lp + (int64_t)gm * p.R + (in_R ? r0 : 0));
+        for (int i = 0; i < 8; i++) lv[i] = *(const lf_u32x4*)(Lp + (int64_t)(wrow0 + i * 16 + l16) * p.R + (in_R ? r0 : 0));
 #pragma unroll
-          for (int d = 0; d < 4; d++) v[d] = in_R ? v[d] : 0u;
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+          for (int d = 0; d < 4; d++) rf[j][d] = in_r ? rf[j][d] : 0u;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+#pragma unroll
+          for (int d = 0; d < 4; d++) lv[i][d] = in_R ? lv[i][d] : 0u;
           if (p.mult_mode == 0 && mult != 1.f) {
             // the forward scale goes into the 16-bit L fragment (fp32 product, one rounding; exact for powers of two)
 #pragma unroll
             for (int d = 0; d < 4; d++)
-              v[d] = BigOp<T>::pack2(BigOp<T>::to_float((uint16_t)(v[d] & 0xffffu)) * mult, BigOp<T>::to_float((uint16_t)(v[d] >> 16)) * mult);
+              lv[i][d] = BigOp<T>::pack2(BigOp<T>::to_float((uint16_t)(lv[i][d] & 0xffffu)) * mult, BigOp<T>::to_float((uint16_t)(lv[i][d] >> 16)) * mult);
           }
-          // The MFMAs are inline assembly, which the compiler's hazard recogniser does not see: a vector ALU result
-          // (the selects and the scaling above) needs wait states before an MFMA reads it.  The empty-bodied nop takes
-          // the operands as in/outs, so every instruction that produces them stays in front of it.
-          if (i == 0) {
-            asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]), "+v"(v));
-          } else {
-            asm volatile("s_nop 3" : "+v"(v));
-          }
-#pragma unroll
-          for (int j = 0; j < 8; j++) BigOp<T>::mfma(acc[i][j], rf[j], v);
-          __builtin_amdgcn_sched_barrier(0);
         }
+        // The MFMAs are inline assembly, which the compiler's hazard recogniser does not see: a vector ALU result
+        // (the selects and the scaling above) needs wait states before an MFMA reads it.  The nop takes the operands
+        // as in/outs, so every instruction that produces them stays in front of it and every MFMA behind.
+        asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
+                                 "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]));
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+          for (int j = 0; j < 8; j++) BigOp<T>::mfma(acc[i][j], rf[j], lv[i]);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      int t = 0;
+      for (; t + 1 < n_chunks; t++) chunk(t);
+      // A lane reads the four mask bytes of its four accumulator columns of every block.  The loads are issued
+      // whether or not a mask applies (without one: 64 times the first dword of L): defined under a condition and
+      // used under another, the 64 values are spilled one by one, each behind its own wait.
+      uint32_t mk[8][8];
+      {
+        const uint8_t* mrow = sel ? p.mask + (int64_t)(wrow0 + l16) * p.ldmask + n0 + wn * 128 + kg * 4 : (const uint8_t*)Lp;
+        const int64_t mstride = sel ? 16 * p.ldmask : 0;
+        const int jstride = sel ? 16 : 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+          for (int j = 0; j < 8; j++) mk[i][j] = *(const uint32_t*)(mrow + i * mstride + j * jstride);
       }
-      mfma_fence();
-      if (p.mult_mode == 1 && use_mask) {
-        // keep-mask select and 1/(1-p) in fp32, one block row at a time: a lane reads the four mask bytes of its four
-        // accumulator columns of every block (one dword each)
-        const uint8_t* mrow = p.mask + (int64_t)(wrow0 + l16) * p.ldmask + n0 + wn * 128 + kg * 4;
+      chunk(t);
+      if (sel) {
+        mfma_fence();
+        // keep-mask select and 1/(1-p) in fp32, one block row at a time
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-          uint32_t mk[8];
-#pragma unroll
-          for (int j = 0; j < 8; j++) mk[j] = *(const uint32_t*)(mrow + (int64_t)(i * 16) * p.ldmask + j * 16);
 #pragma unroll
           for (int j = 0; j < 8; j++) {
+            // a definition right in front of the use: the copies out of the accumulation registers cannot rise above
+            // it (without it, all 256 are read up front)
+            asm volatile("" : "+a"(acc[i][j]));
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc[i][j][e] = ((mk[j] >> (8 * e)) & 0xffu) ? acc[i][j][e] * mult : 0.f;
+            for (int e = 0; e < 4; e++) acc[i][j][e] = ((mk[i][j] >> (8 * e)) & 0xffu) ? acc[i][j][e] * mult : 0.f;
             asm volatile("" : "+a"(acc[i][j]));  // back into the accumulation registers now, not at the next use
           }
           __builtin_amdgcn_sched_barrier(0);
         }
-        mfma_fence();
       }
+      mfma_fence();
     }
 
     // ------------------------------------------------------------ fragment addresses
