@@ -10,8 +10,9 @@
  *    `lf_routing` and the `*_ptrs` arrays are HOST memory, read during the call only.
  *  - dtype: LF_BF16 or LF_F16 for all 16-bit tensors of a call; accumulation is fp32.
  *  - Return 0 on success, a negative LF_E* code otherwise (lf_strerror gives the text).  The
- *    library may be called from several host threads: the only state it keeps is set once per
- *    device and then only read (per-kernel LDS limits, the address of the static scratch buffer);
+ *    library may be called from several host threads: the state it keeps is set once per device
+ *    and then only read (per-kernel LDS limits, the compute-unit count, the address of the static
+ *    scratch buffer), plus the one process-wide test knob of lf_set_tile_cfg (an atomic int);
  *    lf_lora_bwd_static is the one entry point whose calls share memory (see there).
  *  - Work is enqueued on `stream` (a hipStream_t, passed as void*); nothing synchronises.
  *  - The library allocates nothing: scratch memory comes in through `workspace`
@@ -52,7 +53,11 @@ extern "C" {
  * and `p` apply to all M rows.  Multi-LoRA: the per-block tables built by
  * prepare_multi_lora_batch_info (lorafusion/ops/multi_lora.py:348-453): block_table[b] =
  * (rank, valid_rows, first_block_of_segment); segment s owns blocks
- * [seg_first_block[s], seg_first_block[s+1]) and M must equal n_blocks * block_size_m. */
+ * [seg_first_block[s], seg_first_block[s+1]) and M must equal n_blocks * block_size_m.
+ * One segment per adapter: dA_i / dB_i of a segment are written, not accumulated, so an adapter
+ * whose tokens sit in two separate row ranges of one call would keep the second range's gradient
+ * only -- pack each adapter's tokens contiguously, as prepare_multi_lora_batch_info's callers do
+ * (lorafusion/train/training_utils.py:1304-1334 sorts by adapter), or sum the two outputs. */
 typedef struct lf_routing {
   int32_t n_seg;
   int32_t block_size_m;

@@ -160,7 +160,7 @@ def make_dropout_mask(shape, p, seed: int | None, device, routing: "MultiRouting
     return mask
 
 
-def seeded_dropout(x: torch.Tensor, p: float, seed: int, *, store_mask: bool = True):
+def seeded_dropout(x: torch.Tensor, p: float, seed: int | None = None, *, store_mask: bool = True):
     """``(where(mask, x/(1-p), 0), mask)`` -- lorafusion/ops/triton_ops/dropout.py:71-93.
 
     Kept for API parity; the fused path never materialises the dropped tensor.  The mask comes
@@ -205,8 +205,8 @@ def blocked_seeded_dropout(x: torch.Tensor, block_to_dropout_p: torch.Tensor, bl
     return out, (mask if store_mask else None)
 
 
-def fused_dropout_matmul(x: torch.Tensor, a: torch.Tensor, dropout_p: float, seed: int | None = None, *,
-                         store_mask: bool = True, store_masked_scaled_x: bool = False,
+def fused_dropout_matmul(x: torch.Tensor, a: torch.Tensor, dropout_p: float, seed: int = 42, *,
+                         store_mask: bool = False, store_masked_scaled_x: bool = False,
                          dropout_mask: torch.Tensor | None = None):
     """``S = drop(x) @ a.T`` -- lorafusion/ops/triton_ops/fused_dropout_matmul.py:280-354.
 

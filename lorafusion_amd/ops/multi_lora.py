@@ -8,7 +8,8 @@ and is left out).
 Differences from the reference, all deliberate:
  * ``S`` is computed per row with the row's own adapter (the reference multiplies every token by
    every adapter, multi_lora.py:502) and always from the *dropped* input, as in the single path;
- * per-block ``alpha`` / ``p`` default to fp32 (the reference stores bf16, multi_lora.py:393-394);
+ * per-block ``alpha`` / ``p`` are stored in ``output_dtype`` (bf16 by default, multi_lora.py:355,393-394) and
+   widened to fp32 once per micro-batch, when the routing is built, not in every kernel;
  * heterogeneous dropout works (the reference's call raises TypeError, multi_lora.py:490-496);
  * any number of adapters up to 32 (the reference stops at 4);
  * padded rows of ``y`` hold the base GEMM (+bias) and padded rows of ``dx`` hold ``dy W``
@@ -61,6 +62,19 @@ class MultiLoRABatchInfo:
     def num_active_adapters(self) -> int:
         return len(set(self.lora_idx_list))
 
+    def routing(self, *, enable_dropout: bool) -> MultiRouting:
+        """The kernels' view of this micro-batch (fp32 copies of the per-block tables on the device plus
+        the host struct of segment bounds and ranks), built on first use and kept: every LoRA linear of
+        every layer that runs this micro-batch shares it, where the reference rebuilds its pointer lists in
+        every layer call (lorafusion/ops/multi_lora.py:519-523)."""
+        cache = self.__dict__.setdefault("_routing_cache", {})
+        key = bool(enable_dropout)
+        if key not in cache:
+            cache[key] = MultiRouting(self.padded_seq_len_list, self.lora_rank_list, self.block_to_lookup_table,
+                                      self.block_to_alpha, self.block_to_dropout_p, enable_dropout=key,
+                                      block_size_m=self.block_size_m)
+        return cache[key]
+
 
 def build_block_tables(seq_len_list, lora_rank_list, dropout_p_list, alpha_list, block_size_m):
     """Vectorised routing tables (numpy): returns (padded_seq_len_list, lookup int32 [nb,3],
@@ -97,22 +111,20 @@ def prepare_multi_lora_batch_info(
     dropout_p_list: list[float],
     alpha_list: list[float],
     block_size_m: int,
-    output_dtype: torch.dtype = torch.float32,
+    output_dtype: torch.dtype = torch.bfloat16,
     micro_batch_info: Any | None = None,
     *,
     allow_empty_micro_batch_info: bool = False,
-    device: str | torch.device | None = None,
 ) -> MultiLoRABatchInfo:
     """Build the per-block tables of a packed batch (lorafusion/ops/multi_lora.py:348-453).
 
-    ``device`` defaults to ``"cuda"`` when a GPU is present (as in the reference) and to the CPU
-    otherwise, so the integer routing can be checked without a GPU.
+    The tensors live on ``"cuda"`` as in the reference (multi_lora.py:427-429); without a GPU they
+    stay on the CPU, so the integer routing can be checked there.
     """
     padded, lookup, block_p, block_alpha = build_block_tables(
         seq_len_list, lora_rank_list, dropout_p_list, alpha_list, block_size_m
     )
-    if device is None:
-        device = "cuda" if torch.cuda.is_available() else "cpu"
+    device = "cuda" if torch.cuda.is_available() else "cpu"
     same = all(p == dropout_p_list[0] for p in dropout_p_list)
     return MultiLoRABatchInfo(
         seq_len_list=seq_len_list,
@@ -137,8 +149,7 @@ def batch_info_from_micro_batch(
     micro_batch_info: Any,
     lora_configs: "Sequence[Any] | dict[int, Any]",
     block_size_m: int = FUSED_MULTI_LORA_BLOCK_SIZE_M,
-    output_dtype: torch.dtype = torch.float32,
-    device: str | torch.device | None = None,
+    output_dtype: torch.dtype = torch.bfloat16,
 ) -> MultiLoRABatchInfo:
     """Routing tables straight from a scheduler micro-batch descriptor.
 
@@ -172,7 +183,6 @@ def batch_info_from_micro_batch(
         block_size_m=block_size_m,
         output_dtype=output_dtype,
         micro_batch_info=micro_batch_info,
-        device=device,
     )
     padded_pairs = getattr(micro_batch_info, "padded_adapter_num_tokens_pairs", None)
     if padded_pairs is not None:
@@ -300,6 +310,7 @@ def fused_linear_multi_lora(
     dropout_mask: torch.Tensor | None = None,
     seed: int | None = None,
     quant_state=None,
+    routing: MultiRouting | None = None,
 ) -> torch.Tensor:
     """Fused multi-adapter LoRA linear (lorafusion/ops/multi_lora.py:762-830).
 
@@ -307,7 +318,9 @@ def fused_linear_multi_lora(
     ``[cur_i, cur_i + seq_len_list[i])`` with ``cur`` advancing by the padded lengths.
     ``dropout_mask`` / ``seed`` are extensions for reproducible runs.  With ``quant_state`` (the
     bitsandbytes-style state ``dequantize_nf4_triton`` takes) ``linear_w`` holds packed NF4 codes and
-    is dequantised inside the forward and backward calls.
+    is dequantised inside the forward and backward calls.  ``routing`` (extension) is the cached
+    ``MultiLoRABatchInfo.routing(...)`` of the micro-batch the table arguments come from; without it the same
+    object is built here, per call.
     """
     if len(lora_a_list) != len(lora_b_list):
         raise ValueError("lora_a_list and lora_b_list must have the same length")
@@ -320,8 +333,12 @@ def fused_linear_multi_lora(
     rank_list = [a.shape[0] for a in lora_a_list]
     if max(rank_list) > max_r:
         raise ValueError(f"max_r={max_r} is smaller than the largest adapter rank {max(rank_list)}")
-    routing = MultiRouting(padded_seq_len_list, rank_list, block_to_lookup_table, block_to_alpha,
-                           block_to_dropout_p, enable_dropout=enable_dropout)
+    if routing is None:
+        routing = MultiRouting(padded_seq_len_list, rank_list, block_to_lookup_table, block_to_alpha,
+                               block_to_dropout_p, enable_dropout=enable_dropout)
+    elif (routing.padded_seq_len_list != list(padded_seq_len_list) or routing.rank_list != rank_list
+          or routing.enable_dropout != bool(enable_dropout) or routing.table.data_ptr() != block_to_lookup_table.data_ptr()):
+        raise ValueError("routing does not belong to the batch tables passed with it")
     return FusedLinearMultiLoRA.apply(padded_x, linear_w, linear_bias, dropout_mask, seed, routing, quant_state,
                                       len(lora_a_list), *lora_a_list, *lora_b_list)
 
@@ -331,9 +348,11 @@ def fused_linear_multi_lora(
 multi_lora_manager: "MultiLoRAManager | None" = None
 
 
-def init_multi_lora_manager(lora_configs, num_pipeline_stages: int = 1,
-                            multi_lora_max_microbatch_tokens: int | None = None,
+def init_multi_lora_manager(lora_configs, num_pipeline_stages: int,
+                            multi_lora_max_microbatch_tokens: int | None,
                             multi_lora_global_batch_sizes: list[int] | None = None) -> "MultiLoRAManager":
+    """lorafusion/ops/multi_lora.py:40-57 (``multi_lora_global_batch_sizes`` has a default there too, and is
+    rejected when left at None, multi_lora.py:92-94)."""
     global multi_lora_manager
     if multi_lora_manager is not None:
         raise ValueError("Multi-LoRA manager has already been initialized")
@@ -359,14 +378,16 @@ class MultiLoRAManager:
     stepping (multi_lora.py:125-184) belong to the multi-GPU runtime and are not provided.
     """
 
-    def __init__(self, lora_configs, num_pipeline_stages: int = 1,
-                 multi_lora_max_microbatch_tokens: int | None = None,
+    def __init__(self, lora_configs, num_pipeline_stages: int,
+                 multi_lora_max_microbatch_tokens: int | None,
                  multi_lora_global_batch_sizes: list[int] | None = None) -> None:
         self.lora_configs = lora_configs
         self.num_pipeline_stages = num_pipeline_stages
         self.multi_lora_max_microbatch_tokens = multi_lora_max_microbatch_tokens
         self.multi_lora_global_batch_sizes = multi_lora_global_batch_sizes
-        if multi_lora_global_batch_sizes is not None and len(multi_lora_global_batch_sizes) != len(lora_configs):
+        if multi_lora_global_batch_sizes is None:
+            raise ValueError("multi_lora_global_batch_sizes is not provided")
+        if len(multi_lora_global_batch_sizes) != len(lora_configs):
             raise ValueError(f"Expected {len(lora_configs)} batch sizes, got {len(multi_lora_global_batch_sizes)}")
         self.adapter_sample_counts = dict.fromkeys(range(len(lora_configs)), 0)
         self.batch_info_deque: deque = deque(maxlen=num_pipeline_stages)
@@ -388,6 +409,9 @@ class MultiLoRAManager:
         batch_info.microbatch_idx = self.microbatch_idx
         self.microbatch_idx += 1
         self.batch_info_deque.append(batch_info)
+        if batch_info.block_to_lookup_table.is_cuda:
+            # once per micro-batch, here, instead of once per LoRA linear per layer
+            batch_info.routing(enable_dropout=batch_info.enable_dropout)
         micro = getattr(batch_info, "micro_batch_info", None)
         if micro is None:
             if batch_info.allow_empty_micro_batch_info:

@@ -81,7 +81,7 @@ def construct_ds_and_a_ptrs_list(raw_ds_list, raw_a_list, block_size_m, *, retur
     return construct_s_and_b_ptrs_list(raw_ds_list, raw_a_list, block_size_m, return_tensor_list=return_tensor_list)
 
 
-def fused_multi_lora_xw_sb(x, w, *, block_to_lookup_table, block_to_alpha, max_r, total_r=None, s_ptrs_list=None,
+def fused_multi_lora_xw_sb(x, w, *, block_to_lookup_table, block_to_alpha, max_r, total_r, s_ptrs_list=None,
                            b_ptrs_list=None, raw_s_list=None, raw_b_list=None, bias=None, init_zeros: bool = False,
                            block_size_m=None, config=None, **kwargs):
     """``y = x w^T + alpha_i * s_i b_i^T`` per adapter segment (fused_multi_lora_xw_sb.py:221-339).
@@ -99,7 +99,7 @@ def fused_multi_lora_xw_sb(x, w, *, block_to_lookup_table, block_to_alpha, max_r
     return hip_ops.fused_multi_lora_xw_sb(x, w, s_full, [b.contiguous() for b in b_list], routing, bias)
 
 
-def fused_multi_lora_dys_dyb(dy, block_to_lookup_table, block_to_alpha, max_r, total_r=None, s_ptrs_list=None,
+def fused_multi_lora_dys_dyb(dy, block_to_lookup_table, block_to_alpha, max_r, total_r, s_ptrs_list=None,
                              b_ptrs_list=None, raw_s_list=None, raw_b_list=None, *, block_size_m=None, config=None,
                              **kwargs):
     """``db_i = alpha_i dy_i^T s_i``, ``ds_i = alpha_i dy_i b_i`` (fused_multi_lora_dys_dyb.py:188-321).

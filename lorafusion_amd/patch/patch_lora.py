@@ -102,6 +102,7 @@ def lora_forward(model, x: torch.Tensor, *args, use_fused: bool = True, **kwargs
     weight = model.base_layer.weight
     qs = _nf4_state(weight)
     if use_fused:
+        enable_dropout = bool(model.training and info.enable_dropout)
         result = fused_linear_multi_lora(
             padded_x=x,
             linear_w=weight if qs is None else weight.detach().reshape(-1),
@@ -113,10 +114,11 @@ def lora_forward(model, x: torch.Tensor, *args, use_fused: bool = True, **kwargs
             block_to_lookup_table=info.block_to_lookup_table,
             block_to_dropout_p=info.block_to_dropout_p,
             block_to_alpha=info.block_to_alpha,
-            enable_dropout=model.training and info.enable_dropout,
+            enable_dropout=enable_dropout,
             same_dropout_p_value=info.same_dropout_p_value,
             max_r=info.max_r,
             linear_bias=linear_bias,
+            routing=info.routing(enable_dropout=enable_dropout),
         )
     else:
         result = torch_ref_linear_multi_lora(

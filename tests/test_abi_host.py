@@ -109,11 +109,16 @@ def test_manager_and_patch_host_logic():
     from lorafusion_amd.patch import patch_lora
 
     ml.reset_multi_lora_manager()
-    mgr = ml.init_multi_lora_manager([object(), object()], num_pipeline_stages=2)
+    with pytest.raises(ValueError, match="multi_lora_global_batch_sizes is not provided"):
+        ml.init_multi_lora_manager([object(), object()], 2, None)   # as lorafusion/ops/multi_lora.py:92-94
+    with pytest.raises(ValueError, match="Expected 2 batch sizes"):
+        ml.MultiLoRAManager([object(), object()], 2, None, [8])
+    assert ml.get_multi_lora_manager() is None
+    mgr = ml.init_multi_lora_manager([object(), object()], 2, None, [8, 8])
     with pytest.raises(ValueError):
-        ml.init_multi_lora_manager([object()], 1)
-    info_a = ml.prepare_multi_lora_batch_info([5], [0], [16], [0.0], [1.0], 128, device="cpu", allow_empty_micro_batch_info=True)
-    info_b = ml.prepare_multi_lora_batch_info([7], [1], [16], [0.0], [1.0], 128, device="cpu", allow_empty_micro_batch_info=True)
+        ml.init_multi_lora_manager([object()], 1, None, [8])
+    info_a = ml.prepare_multi_lora_batch_info([5], [0], [16], [0.0], [1.0], 128, allow_empty_micro_batch_info=True)
+    info_b = ml.prepare_multi_lora_batch_info([7], [1], [16], [0.0], [1.0], 128, allow_empty_micro_batch_info=True)
     mgr.add_batch_info(info_a)
     mgr.add_batch_info(info_b)
     with pytest.raises(ValueError):
@@ -125,7 +130,7 @@ def test_manager_and_patch_host_logic():
     assert mgr.pop_oldest_batch_info() is info_a
     mgr.mark_forward_pass_started()
     assert mgr.is_in_forward
-    strict = ml.prepare_multi_lora_batch_info([7], [1], [16], [0.0], [1.0], 128, device="cpu")
+    strict = ml.prepare_multi_lora_batch_info([7], [1], [16], [0.0], [1.0], 128)
     with pytest.raises(ValueError):
         mgr.add_batch_info(strict)   # MicroBatchInfo missing and not allowed to be empty
     ml.reset_multi_lora_manager()

@@ -94,7 +94,7 @@ def test_tier2_wrappers():
     x, w, a, b, dy, mask, bias = (d[k].cuda() for k in ("x", "w", "a", "b", "dy", "mask", "bias"))
     xt = lora_ref.dropout_explicit(d["x"].float(), d["mask"], p)
 
-    s, m_out, xs = T.fused_dropout_matmul(x, a, p, dropout_mask=mask, store_masked_scaled_x=True)
+    s, m_out, xs = T.fused_dropout_matmul(x, a, p, dropout_mask=mask, store_mask=True, store_masked_scaled_x=True)
     s_e = xt @ d["a"].float().T
     _close(s[:, :r], s_e, "fused_dropout_matmul s")
     assert torch.equal(m_out, mask)

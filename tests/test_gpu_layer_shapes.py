@@ -115,7 +115,7 @@ def _run_multi(tokens, K, N, ranks, p_list, scale_list, nf4=False, seed=0):
         start += pl
 
 
-@pytest.mark.parametrize("K,N", [(4096, 6144), (4096, 1024), (4096, 14336), (14336, 4096)])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (4096, 1024), (4096, 14336), (4096, 28672), (14336, 4096)])
 def test_8b_layer_projections(K, N):
     """16384 packed tokens, 4 adapters r=16, scales {1,2,2,4}, p {0,.05,.1,.1}."""
     _run_multi(16384, K, N, [16] * 4, [0.0, 0.05, 0.1, 0.1], [1.0, 2.0, 2.0, 4.0])

@@ -117,7 +117,7 @@ def test_multi_adapter_layer_through_manager(nf4):
     layer = FakeLoRALinear(w_dev, adapters, bias=d["bias"].cuda(), quant_state=qs).cuda()
 
     ml.reset_multi_lora_manager()
-    mgr = ml.init_multi_lora_manager([object()] * 4, num_pipeline_stages=1)
+    mgr = ml.init_multi_lora_manager([object()] * 4, 1, None, [1] * 4)
     try:
         info = ml.prepare_multi_lora_batch_info(seq, idx, ranks, p_list, scales, 128, allow_empty_micro_batch_info=True)
         assert info.padded_seq_len_list == d["padded"]

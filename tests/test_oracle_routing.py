@@ -65,12 +65,16 @@ def test_product_table_builder_bit_exact(seq, block):
     assert padded == exp_padded
     assert lookup.dtype == np.int32 and np.array_equal(lookup, exp_lookup)
     assert np.array_equal(bp, exp_p) and np.array_equal(ba, exp_a)
-    info = prepare_multi_lora_batch_info(seq, list(range(len(seq))), ranks, ps, alphas, block, device="cpu")
-    assert np.array_equal(info.block_to_lookup_table.numpy(), exp_lookup)
+    info = prepare_multi_lora_batch_info(seq, list(range(len(seq))), ranks, ps, alphas, block, output_dtype=torch.float32)
+    assert np.array_equal(info.block_to_lookup_table.cpu().numpy(), exp_lookup)
     assert info.block_to_lookup_table.dtype == torch.int32
     assert info.max_r == max_r and info.enable_dropout == en and info.same_dropout_p_value == same
     assert info.block_to_alpha.dtype == torch.float32
-    assert np.array_equal(info.block_to_alpha.numpy(), exp_a.astype(np.float32))
+    assert np.array_equal(info.block_to_alpha.cpu().numpy(), exp_a.astype(np.float32))
+    # the default storage type is the reference's (multi_lora.py:355)
+    info16 = prepare_multi_lora_batch_info(seq, list(range(len(seq))), ranks, ps, alphas, block)
+    assert info16.block_to_alpha.dtype == info16.block_to_dropout_p.dtype == torch.bfloat16
+    assert torch.equal(info16.block_to_alpha.cpu(), torch.from_numpy(exp_a).to(torch.bfloat16))
     assert info.num_active_adapters == len(seq)
 
 
@@ -78,13 +82,13 @@ def test_product_table_builder_errors_and_bf16_option():
     from lorafusion_amd.ops.multi_lora import prepare_multi_lora_batch_info
 
     with pytest.raises(ValueError):
-        prepare_multi_lora_batch_info([], [], [], [], [], 128, device="cpu")
+        prepare_multi_lora_batch_info([], [], [], [], [], 128)
     with pytest.raises(ValueError):
-        prepare_multi_lora_batch_info([0, 5], [0, 1], [16, 16], [0.0, 0.0], [1.0, 1.0], 128, device="cpu")
+        prepare_multi_lora_batch_info([0, 5], [0, 1], [16, 16], [0.0, 0.0], [1.0, 1.0], 128)
     with pytest.raises(ValueError):
-        prepare_multi_lora_batch_info([5], [0], [16, 16], [0.0], [1.0], 128, device="cpu")
+        prepare_multi_lora_batch_info([5], [0], [16, 16], [0.0], [1.0], 128)
     info = prepare_multi_lora_batch_info([100, 200], [3, 1], [16, 16], [0.1, 0.05], [2.0, 4.0], 128,
-                                         output_dtype=torch.bfloat16, device="cpu")
+                                         output_dtype=torch.bfloat16)
     # the reference's bf16 storage of p (multi_lora.py:393-394): 0.1 -> 0.10009765625
     assert info.block_to_dropout_p.dtype == torch.bfloat16
     assert float(info.block_to_dropout_p[0]) == 0.10009765625
@@ -106,17 +110,17 @@ def test_batch_info_from_micro_batch_descriptor():
         padded_adapter_num_tokens_pairs={a: ((n - 1) // 128 + 1) * 128 for a, n in tokens.items()},
         adapter_padding_multiple=128, is_empty_marker=False)
     cfgs = {a: SimpleNamespace(r=16 * (1 + a % 2), lora_dropout=0.05 * (a % 3), lora_alpha=16.0 + a) for a in tokens}
-    info = batch_info_from_micro_batch(mb, cfgs, device="cpu")
+    info = batch_info_from_micro_batch(mb, cfgs, output_dtype=torch.float32)
     assert info.lora_idx_list == [0, 3, 7] and info.seq_len_list == [130, 129, 128]
     padded, lookup, block_p, block_alpha, *_ = routing.block_tables([130, 129, 128], [16, 32, 32], [0.0, 0.0, 0.05],
                                                                     [16.0, 19.0, 23.0], 128)
     assert info.padded_seq_len_list == padded == [256, 256, 128]
-    assert np.array_equal(info.block_to_lookup_table.numpy(), lookup)
-    assert np.allclose(info.block_to_dropout_p.numpy(), block_p) and np.allclose(info.block_to_alpha.numpy(), block_alpha)
+    assert np.array_equal(info.block_to_lookup_table.cpu().numpy(), lookup)
+    assert np.allclose(info.block_to_dropout_p.cpu().numpy(), block_p) and np.allclose(info.block_to_alpha.cpu().numpy(), block_alpha)
     assert info.micro_batch_info is mb and info.max_r == 32
     # a descriptor padded to another multiple cannot drive 128-row kernels
     mb.adapter_padding_multiple = 64
     with pytest.raises(ValueError):
-        batch_info_from_micro_batch(mb, cfgs, device="cpu")
+        batch_info_from_micro_batch(mb, cfgs)
     with pytest.raises(ValueError):
-        batch_info_from_micro_batch(SimpleNamespace(is_empty_marker=True), cfgs, device="cpu")
+        batch_info_from_micro_batch(SimpleNamespace(is_empty_marker=True), cfgs)
