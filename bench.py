@@ -1,26 +1,34 @@
 #!/usr/bin/env python3
 """Benchmark of the fused LoRA-linear hot path on one MI355X.
 
-Workload (the configuration the headline metric is quoted on): the multi-LoRA packed batch --
-4 adapters of rank 16, scales {16,32,32,64}/16, dropout {0,.05,.1,.1}, lognormal(6.5, 0.8) token
-segments clipped to [64,4096] and packed to 8192 tokens, each adapter padded to 128 rows, shared
-base W[4096,4096] bf16, explicit seeded Bernoulli keep-mask, forward + backward (dX, dA_i, dB_i).
-One "step" = one fused forward + backward of that linear layer with all inputs resident in HBM.
+Headline workload (the configuration the metric names: "8B layer, r=16"): the seven LoRA projections of a
+Llama-3-8B-shaped decoder layer -- hidden 4096, kv 1024, MLP 14336 -- run the way the reference's layer runs
+them, as four LoRA linears (q/k/v merged into one N=6144 linear, gate/up merged into one N=28672 linear,
+lorafusion/patch/patch_transformers.py:50-163): 16384 packed tokens of 4 adapters (rank 16, multipliers
+{1,2,2,4}, dropout {0,.05,.1,.1}, lognormal segment lengths up to 8192), each adapter padded to 128 rows,
+bf16, training mode (dropout masks drawn in the rank-r pass), forward + backward (dX, dA_i, dB_i).  The
+micro-batch comes in as a scheduler descriptor, goes through the MultiLoRAManager, and every linear is
+called through the patched layer's forward.  Attention, rotary embedding, norms and the activation are not
+part of the path and not run.  One "step" = forward + backward of the four linears, inputs resident in HBM.
 
-Prints ONE JSON line.  `value` = algorithmic TFLOP/s of the whole step, counted on the 8192 real
-tokens: 2*(2MKN) + 6*M*r*(K+N).  `roofline` describes the dominant kernel (the MFMA GEMM of the
-backward, dX = dY W + LoRA term), timed live with HIP events on the launch stream.  `cpu_baseline`
-is the unfused PyTorch expression (the oracle's bf16 op-by-op arithmetic with autograd backward) on
-a bounded sample of the same workload on the host cores.
+Prints ONE JSON line.  `value` = algorithmic TFLOP/s of the step, counted on the 16384 real tokens:
+per linear 2*(2*M*K*N) + 6*M*r*(K+N).  `roofline` describes the dominant kernel of the step -- the persistent
+256x256-tile MFMA GEMM of the backward (dX = dY W + mask*(dS A)/(1-p)) -- over its four launches per step,
+each timed live with HIP events on the launch stream.  `cpu_baseline` is the unfused PyTorch expression
+(the oracle's bf16 op-by-op arithmetic with autograd backward) on the host cores.  `workloads` holds the
+reference's other configurations (c1 single linear, c2 packed multi-LoRA linear, c3 NF4 linear, c5 70B-class
+NF4 layer), each with its own roofline entry, and `nf4_dequant` the standalone dequant kernel against HBM peak.
 """
 
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
 import time
+from types import SimpleNamespace
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
@@ -30,13 +38,33 @@ import torch  # noqa: E402
 
 BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 HBM_PEAK_GBS = 8000.0
-
-K = N = 4096
-RANK = 16
-TOKENS = 8192
-SCALES = [1.0, 2.0, 2.0, 4.0]
-DROPOUT = [0.0, 0.05, 0.1, 0.1]
 BLOCK = 128
+METRIC = "fused LoRA fwd+bwd TFLOP/s (8B layer, r=16); NF4 dequant GB/s; % roofline"
+
+# (tokens, adapters, rank, multipliers, dropout, NF4 base weight, longest segment, [(linear, K, N)])
+WORKLOADS = {
+    "c1": (2048, 1, 16, [2.0], [0.1], False, 4096, [("linear", 4096, 4096)]),
+    "c2": (8192, 4, 16, [1.0, 2.0, 2.0, 4.0], [0.0, 0.05, 0.1, 0.1], False, 4096, [("linear", 4096, 4096)]),
+    "c3": (4096, 1, 16, [2.0], [0.0], True, 4096, [("linear", 4096, 14336)]),
+    "c4": (16384, 4, 16, [1.0, 2.0, 2.0, 4.0], [0.0, 0.05, 0.1, 0.1], False, 8192,
+           [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]),
+    "c5": (8192, 8, 64, [1.0, 2.0, 2.0, 4.0] * 2, [0.0, 0.05, 0.1, 0.1] * 2, True, 4096,
+           [("q", 8192, 8192), ("k", 8192, 1024), ("v", 8192, 1024), ("o", 8192, 8192),
+            ("gate", 8192, 28672), ("up", 8192, 28672), ("down", 28672, 8192)]),
+}
+NAMES = {
+    "c1": "single LoRA linear, 2048 tokens, K=N=4096, r=16, p=0.1, explicit mask, fwd+bwd",
+    "c2": "multi-LoRA packed batch: 4 adapters r=16, 8192 tokens (lognormal segments, seed 0), K=N=4096, fwd+bwd, "
+          "explicit dropout mask",
+    "c3": "NF4 QLoRA linear 4096 -> 14336, 4096 tokens, r=16, dequantisation inside the call, fwd+bwd",
+    "c4": "the seven LoRA projections of an 8B-class decoder layer (hidden 4096, kv 1024, MLP 14336) as the four LoRA "
+          "linears of the merged layer (qkv N=6144, o, gate+up N=28672, down), 16384 packed tokens, 4 adapters r=16, "
+          "training-mode dropout drawn in the rank-r pass, fwd+bwd, driven by a micro-batch descriptor through the "
+          "patched layer; attention, rotary embedding, norms and activation are not part of the path and not run",
+    "c5": "the seven LoRA linears of a 70B-class decoder layer (hidden 8192, kv 1024, MLP 28672) with NF4 base "
+          "weights (dequantised inside every call), 8192 packed tokens, 8 adapters r=64, explicit masks, fwd+bwd; "
+          "attention, norms and activation are not part of the path",
+}
 
 
 def segments(total_tokens: int, n_adapters: int, seed: int = 0, longest: int = 4096):
@@ -53,30 +81,8 @@ def segments(total_tokens: int, n_adapters: int, seed: int = 0, longest: int = 4
     return per
 
 
-def build_inputs(device, seq, dtype=torch.bfloat16):
-    g = torch.Generator().manual_seed(0)
-    padded = [((n - 1) // BLOCK + 1) * BLOCK for n in seq]
-    Mp = sum(padded)
-    x = torch.randn(Mp, K, generator=g).to(dtype)
-    w = (torch.randn(N, K, generator=g) * 0.02).to(dtype)
-    dy = torch.randn(Mp, N, generator=g).to(dtype)
-    a_list, b_list = [], []
-    for i in range(len(seq)):
-        ga = torch.Generator().manual_seed(10 + i)
-        a_list.append(((torch.rand(RANK, K, generator=ga) * 2 - 1) / K ** 0.5).to(dtype))
-        b_list.append((torch.randn(N, RANK, generator=ga) * 0.01).to(dtype))
-    gm = torch.Generator().manual_seed(1)
-    row_p = torch.cat([torch.full((pl,), p) for pl, p in zip(padded, DROPOUT)])
-    mask = torch.rand(Mp, K, generator=gm) >= row_p[:, None]
-    t = dict(x=x, w=w, dy=dy, a_list=a_list, b_list=b_list, mask=mask)
-    if device is not None:
-        t = {k: ([v.to(device) for v in val] if isinstance(val, list) else val.to(device)) for k, val in t.items()}
-    t["padded"] = padded
-    return t
-
-
-def step_flops(tokens: int) -> float:
-    return 2 * (2.0 * tokens * K * N) + 6.0 * tokens * RANK * (K + N)
+def linear_flops(tokens: int, k: int, n: int, rank: int) -> float:
+    return 2 * (2.0 * tokens * k * n) + 6.0 * tokens * rank * (k + n)
 
 
 def event_time_ms(fn, reps: int) -> float:
@@ -119,109 +125,343 @@ def graph_time_ms(fn, reps: int, inner: int = 10) -> float:
     return e0.elapsed_time(e1) / (n * inner)
 
 
-# The other benchmark configurations of the reference, as linear layers of the same fused path:
-# (tokens, adapters, rank, scales, dropout, NF4 base weight, longest segment, [(projection, K, N)]).
-LAYER_WORKLOADS = {
-    "c1": (2048, 1, 16, [2.0], [0.1], False, 4096, [("linear", 4096, 4096)]),
-    "c3": (4096, 1, 16, [2.0], [0.0], True, 4096, [("linear", 4096, 14336)]),
-    "c4": (16384, 4, 16, [1.0, 2.0, 2.0, 4.0], [0.0, 0.05, 0.1, 0.1], False, 8192,
-           [("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024), ("o", 4096, 4096),
-            ("gate", 4096, 14336), ("up", 4096, 14336), ("down", 14336, 4096)]),
-    "c5": (8192, 8, 64, [1.0, 2.0, 2.0, 4.0] * 2, [0.0, 0.05, 0.1, 0.1] * 2, True, 4096,
-           [("q", 8192, 8192), ("k", 8192, 1024), ("v", 8192, 1024), ("o", 8192, 8192),
-            ("gate", 8192, 28672), ("up", 8192, 28672), ("down", 28672, 8192)]),
-}
-LAYER_NAMES = {
-    "c1": "single LoRA linear, 2048 tokens, K=N=4096, r=16, p=0.1, explicit mask, fwd+bwd",
-    "c3": "NF4 QLoRA linear 4096 -> 14336, 4096 tokens, r=16, dequantisation inside the call, fwd+bwd",
-    "c4": "the seven LoRA linears of an 8B-class decoder layer (hidden 4096, kv 1024, MLP 14336), 16384 packed "
-          "tokens, 4 adapters r=16, fwd+bwd; attention, norms and activation are not part of the path",
-    "c5": "the seven LoRA linears of a 70B-class decoder layer (hidden 8192, kv 1024, MLP 28672) with NF4 base "
-          "weights, 8192 packed tokens, 8 adapters r=64, fwd+bwd; attention, norms and activation are not part of the path",
-}
+def wall_time_ms(fn, steps: int, warmup: int) -> float:
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
 
 
-def layer_workload(args, name: str) -> None:
-    """One of the reference's other configurations: every projection timed on its own (inputs of one
-    projection resident at a time), `value` = algorithmic flops of all projections / the sum of their times."""
-    from lorafusion_amd.ops import hip_ops
-    from lorafusion_amd.ops.multi_lora import prepare_multi_lora_batch_info
-    from lorafusion_amd.ops.nf4 import NF4WeightRef, quantize_nf4
+class Batch:
+    """Routing of one packed batch on the device (shared by all linears of a workload)."""
 
-    tokens, n_ad, rank, scales, drops, nf4, longest, projs = LAYER_WORKLOADS[name]
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    seq = segments(tokens, n_ad, longest=longest) if n_ad > 1 else [tokens]
-    info = prepare_multi_lora_batch_info(seq, list(range(n_ad)), [rank] * n_ad, drops, scales, BLOCK)
-    padded = info.padded_seq_len_list
-    Mp = sum(padded)
-    routing = hip_ops.MultiRouting(padded, [rank] * n_ad, info.block_to_lookup_table, info.block_to_alpha, info.block_to_dropout_p)
-    row_p = torch.cat([torch.full((pl,), float(p)) for pl, p in zip(padded, drops)]).to(dev)
-    g = torch.Generator(device=dev).manual_seed(0)
-    per_proj, total_ms, total_flops = {}, 0.0, 0.0
-    for pname, k, n in projs:
-        x = torch.randn(Mp, k, generator=g, device=dev).to(torch.bfloat16)
-        dy = torch.randn(Mp, n, generator=g, device=dev).to(torch.bfloat16)
+    def __init__(self, name: str, dev):
+        from lorafusion_amd.ops import hip_ops
+        from lorafusion_amd.ops.multi_lora import prepare_multi_lora_batch_info
+
+        self.tokens, self.n_ad, self.rank, self.scales, self.drops, self.nf4, longest, self.projs = WORKLOADS[name]
+        self.seq = segments(self.tokens, self.n_ad, longest=longest) if self.n_ad > 1 else [self.tokens]
+        self.info = prepare_multi_lora_batch_info(self.seq, list(range(self.n_ad)), [self.rank] * self.n_ad, self.drops,
+                                                  self.scales, BLOCK, output_dtype=torch.float32)
+        self.padded = self.info.padded_seq_len_list
+        self.Mp = sum(self.padded)
+        self.routing = hip_ops.MultiRouting(self.padded, [self.rank] * self.n_ad, self.info.block_to_lookup_table,
+                                            self.info.block_to_alpha, self.info.block_to_dropout_p)
+        self.row_p = torch.cat([torch.full((pl,), float(p)) for pl, p in zip(self.padded, self.drops)]).to(dev)
+        self.dropout = any(p > 0 for p in self.drops)
+
+    def head(self, rows: int):
+        """Routing of rows [0, rows) alone (rows is a multiple of the block size)."""
+        from lorafusion_amd.ops import hip_ops
+
+        nb = rows // BLOCK
+        pad, left = [], rows
+        for pl in self.padded:
+            take = min(pl, left)
+            if take > 0:
+                pad.append(take)
+            left -= take
+        return hip_ops.MultiRouting(pad, [self.rank] * len(pad), self.info.block_to_lookup_table[:nb].contiguous(),
+                                    self.info.block_to_alpha[:nb].contiguous(), self.info.block_to_dropout_p[:nb].contiguous())
+
+
+class Linear:
+    """Device tensors of one LoRA linear of a workload and its raw (autograd-free) forward + backward."""
+
+    def __init__(self, batch: Batch, name: str, k: int, n: int, g, dev):
+        from lorafusion_amd.ops.nf4 import NF4WeightRef, quantize_nf4
+
+        b = self.batch = batch
+        self.name, self.k, self.n = name, k, n
+        self.x = torch.randn(b.Mp, k, generator=g, device=dev).to(torch.bfloat16)
+        self.dy = torch.randn(b.Mp, n, generator=g, device=dev).to(torch.bfloat16)
         w = (torch.randn(n, k, generator=g, device=dev) * 0.02).to(torch.bfloat16)
-        a_l = [((torch.rand(rank, k, generator=g, device=dev) * 2 - 1) / k ** 0.5).to(torch.bfloat16) for _ in range(n_ad)]
-        b_l = [(torch.randn(n, rank, generator=g, device=dev) * 0.01).to(torch.bfloat16) for _ in range(n_ad)]
-        mask = (torch.rand(Mp, k, generator=g, device=dev) >= row_p[:, None]) if any(p > 0 for p in drops) else None
-        if nf4:
-            packed, qs = quantize_nf4(w.float())
-            wref = NF4WeightRef(packed, qs)
-            del w
-
-            def step():
-                y, s_ = hip_ops.nf4_lora_forward(x, wref, a_l, b_l, routing.c, routing.R, mask, None)
-                return y, hip_ops.nf4_lora_backward(dy, x, wref, a_l, b_l, s_, routing.c, routing.R, mask, [rank] * n_ad)
+        self.a = [((torch.rand(b.rank, k, generator=g, device=dev) * 2 - 1) / k ** 0.5).to(torch.bfloat16) for _ in range(b.n_ad)]
+        self.b = [(torch.randn(n, b.rank, generator=g, device=dev) * 0.01).to(torch.bfloat16) for _ in range(b.n_ad)]
+        self.mask = (torch.rand(b.Mp, k, generator=g, device=dev) >= b.row_p[:, None]) if b.dropout else None
+        self.wref = None
+        if b.nf4:
+            self.packed, self.qs = quantize_nf4(w.float())
+            self.wref = NF4WeightRef(self.packed, self.qs)
+            self.w = None
         else:
-            def step():
-                y, s_ = hip_ops.lora_forward(x, w, a_l, b_l, routing.c, routing.R, mask, None)
-                return y, hip_ops.lora_backward(dy, x, w, a_l, b_l, s_, routing.c, routing.R, mask, [rank] * n_ad)
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        flops = 2 * (2.0 * tokens * k * n) + 6.0 * tokens * rank * (k + n)
-        per_proj[pname] = {"K": k, "N": n, "ms": round(ms, 4), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1)}
-        total_ms += ms
-        total_flops += flops
-        del x, dy, mask, a_l, b_l, step
-        torch.cuda.empty_cache()
-    print(json.dumps({
-        "metric": "fused LoRA fwd+bwd TFLOP/s (8B layer, r=16); NF4 dequant GB/s; % roofline",
-        "value": round(total_flops / (total_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(total_ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": LAYER_NAMES[name], "tokens": tokens, "rows_launched": Mp, "rank": rank, "adapters": n_ad,
-                   "nf4_base": nf4, "seq_len_list": seq},
-        "projections": per_proj, "roofline": None, "cpu_baseline": None,
-    }))
+            self.w = w
+        self.flops = linear_flops(b.tokens, k, n, b.rank)
+
+    def step(self):
+        from lorafusion_amd.ops import hip_ops
+
+        r = self.batch.routing
+        ranks = [self.batch.rank] * self.batch.n_ad
+        if self.wref is not None:
+            y, s_ = hip_ops.nf4_lora_forward(self.x, self.wref, self.a, self.b, r.c, r.R, self.mask, None)
+            return y, hip_ops.nf4_lora_backward(self.dy, self.x, self.wref, self.a, self.b, s_, r.c, r.R, self.mask, ranks)
+        y, s_ = hip_ops.lora_forward(self.x, self.w, self.a, self.b, r.c, r.R, self.mask, None)
+        return y, hip_ops.lora_backward(self.dy, self.x, self.w, self.a, self.b, s_, r.c, r.R, self.mask, ranks)
+
+    def dense_weight(self):
+        from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
+
+        if self.w is not None:
+            return self.w
+        return dequantize_nf4_triton(self.packed, self.qs).reshape(self.n, self.k)
 
 
-def cpu_baseline(seq, budget_s: float = 15.0):
-    """Oracle (bf16 op-by-op, autograd backward) on the host cores: the whole 8192-token batch when one
-    run takes under a second (it does on the GPU box's host), else the first 256 tokens of every
-    adapter; as many runs as fit in about `budget_s` seconds (at least 3), median reported."""
+def gemm_plan(M: int, N: int, routed: bool):
+    from lorafusion_amd import _lib as L
+
+    rows, ch, ct = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    L.check(L.lib().lf_gemm_plan(M, N, BLOCK if routed else 0, ctypes.byref(rows), ctypes.byref(ch), ctypes.byref(ct)), "lf_gemm_plan")
+    return rows.value, ch.value, ct.value
+
+
+def kernel_breakdown(linears, reps: int):
+    """Per-kernel times of a workload's linears (summed over them) and the roofline entry of the dominant
+    kernel: the dX GEMM.  Where the library runs a row count as whole rounds of 256x256 tiles plus a short
+    second launch, the dominant launch is timed alone on its own rows (same grid, same data), so the figure is
+    one kernel's duration, comparable with a kernel trace."""
+    from lorafusion_amd.ops import hip_ops
+
+    t = dict(xa=0.0, gemm_fwd=0.0, dys_dyb=0.0, da=0.0, gemm_bwd=0.0, plain_gemm_nt=0.0, plain_gemm_nn=0.0)
+    dom_ms, dom_flops, launches, kinds = 0.0, 0.0, [], set()
+    for lin in linears:
+        b = lin.batch
+        r, w = b.routing, lin.dense_weight()
+        s = hip_ops.fused_multi_lora_xa(lin.x, lin.a, r, lin.mask)
+        _, ds = hip_ops.fused_multi_lora_dys_dyb(lin.dy, s, lin.b, r)
+        t["gemm_fwd"] += event_time_ms(lambda: hip_ops.fused_multi_lora_xw_sb(lin.x, w, s, lin.b, r), reps)
+        t["gemm_bwd"] += event_time_ms(lambda: hip_ops.fused_multi_lora_dyw_dsa(lin.dy, w, ds, lin.a, r, lin.mask), reps)
+        t["plain_gemm_nt"] += event_time_ms(lambda: hip_ops.gemm(lin.x, w, trans_b=True), reps)
+        t["plain_gemm_nn"] += event_time_ms(lambda: hip_ops.gemm(lin.dy, w, trans_b=False), reps)
+        t["xa"] += graph_time_ms(lambda: hip_ops.fused_multi_lora_xa(lin.x, lin.a, r, lin.mask), reps)
+        t["dys_dyb"] += graph_time_ms(lambda: hip_ops.fused_multi_lora_dys_dyb(lin.dy, s, lin.b, r), reps)
+        t["da"] += graph_time_ms(lambda: hip_ops.fused_multi_lora_da(lin.x, ds, r, lin.mask), reps)
+        # the dX GEMM's main launch: output [Mp, K], reduction over N
+        rows, cfg, _ = gemm_plan(b.Mp, lin.k, True)
+        if rows < b.Mp:
+            rh = b.head(rows)
+            nseg = len(rh.padded_seq_len_list)
+            dy_h, ds_h = lin.dy[:rows], ds[:rows]
+            mask_h = lin.mask[:rows] if lin.mask is not None else None
+            ms = event_time_ms(lambda: hip_ops.fused_multi_lora_dyw_dsa(dy_h, w, ds_h, lin.a[:nseg], rh, mask_h), reps)
+        else:
+            ms = event_time_ms(lambda: hip_ops.fused_multi_lora_dyw_dsa(lin.dy, w, ds, lin.a, r, lin.mask), reps)
+        fl = 2.0 * rows * lin.k * lin.n + 2.0 * rows * r.R * lin.k
+        dom_ms += ms
+        dom_flops += fl
+        kinds.add(cfg)
+        launches.append({"linear": lin.name, "rows": rows, "K_out": lin.k, "N_red": lin.n, "tile_cfg": cfg, "ms": round(ms, 4),
+                         "TFLOP/s": round(fl / (ms * 1e-3) / 1e12, 1)})
+        del w, s, ds
+    kern = ("gemm_big_kernel<bf16, NN, LoRA> (persistent 256x256 tiles)" if kinds == {7} else
+            "gemm_lora_kernel / gemm_big_kernel, NN (tile configurations %s)" % sorted(kinds))
+    achieved = dom_flops / (dom_ms * 1e-3) / 1e12
+    n = len(launches)
+    roofline = {
+        "bound": "mfma", "achieved": round(achieved, 2), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved / BF16_PEAK_TFLOPS, 4), "traffic": None, "traffic_source": None,
+        "kernel": kern + ": dX = dY W + mask*(dS A)/(1-p), main launch of each linear",
+        "launches_per_step": n, "launch_ms": round(dom_ms / n, 4), "flops_per_launch": dom_flops / n, "launches": launches,
+    }
+    t = {k: round(v, 4) for k, v in t.items()}
+    overhead = (t["xa"] + t["gemm_fwd"] + t["dys_dyb"] + t["da"] + t["gemm_bwd"]) / (t["plain_gemm_nt"] + t["plain_gemm_nn"]) - 1.0
+    return t, roofline, round(overhead, 4)
+
+
+def read_traffic(roofline: dict, fname: str) -> None:
+    """HBM-side bytes per launch of the dominant kernel from the committed counter summary (FETCH_SIZE /
+    WRITE_SIZE runs are separate rocprofv3 passes; the figure is not measured in this run)."""
+    path = os.path.join(ROOT, "profiles", fname)
+    if os.path.exists(path):
+        with open(path) as f:
+            for line in f:
+                if line.startswith("dominant_kernel_bytes_per_launch"):
+                    roofline["traffic"] = int(line.split()[1])
+                    roofline["traffic_source"] = f"profiles/{fname} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, separate runs)"
+
+
+def raw_workload(name: str, args, dev, breakdown: bool = True) -> dict:
+    """One of the reference's configurations through the raw ops: all linears resident, K steps of all of them."""
+    batch = Batch(name, dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    linears = [Linear(batch, pn, k, n, g, dev) for pn, k, n in batch.projs]
+
+    def step():
+        for lin in linears:
+            lin.step()
+
+    ms = wall_time_ms(step, args.steps, args.warmup)
+    flops = sum(lin.flops for lin in linears)
+    per = {}
+    for lin in linears:
+        pm = event_time_ms(lin.step, max(3, args.steps // 4))
+        per[lin.name] = {"K": lin.k, "N": lin.n, "ms": round(pm, 4), "TFLOP/s": round(lin.flops / (pm * 1e-3) / 1e12, 1)}
+    res = {
+        "workload": NAMES[name], "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 4),
+        "tokens": batch.tokens, "rows_launched": batch.Mp, "rank": batch.rank, "adapters": batch.n_ad, "nf4_base": batch.nf4,
+        "seq_len_list": batch.seq, "linears": per,
+    }
+    if breakdown:
+        res["kernels_ms"], res["roofline"], res["lora_overhead_vs_plain_gemms"] = kernel_breakdown(linears, 10)
+    if name == "c2" and breakdown:
+        from lorafusion_amd.ops import hip_ops
+
+        lin = linears[0]
+        r = batch.routing
+        read_traffic(res["roofline"], "bench_c2_hbm_traffic.txt")
+        res["kernels_ms"]["seeded_mask"] = round(graph_time_ms(
+            lambda: hip_ops.make_dropout_mask(lin.x.shape, None, 1234, dev, routing=r), 20), 4)
+        res["kernels_ms"]["fwd_seeded_xa_plus_gemm"] = round(event_time_ms(
+            lambda: hip_ops.lora_forward_seeded(lin.x, lin.w, lin.a, lin.b, r.c, r.R, 1234, None), 20), 4)
+        # the same forward + backward captured once as a HIP graph and replayed
+        side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            lin.step()
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                keep = lin.step()
+        torch.cuda.synchronize()
+        mg = wall_time_ms(graph.replay, args.steps, args.warmup)
+        del keep
+        res["hipgraph_replay"] = {"ms_per_step": round(mg, 4), "TFLOP/s": round(flops / (mg * 1e-3) / 1e12, 2)}
+    del linears
+    torch.cuda.empty_cache()
+    return res
+
+
+def nf4_dequant_block(dev) -> dict:
+    """Standalone NF4 dequant of W[14336,4096], blocksize 64, double quantised: 2.516 B/element."""
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton, quantize_nf4
+
+    wq = torch.randn(14336, 4096, device=dev) * 0.02
+    packed, qs = quantize_nf4(wq)
+    out = torch.empty(14336 * 4096, dtype=torch.bfloat16, device=dev)
+    t_op = event_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), 20)     # as called from Python
+    t_k = graph_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), 100)     # the kernel alone
+    n = 14336 * 4096
+    nbytes = n / 2 + n / 64 + 4 * n / 16384 + 1028 + 2 * n
+    gbs = nbytes / (t_k * 1e-3) / 1e9
+    return {"GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "launch_ms": round(t_k, 4),
+            "op_ms_from_python": round(t_op, 4), "bytes_per_launch": nbytes, "shape": [14336, 4096],
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "nf4_dequant_kernel"}}
+
+
+# --------------------------------------------------------------------------- the headline: the 8B layer
+
+def layer_c4(args, dev):
+    """The four merged LoRA linears of the 8B-class layer, called through the patched layer module with the
+    micro-batch registered at the MultiLoRAManager from a scheduler descriptor."""
+    from lorafusion_amd.ops import multi_lora as ml
+    from lorafusion_amd.patch.patch_transformers import DecoderLayerLoRAProjections
+
+    tokens, n_ad, rank, scales, drops, _, longest, projs = WORKLOADS["c4"]
+    seq = segments(tokens, n_ad, longest=longest)
+    # the reference's data provider hands lora_alpha to the kernels as the multiplier (training_utils.py:1323)
+    cfgs = [SimpleNamespace(r=rank, lora_alpha=s, lora_dropout=p) for s, p in zip(scales, drops)]
+    adapters = {f"lora_{i}": (c.r, c.lora_alpha, c.lora_dropout) for i, c in enumerate(cfgs)}
+    layer = DecoderLayerLoRAProjections.from_shapes(4096, 1024, 14336, adapters, device=dev, seed=0)
+    layer.train()
+    g = torch.Generator(device=dev).manual_seed(1)
+    with torch.no_grad():
+        for lin in layer.linears().values():
+            for nm in lin.lora_B:
+                lin.lora_B[nm].weight.copy_(torch.randn(lin.lora_B[nm].weight.shape, generator=g, device=dev) * 0.01)
+    mb = SimpleNamespace(
+        adapter_group_info=set(range(n_ad)), adapter_num_tokens_pairs=dict(enumerate(seq)),
+        padded_adapter_num_tokens_pairs={i: ((n - 1) // BLOCK + 1) * BLOCK for i, n in enumerate(seq)},
+        adapter_num_samples_pairs={i: 1 for i in range(n_ad)}, adapter_padding_multiple=BLOCK, is_empty_marker=False)
+    ml.reset_multi_lora_manager()
+    mgr = ml.init_multi_lora_manager(cfgs, 1, None, [1] * n_ad)
+    info = ml.batch_info_from_micro_batch(mb, cfgs)
+    mgr.add_batch_info(info)
+    Mp = sum(info.padded_seq_len_list)
+    lins = layer.linears()
+    io = {}
+    for name, k, n in projs:
+        x = torch.randn(1, Mp, k, generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
+        dy = torch.randn(1, Mp, n, generator=g, device=dev).to(torch.bfloat16)
+        io[name] = (x, dy)
+    params = [p for lin in lins.values() for p in lin.parameters() if p.requires_grad]
+
+    def step():
+        for name, lin in lins.items():
+            x, dy = io[name]
+            mgr.mark_forward_pass_started()
+            y = lin(x)
+            mgr.mark_backward_pass_started()
+            y.backward(dy)
+            x.grad = None
+        for p in params:
+            p.grad = None
+
+    ms = wall_time_ms(step, args.steps, args.warmup)
+    flops = sum(linear_flops(tokens, k, n, rank) for _, k, n in projs)
+    per = {}
+    for name, k, n in projs:
+        x, dy = io[name]
+
+        own = [p for p in lins[name].parameters() if p.requires_grad]
+
+        def one(lin=lins[name], x=x, dy=dy, own=own):
+            mgr.mark_forward_pass_started()
+            y = lin(x)
+            mgr.mark_backward_pass_started()
+            y.backward(dy)
+            x.grad = None
+            for p in own:
+                p.grad = None
+
+        pm = event_time_ms(one, max(3, args.steps // 4))
+        fl = linear_flops(tokens, k, n, rank)
+        per[name] = {"K": k, "N": n, "ms": round(pm, 4), "TFLOP/s": round(fl / (pm * 1e-3) / 1e12, 1)}
+    for p in params:
+        p.grad = None
+    ml.reset_multi_lora_manager()
+    del layer, io, lins, params
+    torch.cuda.empty_cache()
+    return ms, flops, seq, Mp, per
+
+
+def cpu_baseline_c4(budget_s: float = 20.0):
+    """Oracle (bf16 op-by-op, autograd backward) of the four linears on the host cores: the whole 16384-token
+    batch when three runs of it fit the budget (estimated from a 1024-token run), else 256 tokens per adapter;
+    median of at least 3 runs."""
     from oracle import lora_ref
 
+    tokens, n_ad, rank, scales, drops, _, longest, projs = WORKLOADS["c4"]
+    seq = segments(tokens, n_ad, longest=longest)
     cores = os.cpu_count() or 1
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
+
     def make(sample):
         sseq = [min(n, sample) for n in seq]
-        t = build_inputs(None, sseq)
+        padded = [((n - 1) // BLOCK + 1) * BLOCK for n in sseq]
+        Mp = sum(padded)
+        g = torch.Generator().manual_seed(0)
+        row_p = torch.cat([torch.full((pl,), float(p)) for pl, p in zip(padded, drops)])
+        data = []
+        for _, k, n in projs:
+            x = torch.randn(Mp, k, generator=g).to(torch.bfloat16)
+            w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16)
+            dy = torch.randn(Mp, n, generator=g).to(torch.bfloat16)
+            a = [((torch.rand(rank, k, generator=g) * 2 - 1) / k ** 0.5).to(torch.bfloat16) for _ in range(n_ad)]
+            b = [(torch.randn(n, rank, generator=g) * 0.01).to(torch.bfloat16) for _ in range(n_ad)]
+            mask = torch.rand(Mp, k, generator=g) >= row_p[:, None]
+            data.append((x, w, dy, a, b, mask))
 
         def one():
-            x = t["x"].clone().requires_grad_(True)
-            a = [v.clone().requires_grad_(True) for v in t["a_list"]]
-            b = [v.clone().requires_grad_(True) for v in t["b_list"]]
-            y = lora_ref.linear_multi_lora_bf16_opbyop(x, t["w"], a, b, sseq, t["padded"], SCALES, DROPOUT, t["mask"])
-            y.backward(t["dy"])
+            for x, w, dy, a, b, mask in data:
+                xr = x.clone().requires_grad_(True)
+                ar = [v.clone().requires_grad_(True) for v in a]
+                br = [v.clone().requires_grad_(True) for v in b]
+                y = lora_ref.linear_multi_lora_bf16_opbyop(xr, w, ar, br, sseq, padded, scales, drops, mask)
+                y.backward(dy)
 
         return sseq, one
 
@@ -231,7 +471,7 @@ def cpu_baseline(seq, budget_s: float = 15.0):
     one()
     small = time.perf_counter() - t0
     what = "256 tokens per adapter"
-    if small * (sum(seq) / sum(sseq)) < 1.0:  # the full batch fits the budget many times over
+    if 3 * small * (sum(seq) / sum(sseq)) < budget_s:
         sseq, one = make(max(seq))
         one()
         what = "the whole batch"
@@ -241,15 +481,13 @@ def cpu_baseline(seq, budget_s: float = 15.0):
         t0 = time.perf_counter()
         one()
         times.append(time.perf_counter() - t0)
-        if len(times) >= 200:
+        if len(times) >= 100:
             break
     med = sorted(times)[len(times) // 2]
+    fl = sum(linear_flops(sum(sseq), k, n, rank) for _, k, n in projs)
     return {
-        "value": step_flops(sum(sseq)) / med / 1e12,
-        "unit": "TFLOP/s",
-        "cores": cores,
-        "kind": "port",
-        "sample": f"{sum(sseq)} tokens ({what}) of the same multi-LoRA batch, bf16 op-by-op + autograd, "
+        "value": fl / med / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"{sum(sseq)} tokens ({what}) of the same four LoRA linears, bf16 op-by-op + autograd, "
                   f"median of {len(times)} runs over {time.perf_counter() - t_start:.0f} s, {med * 1e3:.1f} ms/run",
     }
 
@@ -257,12 +495,12 @@ def cpu_baseline(seq, budget_s: float = 15.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["c2", *LAYER_WORKLOADS], default="c2",
-                    help="c2 (default): the multi-LoRA packed batch the metric is quoted on; c1, c3, c4, c5: the "
-                         "reference's other configurations, one line with a per-projection breakdown and no roofline entry")
+    ap.add_argument("--no-extras", action="store_true", help="only the headline workload (c4), its roofline and the CPU baseline")
+    ap.add_argument("--only", choices=sorted(WORKLOADS), default=None,
+                    help="run one workload through the raw ops and print its entry alone (for profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -270,34 +508,8 @@ def main():
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (MI355X); none is visible.")
-
-    if args.workload != "c2":
-        return layer_workload(args, args.workload)
-
-    from lorafusion_amd.ops import hip_ops
-    from lorafusion_amd.ops.multi_lora import fused_linear_multi_lora, prepare_multi_lora_batch_info
-    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton, quantize_nf4
-
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    seq = segments(TOKENS, 4)
-    t = build_inputs(dev, seq)
-    info = prepare_multi_lora_batch_info(seq, [0, 1, 2, 3], [RANK] * 4, DROPOUT, SCALES, BLOCK)
-    x = t["x"].requires_grad_(True)
-    a_list = [a.requires_grad_(True) for a in t["a_list"]]
-    b_list = [b.requires_grad_(True) for b in t["b_list"]]
-    x3, dy3 = x.unsqueeze(0), t["dy"].unsqueeze(0)
-
-    def step():
-        y = fused_linear_multi_lora(
-            x3, t["w"], lora_a_list=a_list, lora_b_list=b_list, seq_len_list=seq,
-            padded_seq_len_list=info.padded_seq_len_list, block_to_lookup_table=info.block_to_lookup_table,
-            block_to_dropout_p=info.block_to_dropout_p, block_to_alpha=info.block_to_alpha,
-            enable_dropout=True, same_dropout_p_value=None, max_r=RANK, dropout_mask=t["mask"])
-        y.backward(dy3)
-        x.grad = None
-        for p in a_list + b_list:
-            p.grad = None
 
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -306,108 +518,16 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    value = step_flops(TOKENS) / (ms * 1e-3) / 1e12
+    if args.only is not None:
+        print(json.dumps({"metric": METRIC, **raw_workload(args.only, args, dev, breakdown=not args.no_extras)}))
+        return
 
-    # ---- the same forward + backward captured once as a HIP graph and replayed (what a training loop
-    # that captures its step gets: no host launch work, shorter gaps between the kernels)
-    routing_g = hip_ops.MultiRouting(info.padded_seq_len_list, [RANK] * 4, info.block_to_lookup_table,
-                                     info.block_to_alpha, info.block_to_dropout_p)
-    xg, ag, bg = x.detach(), [a.detach() for a in a_list], [b.detach() for b in b_list]
-
-    def raw_step():
-        y, s_ = hip_ops.lora_forward(xg, t["w"], ag, bg, routing_g.c, routing_g.R, t["mask"], None)
-        return y, hip_ops.lora_backward(t["dy"], xg, t["w"], ag, bg, s_, routing_g.c, routing_g.R, t["mask"], [RANK] * 4)
-
-    side = torch.cuda.Stream()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.stream(side):
-        raw_step()
-        side.synchronize()
-        with torch.cuda.graph(graph, stream=side):
-            graph_out = raw_step()
-    torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        graph.replay()
-    torch.cuda.synchronize()
-    ms_graph = (time.perf_counter() - t0) * 1e3 / args.steps
-    del graph_out
-
-    # ---- per-kernel timings with HIP events: the GEMMs as plain back-to-back launches, the short rank-r,
-    # mask and dequant kernels replayed from a graph (their wrappers take longer than they run)
-    routing = hip_ops.MultiRouting(info.padded_seq_len_list, [RANK] * 4, info.block_to_lookup_table,
-                                   info.block_to_alpha, info.block_to_dropout_p)
-    xd, wd, dyd, mask = x.detach(), t["w"], t["dy"], t["mask"]
-    ad = [a.detach() for a in a_list]
-    bd = [b.detach() for b in b_list]
-    s = hip_ops.fused_multi_lora_xa(xd, ad, routing, mask)
-    _, ds = hip_ops.fused_multi_lora_dys_dyb(dyd, s, bd, routing)
-    Mp = xd.shape[0]
-    reps = 20
-    t_fwd = event_time_ms(lambda: hip_ops.fused_multi_lora_xw_sb(xd, wd, s, bd, routing), reps)
-    t_bwd = event_time_ms(lambda: hip_ops.fused_multi_lora_dyw_dsa(dyd, wd, ds, ad, routing, mask), reps)
-    t_plain_nt = event_time_ms(lambda: hip_ops.gemm(xd, wd, trans_b=True), reps)
-    t_plain_nn = event_time_ms(lambda: hip_ops.gemm(dyd, wd, trans_b=False), reps)
-    t_xa = graph_time_ms(lambda: hip_ops.fused_multi_lora_xa(xd, ad, routing, mask), reps)
-    t_dys = graph_time_ms(lambda: hip_ops.fused_multi_lora_dys_dyb(dyd, s, bd, routing), reps)
-    t_da = graph_time_ms(lambda: hip_ops.fused_multi_lora_da(xd, ds, routing, mask), reps)
-    t_mask = graph_time_ms(lambda: hip_ops.make_dropout_mask(xd.shape, None, 1234, dev, routing=routing), reps)
-    t_fwd_seeded = event_time_ms(lambda: hip_ops.lora_forward_seeded(xd, wd, ad, bd, routing.c, routing.R, 1234, None), reps)
-    # ---- dominant kernel: the 256x256-tile MFMA GEMM of the dX path.  The library runs rows
-    # [0, 8192) of the 8448 in whole rounds of that tile and the last 256 rows as a second, small
-    # launch; the roofline entry times the big launch alone (same grid, same data: the first 64
-    # routing blocks) so that its duration is one kernel's, comparable with a kernel trace.
-    main_rows = (Mp // 4096) * 4096
-    nbm = main_rows // BLOCK
-    pad_main, left = [], main_rows
-    for pl in info.padded_seq_len_list:
-        take = min(pl, left)
-        if take > 0:
-            pad_main.append(take)
-        left -= take
-    routing_main = hip_ops.MultiRouting(pad_main, [RANK] * len(pad_main), info.block_to_lookup_table[:nbm].contiguous(),
-                                        info.block_to_alpha[:nbm].contiguous(), info.block_to_dropout_p[:nbm].contiguous())
-    dy_m, ds_m, mask_m = dyd[:main_rows], ds[:main_rows], mask[:main_rows]
-    ad_m = ad[:len(pad_main)]
-    dom_ms = event_time_ms(lambda: hip_ops.fused_multi_lora_dyw_dsa(dy_m, wd, ds_m, ad_m, routing_main, mask_m), reps)
-    dom_name = "gemm_lora_kernel<256x256 tile, NN> (dX = dY W + mask*(dS A)/(1-p)), rows [0, %d)" % main_rows
-    # algorithmic flops of that launch: 2*M*K*N dense + 2*M*r*N LoRA seed
-    gemm_flops = 2.0 * main_rows * K * N + 2.0 * main_rows * RANK * N
-    achieved = gemm_flops / (dom_ms * 1e-3) / 1e12
-
-    # ---- NF4 dequant (W[14336,4096], blocksize 64, double quantised): 2.516 B/element
-    wq = torch.randn(14336, 4096, device=dev) * 0.02
-    packed, qs = quantize_nf4(wq)
-    out = torch.empty(14336 * 4096, dtype=torch.bfloat16, device=dev)
-    t_nf4_op = event_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), reps)   # as called from Python
-    t_nf4 = graph_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), 5 * reps)   # the kernel alone
-    n = 14336 * 4096
-    nf4_bytes = n / 2 + n / 64 + 4 * n / 16384 + 1028 + 2 * n
-    nf4_gbs = nf4_bytes / (t_nf4 * 1e-3) / 1e9
-
-    # HBM-side bytes per launch of the dominant kernel: the figure of the committed counter summary
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "bench_c2_hbm_traffic.txt")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            for line in f:
-                if line.startswith("dominant_kernel_bytes_per_launch"):
-                    traffic = int(line.split()[1])
-
+    ms, flops, seq, Mp, per = layer_c4(args, dev)
+    raw = raw_workload("c4", args, dev)       # the same four linears through the raw ops, explicit masks: per-kernel times
+    read_traffic(raw["roofline"], "bench_c4_hbm_traffic.txt")
     res = {
-        "metric": "fused LoRA fwd+bwd TFLOP/s (8B layer, r=16); NF4 dequant GB/s; % roofline",
-        "value": round(value, 2),
+        "metric": METRIC,
+        "value": round(flops / (ms * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -418,32 +538,19 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {
-            "workload": "multi-LoRA packed batch: 4 adapters r=16, 8192 tokens (lognormal segments, seed 0) "
-                        f"padded to {Mp} rows, K=N=4096, fwd+bwd, explicit dropout mask",
-            "tokens": TOKENS, "rows_launched": Mp, "K": K, "N": N, "rank": RANK, "adapters": 4,
-            "seq_len_list": seq,
-        },
-        "roofline": {
-            "bound": "mfma", "achieved": round(achieved, 2), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(achieved / BF16_PEAK_TFLOPS, 4), "traffic": traffic,
-            "kernel": dom_name, "launch_ms": round(dom_ms, 4), "flops_per_launch": gemm_flops,
-        },
-        "kernels_ms": {
-            "xa": round(t_xa, 4), "gemm_fwd": round(t_fwd, 4), "dys_dyb": round(t_dys, 4), "da": round(t_da, 4),
-            "gemm_bwd": round(t_bwd, 4), "seeded_mask": round(t_mask, 4), "fwd_seeded_xa_plus_gemm": round(t_fwd_seeded, 4), "plain_gemm_nt": round(t_plain_nt, 4), "plain_gemm_nn": round(t_plain_nn, 4),
-        },
-        "hipgraph_replay": {"ms_per_step": round(ms_graph, 4),
-                            "TFLOP/s": round(step_flops(TOKENS) / (ms_graph * 1e-3) / 1e12, 2)},
-        "lora_overhead_vs_plain_gemms": round((t_xa + t_fwd + t_dys + t_da + t_bwd) / (t_plain_nt + t_plain_nn) - 1.0, 4),
-        "nf4_dequant": {
-            "GB/s": round(nf4_gbs, 1), "frac_of_hbm_peak": round(nf4_gbs / HBM_PEAK_GBS, 4),
-            "launch_ms": round(t_nf4, 4), "op_ms_from_python": round(t_nf4_op, 4), "bytes_per_launch": nf4_bytes,
-            "shape": [14336, 4096],
-        },
+        "config": {"workload": NAMES["c4"], "tokens": 16384, "rows_launched": Mp, "rank": 16, "adapters": 4,
+                   "seq_len_list": seq, "linears": per},
+        "roofline": raw["roofline"],
+        "kernels_ms": raw["kernels_ms"],
+        "lora_overhead_vs_plain_gemms": raw["lora_overhead_vs_plain_gemms"],
+        "raw_ops_explicit_mask": {"ms_per_step": raw["ms_per_step"], "TFLOP/s": raw["value"], "linears": raw["linears"]},
     }
+    if not args.no_extras:
+        res["nf4_dequant"] = nf4_dequant_block(dev)
+        small = argparse.Namespace(steps=max(5, args.steps // 2), warmup=max(2, args.warmup // 2))
+        res["workloads"] = {name: raw_workload(name, args if name == "c2" else small, dev) for name in ("c1", "c2", "c3", "c5")}
     if not args.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline(seq)
+        res["cpu_baseline"] = cpu_baseline_c4()
     print(json.dumps(res))
 
 

@@ -179,6 +179,13 @@ int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int 
  * kernel, needs M, N >= 256).  Returns LF_EINVAL outside -1..7. */
 int lf_set_tile_cfg(int tile_cfg);
 
+/* The launches the library makes for an M x N output (any K) when no configuration is pinned: rows
+ * [0, *rows_head) as one launch of tile configuration *cfg_head and, when *rows_head < M, the rest
+ * as a second launch of *cfg_tail (-1 when there is none).  routing_block_size_m: 0 for a
+ * single-adapter call, else the routing block size.  For benchmarks that time one kernel of a
+ * fused call on its own; no counterpart in the reference (Triton's autotuner picks there). */
+int lf_gemm_plan(int M, int N, int routing_block_size_m, int* rows_head, int* cfg_head, int* cfg_tail);
+
 /* NF4 block dequantisation.  Stands in for dequantize_nf4_triton
  * (lorafusion/ops/triton_ops/dequantize_nf4.py:271-346).  packed: uint8 [n/2] (element 2i in the
  * high nibble of byte i); absmax: uint8 [n/blocksize] when blocksize2 > 0 (double quantised:

@@ -23,7 +23,7 @@ LF_STATIC_SCRATCH_BYTES = 32 << 20
 EXPORTS = (
     "lf_version", "lf_strerror", "lf_workspace_bytes", "lf_lora_xa", "lf_lora_xw_sb", "lf_lora_dys_dyb",
     "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant", "lf_dropout_mask",
-    "lf_lora_xa_seeded", "lf_lora_fwd_seeded", "lf_nf4_lora_fwd", "lf_nf4_lora_bwd", "lf_lora_bwd_static", "lf_set_tile_cfg",
+    "lf_lora_xa_seeded", "lf_lora_fwd_seeded", "lf_nf4_lora_fwd", "lf_nf4_lora_bwd", "lf_lora_bwd_static", "lf_set_tile_cfg", "lf_gemm_plan",
 )
 
 
@@ -90,6 +90,7 @@ def lib() -> ctypes.CDLL:
     l.lf_lora_bwd_static.argtypes = [vp] * 11 + [i, i, i, i, rp, i, vp]
     l.lf_gemm.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, vp]
     l.lf_set_tile_cfg.argtypes = [i]
+    l.lf_gemm_plan.argtypes = [i, i, i, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
     l.lf_nf4_dequant.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, i, i, i, vp]
     l.lf_dropout_mask.argtypes = [vp, i, i, ctypes.c_float, rp, ctypes.c_uint64, vp]
     l.lf_lora_xa_seeded.argtypes = [vp, vp, vp, vp, i, i, i, rp, ctypes.c_uint64, i, vp]

@@ -714,6 +714,24 @@ int lf_pin_tile_cfg(int cfg) {
   return LF_OK;
 }
 
+// The launches lf_launch_gemm makes for an M x N product when no configuration is pinned: rows [0, *rows_head)
+// with *cfg_head and, when *rows_head < M, the remaining rows with *cfg_tail (-1 otherwise).
+void lf_plan_gemm(int M, int N, int routing_block, int* rows_head, int* cfg_head, int* cfg_tail) {
+  const bool allow_big = routing_block <= 0 || (routing_block % 128 == 0 && M % 128 == 0);
+  int ch = 1, ct = 1;
+  const int m_main = choose_split(M, N, allow_big, &ch, &ct);
+  auto demote = [&](int cfg) { return (routing_block > 0 && routing_block % 128 != 0 && (cfg == 0 || cfg == 1 || cfg == 7)) ? 2 : cfg; };
+  if (m_main == 0) {
+    *rows_head = M;
+    *cfg_head = demote(choose_cfg(M, N, allow_big));
+    *cfg_tail = -1;
+  } else {
+    *rows_head = m_main;
+    *cfg_head = demote(ch);
+    *cfg_tail = demote(ct);
+  }
+}
+
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st) {
   if (force_cfg < 0) force_cfg = pinned_cfg.load(std::memory_order_relaxed);
   if (p.M <= 0 || p.N <= 0 || p.K <= 0) return LF_EINVAL;
@@ -734,11 +752,9 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
     return (int)LF_EINVAL;
   };
   if (force_cfg >= 0) return launch(p, force_cfg);
-  // the persistent kernel shifts edge tiles inwards: a wave's 128 rows must stay inside one routing block
-  const bool allow_big = seg.table == nullptr || (seg.block_size_m % 128 == 0 && p.M % 128 == 0);
-  int cfg_head = 1, cfg_tail = 1;
-  const int m_main = choose_split(p.M, p.N, allow_big, &cfg_head, &cfg_tail);
-  if (m_main == 0) return launch(p, choose_cfg(p.M, p.N, allow_big));
+  int m_main = 0, cfg_head = 1, cfg_tail = -1;
+  lf_plan_gemm(p.M, p.N, seg.table != nullptr ? seg.block_size_m : 0, &m_main, &cfg_head, &cfg_tail);
+  if (cfg_tail < 0) return launch(p, cfg_head);
   LfGemmParams head = p, tail = p;
   head.M = m_main;
   tail.M = p.M - m_main;

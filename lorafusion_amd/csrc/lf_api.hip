@@ -239,6 +239,12 @@ int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8
 
 int lf_set_tile_cfg(int tile_cfg) { return lf_pin_tile_cfg(tile_cfg); }
 
+int lf_gemm_plan(int M, int N, int routing_block_size_m, int* rows_head, int* cfg_head, int* cfg_tail) {
+  if (M <= 0 || N <= 0 || rows_head == nullptr || cfg_head == nullptr || cfg_tail == nullptr) return LF_EINVAL;
+  lf_plan_gemm(M, N, routing_block_size_m, rows_head, cfg_head, cfg_tail);
+  return LF_OK;
+}
+
 int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int N, int K, int trans_b, int dtype,
             int tile_cfg, void* stream) {
   if (bad_dtype(dtype) || !A || !B || !C) return LF_EINVAL;

@@ -57,6 +57,7 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
 int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, hipStream_t st);  // persistent 256x256 tiles
 int lf_cu_count();
 int lf_pin_tile_cfg(int cfg);  // -1: automatic choice
+void lf_plan_gemm(int M, int N, int routing_block, int* rows_head, int* cfg_head, int* cfg_tail);
 
 // Raise a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's copy of
 // the function; one flag array per kernel instantiation; threads that race here repeat the same call).
