@@ -245,6 +245,38 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   load_stage(src, 0, 0);
   load_stage(src, nk > 1 ? 1 : 0, 1);
 
+  // Adapter of a wave's 128 rows: rank, skinny operand, multiplier, whether a keep-mask applies.  With a routing table
+  // these are two dependent scalar loads (table row, then the segment's pointer), so a tile's lookup is issued while
+  // the previous tile computes and costs a latency only for a workgroup's first tile.
+  struct Route { int rank; const T* rp; float mult; bool use_mask; };
+  auto route_of = [&](int wave_row0) __attribute__((always_inline)) {
+    Route r;
+    r.rp = (const T*)seg.ptr[0];
+    r.rank = seg.rank[0];
+    // mult_mode 1 without a keep-mask means no dropout, whatever p says: the term is not rescaled
+    r.use_mask = p.mask != nullptr && p.mult_mode == 1 && seg.p > 0.f;
+    r.mult = p.mult_mode == 0 ? seg.scale : (r.use_mask ? 1.f / (1.f - seg.p) : 1.f);
+    if (seg.table != nullptr) {
+      int blk = (p.row0 + wave_row0) / seg.block_size_m;
+      blk = min(blk, seg.n_blocks - 1);
+      r.rank = seg.table[3 * blk + 0];
+      const int fbk = seg.table[3 * blk + 2];
+      int sidx = 0;
+      for (int i = 1; i < seg.n_seg; i++) sidx = (seg.first_block[i] == fbk) ? i : sidx;
+      r.rp = (const T*)seg.ptr[sidx];
+      if (p.mult_mode == 0) {
+        r.mult = seg.block_scale[blk];
+      } else {
+        const float pb = seg.block_p[blk];
+        r.use_mask = p.mask != nullptr && pb > 0.f;
+        r.mult = r.use_mask ? 1.f / (1.f - pb) : 1.f;
+      }
+    }
+    return r;
+  };
+  Route route{};
+  if (LORA && p.L != nullptr) route = route_of(tile.m0 + wm * 128);
+
   int par = 0;  // LDS stage of the current tile's K step 0 (tiles follow each other through the two stages without a gap)
   for (int it = 0; it < n_my; it++) {
     // everything below is scoped to one tile: fragments, accumulators and seed operands do not live across tiles
@@ -298,27 +330,10 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       int sl = lane;
       asm volatile("" : "+v"(sl));   // as in the epilogue: keep the seed's address arithmetic inside the tile loop
       const int l16 = sl & 15, kg = sl >> 4;
-      const T* rp = (const T*)seg.ptr[0];
-      int rank = seg.rank[0];
-      // mult_mode 1 without a keep-mask means no dropout, whatever p says: the term is not rescaled
-      bool use_mask = p.mask != nullptr && p.mult_mode == 1 && seg.p > 0.f;
-      float mult = p.mult_mode == 0 ? seg.scale : (use_mask ? 1.f / (1.f - seg.p) : 1.f);
-      if (seg.table != nullptr) {
-        int blk = (p.row0 + wrow0) / seg.block_size_m;
-        blk = min(blk, seg.n_blocks - 1);
-        rank = seg.table[3 * blk + 0];
-        const int fbk = seg.table[3 * blk + 2];
-        int sidx = 0;
-        for (int i = 1; i < seg.n_seg; i++) sidx = (seg.first_block[i] == fbk) ? i : sidx;
-        rp = (const T*)seg.ptr[sidx];
-        if (p.mult_mode == 0) {
-          mult = seg.block_scale[blk];
-        } else {
-          const float pb = seg.block_p[blk];
-          use_mask = p.mask != nullptr && pb > 0.f;
-          mult = use_mask ? 1.f / (1.f - pb) : 1.f;
-        }
-      }
+      const T* rp = route.rp;
+      const int rank = route.rank;
+      const bool use_mask = route.use_mask;
+      const float mult = route.mult;
       const __amdgpu_buffer_rsrc_t rsrcR = __builtin_amdgcn_make_buffer_rsrc((void*)rp, 0, 0x7fffffff, 0x00020000);
       // Everything the seed reads is requested up front -- per chunk of 32 rank columns the 8 + 8 operand fragments
       // and, together with the last chunk's, the keep-mask bytes of the wave's 128x128 block (one dword per
@@ -410,6 +425,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         }
       }
       mfma_fence();
+      route = route_of(nxt_tile.m0 + wm * 128);  // in flight during this tile's K loop
     }
 
     // ------------------------------------------------------------ fragment addresses
