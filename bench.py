@@ -192,11 +192,16 @@ class Linear:
             self.w = w
         self.flops = linear_flops(b.tokens, k, n, b.rank)
 
-    def step(self):
+    def step(self, keep_dense: bool = False):
         from lorafusion_amd.ops import hip_ops
 
         r = self.batch.routing
         ranks = [self.batch.rank] * self.batch.n_ad
+        if self.wref is not None and keep_dense:
+            # the forward's dequantised weight handed to the backward: one dequantisation per step
+            y, s_, dense = hip_ops.nf4_lora_forward(self.x, self.wref, self.a, self.b, r.c, r.R, self.mask, None, keep_dense=True)
+            return y, hip_ops.nf4_lora_backward(self.dy, self.x, self.wref, self.a, self.b, s_, r.c, r.R, self.mask, ranks,
+                                                dense=dense)
         if self.wref is not None:
             y, s_ = hip_ops.nf4_lora_forward(self.x, self.wref, self.a, self.b, r.c, r.R, self.mask, None)
             return y, hip_ops.nf4_lora_backward(self.dy, self.x, self.wref, self.a, self.b, s_, r.c, r.R, self.mask, ranks)
@@ -305,6 +310,17 @@ def raw_workload(name: str, args, dev, breakdown: bool = True) -> dict:
         "tokens": batch.tokens, "rows_launched": batch.Mp, "rank": batch.rank, "adapters": batch.n_ad, "nf4_base": batch.nf4,
         "seq_len_list": batch.seq, "linears": per,
     }
+    if batch.nf4:
+        def step_keep():
+            for lin in linears:
+                lin.step(keep_dense=True)
+
+        mk = wall_time_ms(step_keep, args.steps, args.warmup)
+        res["reuse_dequantized_weight"] = {
+            "ms_per_step": round(mk, 4), "TFLOP/s": round(flops / (mk * 1e-3) / 1e12, 2),
+            "note": "the forward's dequantised weight is kept for the backward that follows it: one NF4 dequantisation per "
+                    "linear per step instead of two, 2*N*K bytes held in between (the headline figure of this entry "
+                    "dequantises in both calls and holds only the packed weight)"}
     if breakdown:
         res["kernels_ms"], res["roofline"], res["lora_overhead_vs_plain_gemms"] = kernel_breakdown(linears, 10)
     if name == "c2" and breakdown:

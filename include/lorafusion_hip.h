@@ -205,14 +205,22 @@ typedef struct lf_nf4_weight {
   const float* offset;    /* float32 [1] or NULL */
   int32_t blocksize;
   int32_t blocksize2;     /* 0: absmax is float32 (not nested) */
+  void* dense;            /* optional: caller-owned 16-bit [N,K] buffer, 256-byte aligned, or NULL */
+  int32_t dense_valid;    /* with `dense`: 0 = this call dequantises into it; 1 = it already holds the
+                             dequantised weight (of this call's dtype) and nothing is dequantised */
+  int32_t reserved;
 } lf_nf4_weight;
 
 /* QLoRA forward / backward: the base weight is stored as NF4, dequantised into the head of
  * `workspace` (2*N*K bytes, rounded up to 256) and fed to lf_lora_fwd / lf_lora_bwd, whose own
  * workspace follows it; sizes from lf_workspace_bytes(LF_OP_NF4_FWD / LF_OP_NF4_BWD, ...).  Stands
  * in for dequantize_nf4_triton followed by the fused LoRA linear, the flow the reference sketches
- * in lorafusion/ops/experimental/fused_quantized_nf4_lora_xw_sb_tma.py:280-428.  With dX == NULL
- * the backward needs no weight and dequantises nothing. */
+ * in lorafusion/ops/experimental/fused_quantized_nf4_lora_xw_sb_tma.py:280-428.
+ * With W->dense the dequantised weight lives in the caller's buffer instead: the forward fills it
+ * (dense_valid = 0) and a backward that follows while it is still live reuses it (dense_valid = 1)
+ * -- one dequantisation per step instead of two, for 2*N*K bytes held in between; the workspace
+ * is then that of lf_lora_fwd / lf_lora_bwd (LF_OP_FWD / LF_OP_BWD).  With dX == NULL the backward
+ * needs no weight: it dequantises nothing and its workspace is that of LF_OP_BWD. */
 int lf_nf4_lora_fwd(const void* X, const lf_nf4_weight* W, const void* bias, const uint8_t* mask,
                     const void* const* a_ptrs, const void* const* b_ptrs, void* Y, void* S_out, void* workspace,
                     size_t ws_bytes, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream);

@@ -56,6 +56,9 @@ class NF4Weight(ctypes.Structure):
         ("offset", ctypes.c_void_p),
         ("blocksize", ctypes.c_int32),
         ("blocksize2", ctypes.c_int32),
+        ("dense", ctypes.c_void_p),
+        ("dense_valid", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 

@@ -262,34 +262,52 @@ int lf_nf4_dequant(const uint8_t* packed, const void* absmax, const float* code2
                                out_dtype, (hipStream_t)stream);
 }
 
+// Where the dequantised weight of an NF4 call lives: the caller's W->dense, or the head of the workspace.
+static int nf4_dense(const lf_nf4_weight* W, bool needed, void* workspace, size_t ws_bytes, int N, int K, int dtype,
+                     hipStream_t st, const void** dense, size_t* head) {
+  *dense = nullptr;
+  *head = 0;
+  if (!needed) return LF_OK;
+  if (!W || N <= 0 || K <= 0) return LF_EINVAL;
+  void* dst = W->dense;
+  if (dst != nullptr) {
+    if (((uintptr_t)dst & 255) != 0) return LF_EINVAL;
+    *dense = dst;
+    if (W->dense_valid) return LF_OK;
+  } else {
+    *head = align256((size_t)N * K * 2);
+    if (!workspace || ws_bytes < *head || ((uintptr_t)workspace & 255) != 0) return LF_EWORKSPACE;
+    dst = workspace;
+    *dense = dst;
+  }
+  if (!W->packed || !W->absmax) return LF_EINVAL;
+  return lf_launch_nf4_dequant(W->packed, W->absmax, W->code2, W->absmax2, W->offset, dst, (int64_t)N * K, W->blocksize,
+                               W->blocksize2, dtype, st);
+}
+
 int lf_nf4_lora_fwd(const void* X, const lf_nf4_weight* W, const void* bias, const uint8_t* mask,
                     const void* const* a_ptrs, const void* const* b_ptrs, void* Y, void* S_out, void* workspace,
                     size_t ws_bytes, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
-  if (!W || !W->packed || !W->absmax || N <= 0 || K <= 0) return LF_EINVAL;
-  const size_t wbytes = align256((size_t)N * K * 2);
-  if (!workspace || ws_bytes < wbytes || ((uintptr_t)workspace & 255) != 0) return LF_EWORKSPACE;
-  int rc = lf_launch_nf4_dequant(W->packed, W->absmax, W->code2, W->absmax2, W->offset, workspace, (int64_t)N * K,
-                                 W->blocksize, W->blocksize2, dtype, (hipStream_t)stream);
+  if (bad_dtype(dtype)) return LF_EINVAL;
+  const void* dense;
+  size_t head;
+  int rc = nf4_dense(W, true, workspace, ws_bytes, N, K, dtype, (hipStream_t)stream, &dense, &head);
   if (rc != LF_OK) return rc;
-  return lf_lora_fwd(X, workspace, bias, mask, a_ptrs, b_ptrs, Y, S_out, (char*)workspace + wbytes, ws_bytes - wbytes,
-                     M, N, K, R, routing, dtype, stream);
+  return lf_lora_fwd(X, dense, bias, mask, a_ptrs, b_ptrs, Y, S_out, workspace ? (char*)workspace + head : nullptr,
+                     ws_bytes - head, M, N, K, R, routing, dtype, stream);
 }
 
 int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const uint8_t* mask, const void* S,
                     const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
                     void* const* db_ptrs, void* dS_out, void* workspace, size_t ws_bytes, int M, int N, int K, int R,
                     const lf_routing* routing, int dtype, void* stream) {
-  if (N <= 0 || K <= 0) return LF_EINVAL;
-  const size_t wbytes = align256((size_t)N * K * 2);
-  if (!workspace || ws_bytes < wbytes || ((uintptr_t)workspace & 255) != 0) return LF_EWORKSPACE;
-  if (dX) {
-    if (!W || !W->packed || !W->absmax) return LF_EINVAL;
-    int rc = lf_launch_nf4_dequant(W->packed, W->absmax, W->code2, W->absmax2, W->offset, workspace, (int64_t)N * K,
-                                   W->blocksize, W->blocksize2, dtype, (hipStream_t)stream);
-    if (rc != LF_OK) return rc;
-  }
-  return lf_lora_bwd(dY, X, workspace, mask, S, a_ptrs, b_ptrs, dX, da_ptrs, db_ptrs, dS_out, (char*)workspace + wbytes,
-                     ws_bytes - wbytes, M, N, K, R, routing, dtype, stream);
+  if (bad_dtype(dtype)) return LF_EINVAL;
+  const void* dense;
+  size_t head;
+  int rc = nf4_dense(W, dX != nullptr, workspace, ws_bytes, N, K, dtype, (hipStream_t)stream, &dense, &head);
+  if (rc != LF_OK) return rc;
+  return lf_lora_bwd(dY, X, dense, mask, S, a_ptrs, b_ptrs, dX, da_ptrs, db_ptrs, dS_out,
+                     workspace ? (char*)workspace + head : nullptr, ws_bytes - head, M, N, K, R, routing, dtype, stream);
 }
 
 int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream) {

@@ -501,31 +501,42 @@ def lora_backward(dy, x, w, a_list, b_list, s, routing_c, R, mask, rank_list, re
     return dx, da_list, db_list
 
 
-def nf4_lora_forward(x, wref, a_list, b_list, routing_c, R, mask, bias):
+def nf4_lora_forward(x, wref, a_list, b_list, routing_c, R, mask, bias, *, keep_dense: bool = False):
     """``lora_forward`` with the base weight given as NF4 (``nf4.NF4WeightRef``): one C call dequantises it
-    into the call's workspace and runs the forward on it.  Returns (y, s)."""
+    and runs the forward on it.  Returns (y, s), or (y, s, dense) with ``keep_dense``: the dequantised
+    weight then goes into a tensor of its own instead of the call's workspace, for a backward that
+    follows while it is still around (``nf4_lora_backward(..., dense=dense)``)."""
     M, K = x.shape
     N = wref.shape[0]
     y = torch.empty((M, N), dtype=x.dtype, device=x.device)
     s = torch.empty((M, R), dtype=x.dtype, device=x.device)
-    ws, nbytes = _ws(L.LF_OP_NF4_FWD, M, N, K, R, routing_c, x.device)
-    rc = L.lib().lf_nf4_lora_fwd(L.ptr(x), ctypes.byref(wref.c), L.ptr(bias), L.ptr(mask), L.ptr_array(a_list),
+    dense = torch.empty((N, K), dtype=x.dtype, device=x.device) if keep_dense else None
+    wc = wref.with_dense(dense, valid=False)
+    ws, nbytes = _ws(L.LF_OP_FWD if keep_dense else L.LF_OP_NF4_FWD, M, N, K, R, routing_c, x.device)
+    rc = L.lib().lf_nf4_lora_fwd(L.ptr(x), ctypes.byref(wc), L.ptr(bias), L.ptr(mask), L.ptr_array(a_list),
                                  L.ptr_array(b_list), L.ptr(y), L.ptr(s), L.ptr(ws), nbytes, M, N, K, R, routing_c,
                                  L.dtype_id(x.dtype), L.stream_of(x))
     L.check(rc, "lf_nf4_lora_fwd")
-    return y, s
+    return (y, s, dense) if keep_dense else (y, s)
 
 
-def nf4_lora_backward(dy, x, wref, a_list, b_list, s, routing_c, R, mask, rank_list, requires_dx: bool = True):
-    """``lora_backward`` with the base weight given as NF4.  Returns (dx | None, da_list, db_list)."""
+def nf4_lora_backward(dy, x, wref, a_list, b_list, s, routing_c, R, mask, rank_list, requires_dx: bool = True,
+                      dense: torch.Tensor | None = None):
+    """``lora_backward`` with the base weight given as NF4.  ``dense``: the dequantised weight a forward with
+    ``keep_dense`` left behind (nothing is dequantised then).  Returns (dx | None, da_list, db_list)."""
     M, N = dy.shape
     K = x.shape[1]
     dx = torch.empty((M, K), dtype=dy.dtype, device=dy.device) if requires_dx else None
     da_list = [torch.empty((r, K), dtype=dy.dtype, device=dy.device) for r in rank_list]
     db_list = [torch.empty((N, r), dtype=dy.dtype, device=dy.device) for r in rank_list]
     ds = torch.empty((M, R), dtype=dy.dtype, device=dy.device)
-    ws, nbytes = _ws(L.LF_OP_NF4_BWD, M, N, K, R, routing_c, dy.device)
-    rc = L.lib().lf_nf4_lora_bwd(L.ptr(dy), L.ptr(x), ctypes.byref(wref.c), L.ptr(mask), L.ptr(s), L.ptr_array(a_list),
+    if dense is not None and (tuple(dense.shape) != (N, K) or dense.dtype != dy.dtype or not dense.is_contiguous()):
+        raise ValueError(f"dense must be a contiguous [{N}, {K}] tensor of dtype {dy.dtype}.")
+    wc = wref.with_dense(dense, valid=True)
+    # no weight-sized head in the workspace when the weight is handed over, or not needed at all (no dX)
+    lean = dense is not None or not requires_dx
+    ws, nbytes = _ws(L.LF_OP_BWD if lean else L.LF_OP_NF4_BWD, M, N, K, R, routing_c, dy.device)
+    rc = L.lib().lf_nf4_lora_bwd(L.ptr(dy), L.ptr(x), ctypes.byref(wc), L.ptr(mask), L.ptr(s), L.ptr_array(a_list),
                                  L.ptr_array(b_list), L.ptr(dx), L.ptr_array(da_list), L.ptr_array(db_list), L.ptr(ds),
                                  L.ptr(ws), nbytes, M, N, K, R, routing_c, L.dtype_id(dy.dtype), L.stream_of(dy))
     L.check(rc, "lf_nf4_lora_bwd")

@@ -199,7 +199,7 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, padded_x, linear_w, linear_bias, dropout_mask, seed, routing: MultiRouting, quant_state,
-                n_adapters, *ab):
+                keep_dequantized, n_adapters, *ab):
         if padded_x.ndim == THREE_DIM:
             if padded_x.shape[0] != 1:
                 raise ValueError("currently, we only support batch size 1 for multi-linear LoRA")
@@ -235,14 +235,18 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
         if linear_bias is not None and (tuple(linear_bias.shape) != (N,) or linear_bias.dtype != x2d.dtype):
             raise ValueError(f"linear_bias must have shape [{N}] and dtype {x2d.dtype}.")
 
-        mask = None
+        mask, dense = None, None
         bias = linear_bias.contiguous() if linear_bias is not None else None
         if wref is not None:
             if routing.enable_dropout:
                 if dropout_mask is None:
                     dropout_mask = hip_ops.make_dropout_mask((M, K), 0.0, seed, x2d.device, routing=routing)
                 mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
-            y, s = hip_ops.nf4_lora_forward(x2d, wref, a_list, b_list, routing.c, routing.R, mask, bias)
+            if keep_dequantized:
+                y, s, dense = hip_ops.nf4_lora_forward(x2d, wref, a_list, b_list, routing.c, routing.R, mask, bias,
+                                                       keep_dense=True)
+            else:
+                y, s = hip_ops.nf4_lora_forward(x2d, wref, a_list, b_list, routing.c, routing.R, mask, bias)
         elif routing.enable_dropout and dropout_mask is None:
             # per-block p from the routing table, mask drawn inside the rank-r pass
             if seed is None:
@@ -253,7 +257,7 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
                 mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
             y, s = hip_ops.lora_forward(x2d, linear_w, a_list, b_list, routing.c, routing.R, mask, bias)
 
-        ctx.save_for_backward(x2d, linear_w, mask, s, *a_list, *b_list)
+        ctx.save_for_backward(x2d, linear_w, mask, s, dense, *a_list, *b_list)
         ctx.routing = routing
         ctx.quant_state = quant_state
         ctx.n_adapters = n_adapters
@@ -262,7 +266,7 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
-        x2d, linear_w, mask, s, *ab = ctx.saved_tensors
+        x2d, linear_w, mask, s, dense, *ab = ctx.saved_tensors
         n = ctx.n_adapters
         a_list, b_list = list(ab[:n]), list(ab[n:])
         routing = ctx.routing
@@ -280,7 +284,7 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
 
             dx, da_list, db_list = hip_ops.nf4_lora_backward(
                 dy2d, x2d, NF4WeightRef(linear_w, ctx.quant_state), a_list, b_list, s, routing.c, routing.R, mask,
-                routing.rank_list, requires_dx=ctx.needs_input_grad[0],
+                routing.rank_list, requires_dx=ctx.needs_input_grad[0], dense=dense,
             )
         else:
             dx, da_list, db_list = hip_ops.lora_backward(
@@ -289,7 +293,7 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
             )
         if dx is not None and ctx.lead:
             dx = dx.reshape(1, *dx.shape)
-        return (dx, None, None, None, None, None, None, None, *da_list, *db_list)
+        return (dx, None, None, None, None, None, None, None, None, *da_list, *db_list)
 
 
 def fused_linear_multi_lora(
@@ -311,6 +315,7 @@ def fused_linear_multi_lora(
     seed: int | None = None,
     quant_state=None,
     routing: MultiRouting | None = None,
+    keep_dequantized: bool = False,
 ) -> torch.Tensor:
     """Fused multi-adapter LoRA linear (lorafusion/ops/multi_lora.py:762-830).
 
@@ -320,7 +325,8 @@ def fused_linear_multi_lora(
     bitsandbytes-style state ``dequantize_nf4_triton`` takes) ``linear_w`` holds packed NF4 codes and
     is dequantised inside the forward and backward calls.  ``routing`` (extension) is the cached
     ``MultiLoRABatchInfo.routing(...)`` of the micro-batch the table arguments come from; without it the same
-    object is built here, per call.
+    object is built here, per call.  ``keep_dequantized`` (extension, NF4 only): the forward's dequantised
+    weight is kept for the backward, which then dequantises nothing (2*N*K bytes held in between).
     """
     if len(lora_a_list) != len(lora_b_list):
         raise ValueError("lora_a_list and lora_b_list must have the same length")
@@ -340,7 +346,7 @@ def fused_linear_multi_lora(
           or routing.enable_dropout != bool(enable_dropout) or routing.table.data_ptr() != block_to_lookup_table.data_ptr()):
         raise ValueError("routing does not belong to the batch tables passed with it")
     return FusedLinearMultiLoRA.apply(padded_x, linear_w, linear_bias, dropout_mask, seed, routing, quant_state,
-                                      len(lora_a_list), *lora_a_list, *lora_b_list)
+                                      bool(keep_dequantized), len(lora_a_list), *lora_a_list, *lora_b_list)
 
 
 # --------------------------------------------------------------------------- manager

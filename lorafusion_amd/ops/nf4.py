@@ -114,7 +114,15 @@ class NF4WeightRef:
             raise ValueError(f"the quantised weight must be 2-D [N, K], got shape {tuple(shape)}.")
         self.keep = (A, absmax, code, absmax2, offset)
         self.shape, self.dtype = shape, out_dtype
-        self.c = L.NF4Weight(L.ptr(A), L.ptr(absmax), L.ptr(code), L.ptr(absmax2), L.ptr(offset), blocksize, bs2)
+        self.c = L.NF4Weight(L.ptr(A), L.ptr(absmax), L.ptr(code), L.ptr(absmax2), L.ptr(offset), blocksize, bs2, None, 0, 0)
+
+    def with_dense(self, dense, *, valid: bool):
+        """The struct with ``dense`` (a [N, K] tensor for the dequantised weight, or None) filled in."""
+        if dense is None:
+            return self.c
+        c = self.c
+        return L.NF4Weight(c.packed, c.absmax, c.code2, c.absmax2, c.offset, c.blocksize, c.blocksize2,
+                           dense.data_ptr(), 1 if valid else 0, 0)
 
 
 dequantize_nf4 = dequantize_nf4_triton
@@ -175,11 +183,13 @@ class FusedLinearLoRANF4(torch.autograd.Function):
 
     Forward and backward each dequantise the weight into the call's workspace
     (``lf_nf4_lora_fwd`` / ``lf_nf4_lora_bwd``) and run the fused LoRA GEMMs on it; only the
-    packed weight stays resident.
+    packed weight stays resident.  With ``keep_dequantized`` the forward's dequantised weight is
+    kept for the backward instead (one dequantisation per step, 2*N*K bytes held in between).
     """
 
     @staticmethod
-    def forward(ctx, x, packed_w, quant_state, lora_a, lora_b, alpha, dropout_p, seed, linear_bias, dropout_mask):
+    def forward(ctx, x, packed_w, quant_state, lora_a, lora_b, alpha, dropout_p, seed, linear_bias, dropout_mask,
+                keep_dequantized=False):
         from lorafusion_amd.ops import hip_ops
         from lorafusion_amd.ops.lora_v1 import _validate_shapes
 
@@ -204,8 +214,13 @@ class FusedLinearLoRANF4(torch.autograd.Function):
             mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
         p_eff = dropout_p if mask is not None else 0.0
         routing = L.single_routing(r, alpha, p_eff)
-        y, s = hip_ops.nf4_lora_forward(x2d, wref, [lora_a], [lora_b], routing, L.round_rank(r), mask, bias)
-        ctx.save_for_backward(x2d, packed_w, lora_a, lora_b, mask, s)
+        dense = None
+        if keep_dequantized:
+            y, s, dense = hip_ops.nf4_lora_forward(x2d, wref, [lora_a], [lora_b], routing, L.round_rank(r), mask, bias,
+                                                   keep_dense=True)
+        else:
+            y, s = hip_ops.nf4_lora_forward(x2d, wref, [lora_a], [lora_b], routing, L.round_rank(r), mask, bias)
+        ctx.save_for_backward(x2d, packed_w, lora_a, lora_b, mask, s, dense)
         ctx.quant_state, ctx.alpha, ctx.p, ctx.lead = quant_state, alpha, p_eff, lead
         return y if lead is None else y.reshape(*lead, N)
 
@@ -213,21 +228,25 @@ class FusedLinearLoRANF4(torch.autograd.Function):
     def backward(ctx, dy):
         from lorafusion_amd.ops import hip_ops
 
-        x2d, packed_w, lora_a, lora_b, mask, s = ctx.saved_tensors
+        x2d, packed_w, lora_a, lora_b, mask, s, dense = ctx.saved_tensors
         dy2d = dy.reshape(-1, dy.shape[-1]).contiguous()
         r = lora_a.shape[0]
         wref = NF4WeightRef(packed_w, ctx.quant_state)
         routing = L.single_routing(r, ctx.alpha, ctx.p)
         dx, da_list, db_list = hip_ops.nf4_lora_backward(dy2d, x2d, wref, [lora_a], [lora_b], s, routing,
                                                          L.round_rank(r), mask, [r],
-                                                         requires_dx=ctx.needs_input_grad[0])
+                                                         requires_dx=ctx.needs_input_grad[0], dense=dense)
         if dx is not None and ctx.lead is not None:
             dx = dx.reshape(*ctx.lead, -1)
-        return dx, None, None, da_list[0], db_list[0], None, None, None, None, None
+        return dx, None, None, da_list[0], db_list[0], None, None, None, None, None, None
 
 
 def fused_linear_lora_nf4(x, packed_w, quant_state, lora_a, lora_b, alpha, seed=None, dropout_p=0.0,
-                          linear_bias=None, dropout_mask=None):
-    """``fused_linear_lora`` with the base weight stored as NF4 (``packed_w`` + ``quant_state``)."""
+                          linear_bias=None, dropout_mask=None, *, keep_dequantized: bool = False):
+    """``fused_linear_lora`` with the base weight stored as NF4 (``packed_w`` + ``quant_state``).
+
+    ``keep_dequantized``: keep the forward's dequantised weight (2*N*K bytes) until the backward has run, which
+    then dequantises nothing -- for a backward that follows its forward closely (one layer at a time, or a
+    recomputed forward under activation checkpointing); the default holds only the packed weight."""
     return FusedLinearLoRANF4.apply(x, packed_w, quant_state, lora_a, lora_b, alpha, dropout_p, seed,
-                                    linear_bias, dropout_mask)
+                                    linear_bias, dropout_mask, keep_dequantized)

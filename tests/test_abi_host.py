@@ -36,8 +36,8 @@ def test_routing_struct_layout_matches_header():
     assert ctypes.sizeof(_lib.Routing) == 16 + 24 + 8 + 2 * 4 * _lib.LF_MAX_SEG
     r = _lib.single_routing(16, 2.0, 0.1)
     assert r.n_seg == 1 and r.seg_rank[0] == 16 and abs(r.p - 0.1) < 1e-7
-    # struct lf_nf4_weight: 5 pointers + 2 int32
-    assert ctypes.sizeof(_lib.NF4Weight) == 5 * 8 + 2 * 4
+    # struct lf_nf4_weight: 5 pointers + 2 int32 + the optional dense buffer (pointer + 2 int32)
+    assert ctypes.sizeof(_lib.NF4Weight) == 5 * 8 + 2 * 4 + 8 + 2 * 4
 
 
 def test_argument_validation_without_gpu():
@@ -65,7 +65,7 @@ def test_argument_validation_without_gpu():
     wbytes = 256 * 256 * 2
     assert lib.lf_workspace_bytes(_lib.LF_OP_NF4_FWD, 256, 256, 256, 16, r) == wbytes + lib.lf_workspace_bytes(_lib.LF_OP_FWD, 256, 256, 256, 16, r)
     assert lib.lf_workspace_bytes(_lib.LF_OP_NF4_BWD, 256, 256, 256, 16, r) == wbytes + small
-    wq = _lib.NF4Weight(16, 16, None, None, None, 64, 0)
+    wq = _lib.NF4Weight(16, 16, None, None, None, 64, 0, None, 0, 0)
     args_fwd = (one, ctypes.byref(wq), None, None, ptrs, ptrs, one, one)
     assert lib.lf_nf4_lora_fwd(*args_fwd, None, 0, 256, 256, 256, 16, r, 0, None) == -3           # no workspace
     assert lib.lf_nf4_lora_fwd(*args_fwd, ctypes.c_void_p(256), 100, 256, 256, 256, 16, r, 0, None) == -3   # too small

@@ -164,3 +164,66 @@ def test_qlora_linear_adapter_grads_only_and_seeded_mask():
     for got, exp, name in ((y, ye, "y"), (a.grad, dae, "da"), (b.grad, dbe, "db")):
         ok, rel, excess = lora_ref.check_close(got.detach().float().cpu(), exp, rtol=1e-2)
         assert ok, f"{name}: rel {rel:.3e} excess {excess:.3e}"
+
+
+def test_qlora_keep_dequantized_weight_is_bit_identical():
+    """One dequantisation per step: the forward leaves the dequantised weight in a tensor of its own and the
+    backward reuses it.  Outputs and gradients equal the dequantise-twice path bit for bit (single and packed
+    multi-adapter op), and the kept tensor is the oracle's dequantised weight."""
+    from lorafusion_amd.ops import hip_ops
+    from lorafusion_amd.ops.multi_lora import fused_linear_multi_lora, prepare_multi_lora_batch_info
+    from lorafusion_amd.ops.nf4 import NF4WeightRef, fused_linear_lora_nf4
+    from lorafusion_amd import _lib as L
+    from tests.util import multi_inputs
+
+    M, K, N, r, p, scale = 384, 512, 768, 16, 0.1, 2.0
+    d = single_inputs(M, K, N, r, p=p, seed=9)
+    st = onf4.quantize_nf4(d["w"].float().numpy())
+    wq = torch.from_numpy(onf4.dequantize(st).view(np.int16)).view(torch.bfloat16).reshape(N, K)
+    packed, qs = _to_state(st)
+    outs = []
+    for keep in (False, True):
+        x = d["x"].cuda().requires_grad_(True)
+        a = d["a"].cuda().requires_grad_(True)
+        b = d["b"].cuda().requires_grad_(True)
+        y = fused_linear_lora_nf4(x, packed, qs, a, b, scale, dropout_p=p, dropout_mask=d["mask"].cuda(), keep_dequantized=keep)
+        y.backward(d["dy"].cuda())
+        outs.append((y.detach(), x.grad, a.grad, b.grad))
+    for t0, t1 in zip(*outs):
+        assert torch.equal(t0, t1)
+    # the raw ops: the kept tensor is the dequantised weight; a backward handed a weight uses exactly that weight
+    routing = L.single_routing(r, scale, p)
+    wref = NF4WeightRef(packed, qs)
+    xd, ad, bd, mk, dyd = d["x"].cuda(), d["a"].cuda(), d["b"].cuda(), d["mask"].cuda(), d["dy"].cuda()
+    y, s, dense = hip_ops.nf4_lora_forward(xd, wref, [ad], [bd], routing, 16, mk, None, keep_dense=True)
+    assert torch.equal(dense.cpu().view(torch.int16), wq.view(torch.int16))
+    dx_kept, _, _ = hip_ops.nf4_lora_backward(dyd, xd, wref, [ad], [bd], s, routing, 16, mk, [r], dense=dense)
+    assert torch.equal(dx_kept, outs[0][1])
+    dx_zero_w, _, _ = hip_ops.nf4_lora_backward(dyd, xd, wref, [ad], [bd], s, routing, 16, mk, [r], dense=torch.zeros_like(dense))
+    lora_only = dx_zero_w.float().cpu()          # dY * 0 + the LoRA term alone
+    dxe, *_ = lora_ref.linear_lora_bwd_fp32(d["dy"], d["x"], torch.zeros(N, K), d["a"], d["b"], scale, d["mask"], p)
+    ok, rel, excess = lora_ref.check_close(lora_only, dxe, rtol=1e-2)
+    assert ok, f"dx from a handed-over zero weight: rel {rel:.3e} excess {excess:.3e}"
+    with pytest.raises(ValueError):
+        hip_ops.nf4_lora_backward(dyd, xd, wref, [ad], [bd], s, routing, 16, mk, [r], dense=dense[:, :64])
+
+    # packed multi-adapter op
+    seq, ranks, p_list, scales = [130, 257], [16, 32], [0.0, 0.1], [1.0, 2.0]
+    dm = multi_inputs(seq, 512, 384, ranks, p_list, seed=4)
+    stm = onf4.quantize_nf4(dm["w"].float().numpy())
+    packed_m, qs_m = _to_state(stm)
+    info = prepare_multi_lora_batch_info(seq, [0, 1], ranks, p_list, scales, 128)
+    outs = []
+    for keep in (False, True):
+        x = dm["x"].cuda().requires_grad_(True)
+        al = [t.cuda().requires_grad_(True) for t in dm["a_list"]]
+        bl = [t.cuda().requires_grad_(True) for t in dm["b_list"]]
+        y = fused_linear_multi_lora(
+            x.unsqueeze(0), packed_m, lora_a_list=al, lora_b_list=bl, seq_len_list=seq,
+            padded_seq_len_list=info.padded_seq_len_list, block_to_lookup_table=info.block_to_lookup_table,
+            block_to_dropout_p=info.block_to_dropout_p, block_to_alpha=info.block_to_alpha, enable_dropout=True,
+            same_dropout_p_value=None, max_r=32, dropout_mask=dm["mask"].cuda(), quant_state=qs_m, keep_dequantized=keep)
+        y.backward(dm["dy"].cuda().unsqueeze(0))
+        outs.append([y.detach(), x.grad] + [t.grad for t in al + bl])
+    for t0, t1 in zip(*outs):
+        assert torch.equal(t0, t1)
