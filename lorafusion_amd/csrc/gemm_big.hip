@@ -96,7 +96,7 @@ __device__ __forceinline__ void sfor(F&& f) {
 }
 
 #ifdef LF_BIG_TIMING
-__device__ unsigned long long lf_big_timing[8];  // cycles: seed, k loop, epilogue, wall (100 MHz), tiles
+__device__ unsigned long long lf_big_timing[16];  // cycles: seed, k loop, epilogue, wall (100 MHz), tiles
 #define LF_TICK(var) const long long var = __builtin_readcyclecounter()
 #else
 #define LF_TICK(var)
@@ -210,7 +210,11 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     asm volatile("s_add_u32 m0, %0, %1" ::"s"(base), "n"(OFF.value) : "memory", "scc");
   };
   auto issue_load = [&](lf_u32x4 rsrc, uint32_t voff, int soff) __attribute__((always_inline)) {
+#ifndef LF_ABL_NOLOAD
     asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
+#else
+    asm volatile("" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
+#endif
   };
   // all 16 loads of K step k of the tile behind `src` into stage `stage` (prologue only: no MFMAs to hide behind)
   auto load_stage = [&](const LoadSrc& src, int k, int stage) __attribute__((always_inline)) {
@@ -295,6 +299,9 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     // one fragment read of sub-step KS of the stage at LDS byte offset `st`: idx < 8: A fragment idx; else B fragment idx-8
     auto read_one = [&](auto SET, auto KS, uint32_t st, auto IDX) __attribute__((always_inline)) {
       constexpr int idx = IDX.value, set = SET.value, ks = KS.value;
+#ifdef LF_ABL_NOREAD
+      if (st != 0xffffffffu) return;   // (ablation build) never true: the fragments keep their first values
+#endif
       if constexpr (idx < 8) {
         const uint32_t ad = fa_off[ks] + st;
         lf_u32x4 tmp;
@@ -393,32 +400,68 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       };
       int t = 0;
       for (; t + 1 < n_chunks; t++) chunk(t);
-      // A lane reads the four mask bytes of its four accumulator columns of every block.  The loads are issued
-      // whether or not a mask applies (without one: 64 times the first dword of L): defined under a condition and
-      // used under another, the 64 values are spilled one by one, each behind its own wait.
-      uint32_t mk[8][8];
+      // Keep-mask of the wave's 128x128 block: 16 KB.  A lane owns, in every 16x16 accumulator block, row l16 and four
+      // consecutive columns (one dword of mask bytes), so loading "its" dwords directly is 64 instructions that each
+      // touch 16 rows -- 16 cache lines for 256 bytes; measured 17 K cycles per tile, most of the seed.  Instead the
+      // block is read with whole rows per instruction (lane -> row lane>>3, 16-byte chunk lane&7: 8 rows x 128 bytes,
+      // 16 instructions) and each 16-row slab is turned to the accumulator layout through the wave's LDS patch (rows
+      // 144 bytes apart: the 64 dword reads of a slab then hit 64 different banks).  The loads are issued whether or
+      // not a mask applies (without one: 16 times the head of L): defined under a condition and used under another,
+      // the compiler spills the values one by one, each behind its own wait.
+      lf_u32x4 mq[16];
       {
-        const uint8_t* mrow = sel ? p.mask + (int64_t)(wrow0 + l16) * p.ldmask + n0 + wn * 128 + kg * 4 : (const uint8_t*)Lp;
-        const int64_t mstride = sel ? 16 * p.ldmask : 0;
-        const int jstride = sel ? 16 : 0;
+        const uint8_t* mrow = sel ? p.mask + (int64_t)(wrow0 + (sl >> 3)) * p.ldmask + n0 + wn * 128 + (sl & 7) * 16 : (const uint8_t*)Lp;
+        const int64_t qstride = sel ? 8 * p.ldmask : 0;
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-#pragma unroll
-          for (int j = 0; j < 8; j++) mk[i][j] = *(const uint32_t*)(mrow + i * mstride + j * jstride);
+        for (int q = 0; q < 16; q++) {
+#ifndef LF_ABL_NOMASKLOAD
+          mq[q] = *(const lf_u32x4*)(mrow + q * qstride);
+#else
+          mq[q] = lf_u32x4{0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u + (uint32_t)qstride};
+#endif
+        }
       }
       chunk(t);
+#ifdef LF_ABL_NOSELECT
+      if (sel && mult == 12345.f) {
+#else
       if (sel) {
+#endif
         mfma_fence();
-        // keep-mask select and 1/(1-p) in fp32, one block row at a time
+        // keep-mask select and 1/(1-p) in fp32, one block row (16-row slab) at a time
+        constexpr int MPITCH = 144;
+        const uint32_t mp_lds = lds0 + EP_OFF + wave * EP_WAVE;
+        const uint32_t mp_wr = mp_lds + (sl >> 3) * MPITCH + (sl & 7) * 16;   // + 8 rows for the slab's second load
+        const uint32_t mp_rd = mp_lds + l16 * MPITCH + kg * 4;                // + 16 per accumulator block
 #pragma unroll
         for (int i = 0; i < 8; i++) {
+          asm volatile("ds_write_b128 %0, %1" ::"v"(mp_wr), "v"(mq[2 * i]) : "memory");
+          asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(mp_wr), "v"(mq[2 * i + 1]), "n"(8 * MPITCH) : "memory");
+          lgkm0();
+          uint32_t mk[8];
+          {
+            // (written out: inline-assembly operands inside a generic lambda do not compile with this clang)
+            uint32_t k0, k1, k2, k3, k4, k5, k6, k7;
+            asm volatile("ds_read_b32 %0, %1" : "=v"(k0) : "v"(mp_rd) : "memory");
+            asm volatile("ds_read_b32 %0, %1 offset:16" : "=v"(k1) : "v"(mp_rd) : "memory");
+            asm volatile("ds_read_b32 %0, %1 offset:32" : "=v"(k2) : "v"(mp_rd) : "memory");
+            asm volatile("ds_read_b32 %0, %1 offset:48" : "=v"(k3) : "v"(mp_rd) : "memory");
+            asm volatile("ds_read_b32 %0, %1 offset:64" : "=v"(k4) : "v"(mp_rd) : "memory");
+            asm volatile("ds_read_b32 %0, %1 offset:80" : "=v"(k5) : "v"(mp_rd) : "memory");
+            asm volatile("ds_read_b32 %0, %1 offset:96" : "=v"(k6) : "v"(mp_rd) : "memory");
+            asm volatile("ds_read_b32 %0, %1 offset:112" : "=v"(k7) : "v"(mp_rd) : "memory");
+            lgkm0();
+            // the waits are assembly too: the values are used only behind this point
+            asm volatile("" : "+v"(k0), "+v"(k1), "+v"(k2), "+v"(k3), "+v"(k4), "+v"(k5), "+v"(k6), "+v"(k7));
+            mk[0] = k0; mk[1] = k1; mk[2] = k2; mk[3] = k3; mk[4] = k4; mk[5] = k5; mk[6] = k6; mk[7] = k7;
+          }
 #pragma unroll
           for (int j = 0; j < 8; j++) {
             // a definition right in front of the use: the copies out of the accumulation registers cannot rise above
             // it (without it, all 256 are read up front)
             asm volatile("" : "+a"(acc[i][j]));
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc[i][j][e] = ((mk[i][j] >> (8 * e)) & 0xffu) ? acc[i][j][e] * mult : 0.f;
+            for (int e = 0; e < 4; e++) acc[i][j][e] = ((mk[j] >> (8 * e)) & 0xffu) ? acc[i][j][e] * mult : 0.f;
             asm volatile("" : "+a"(acc[i][j]));  // back into the accumulation registers now, not at the next use
           }
           __builtin_amdgcn_sched_barrier(0);
