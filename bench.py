@@ -49,8 +49,10 @@ WORKLOADS = {
     "c4": (16384, 4, 16, [1.0, 2.0, 2.0, 4.0], [0.0, 0.05, 0.1, 0.1], False, 8192,
            [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]),
     "c5": (8192, 8, 64, [1.0, 2.0, 2.0, 4.0] * 2, [0.0, 0.05, 0.1, 0.1] * 2, True, 4096,
-           [("q", 8192, 8192), ("k", 8192, 1024), ("v", 8192, 1024), ("o", 8192, 8192),
-            ("gate", 8192, 28672), ("up", 8192, 28672), ("down", 28672, 8192)]),
+           [("qkv", 8192, 10240), ("o", 8192, 8192), ("gate_up", 8192, 57344), ("down", 28672, 8192)]),
+    "c5_separate": (8192, 8, 64, [1.0, 2.0, 2.0, 4.0] * 2, [0.0, 0.05, 0.1, 0.1] * 2, True, 4096,
+                    [("q", 8192, 8192), ("k", 8192, 1024), ("v", 8192, 1024), ("o", 8192, 8192),
+                     ("gate", 8192, 28672), ("up", 8192, 28672), ("down", 28672, 8192)]),
 }
 NAMES = {
     "c1": "single LoRA linear, 2048 tokens, K=N=4096, r=16, p=0.1, explicit mask, fwd+bwd",
@@ -61,9 +63,12 @@ NAMES = {
           "linears of the merged layer (qkv N=6144, o, gate+up N=28672, down), 16384 packed tokens, 4 adapters r=16, "
           "training-mode dropout drawn in the rank-r pass, fwd+bwd, driven by a micro-batch descriptor through the "
           "patched layer; attention, rotary embedding, norms and activation are not part of the path and not run",
-    "c5": "the seven LoRA linears of a 70B-class decoder layer (hidden 8192, kv 1024, MLP 28672) with NF4 base "
-          "weights (dequantised inside every call), 8192 packed tokens, 8 adapters r=64, explicit masks, fwd+bwd; "
-          "attention, norms and activation are not part of the path",
+    "c5": "the seven LoRA projections of a 70B-class decoder layer (hidden 8192, kv 1024, MLP 28672) as the four LoRA "
+          "linears of the merged layer (qkv N=10240, o, gate+up N=57344, down) with NF4 base weights (dequantised "
+          "inside every call), 8192 packed tokens, 8 adapters r=64, explicit masks, fwd+bwd; attention, norms and "
+          "activation are not part of the path",
+    "c5_separate": "the same 70B-class layer as seven separate LoRA linears (q, k, v, o, gate, up, down), NF4 base weights, "
+                   "8192 packed tokens, 8 adapters r=64, explicit masks, fwd+bwd",
 }
 
 

@@ -95,6 +95,10 @@ __device__ __forceinline__ void sfor(F&& f) {
   [&]<int... I>(std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>{}), ...); }(std::make_integer_sequence<int, N>{});
 }
 
+// Measurement builds only (never defined in the library build): LF_BIG_TIMING adds per-tile cycle counters (seed, K loop,
+// epilogue, waits) summed into lf_big_timing; LF_ABL_NOLOAD / LF_ABL_NOREAD / LF_ABL_NOMASKLOAD / LF_ABL_NOSELECT drop
+// the tile loads, the fragment reads, the keep-mask loads or the keep-mask select (results are then wrong: the
+// builds exist to attribute cycles and clock to the parts of the kernel).
 #ifdef LF_BIG_TIMING
 __device__ unsigned long long lf_big_timing[16];  // cycles: seed, k loop, epilogue, wall (100 MHz), tiles
 #define LF_TICK(var) const long long var = __builtin_readcyclecounter()
