@@ -243,6 +243,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   using S0 = integral_constant<int, 0>;
   using S1 = integral_constant<int, 1>;
   constexpr int RDS = 3;   // a fragment read every RDS MFMAs
+  constexpr int LDP = 4;   // a tile load every LDP MFMAs of sub-step 1 (denser issue queues up in the texture addresser: 2 and 3 measured 2-6 % slower)
   const T* __restrict__ Lp = (const T*)p.L;
   T* __restrict__ C = (T*)p.C;
   const uint16_t* bias16 = (const uint16_t*)p.bias;
@@ -534,11 +535,11 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       sfor<64>([&](auto MM) {
         constexpr int m = MM.value;
         if constexpr (m % RDS == 0 && m / RDS < 16) read_one(S0{}, S0{}, nxt, integral_constant<int, (m / RDS + 8) & 15>{});
-        if constexpr (m % 4 == 0) {
-          if constexpr (m / 4 < 8) set_m0(ma, integral_constant<int, (m / 4) * 4096>{});
-          else set_m0(mb, integral_constant<int, (m / 4 - 8) * M0B_STEP>{});
+        if constexpr (m % LDP == 0 && m / LDP < 16) {
+          if constexpr (m / LDP < 8) set_m0(ma, integral_constant<int, (m / LDP) * 4096>{});
+          else set_m0(mb, integral_constant<int, (m / LDP - 8) * M0B_STEP>{});
         }
-        if constexpr (m % 4 == 1) issue_load(m / 4 < 8 ? ld.ra : ld.rb, m / 4 < 8 ? a_voff : b_voff, soff[m / 4]);
+        if constexpr (m % LDP == 1 && m / LDP < 16) issue_load(m / LDP < 8 ? ld.ra : ld.rb, m / LDP < 8 ? a_voff : b_voff, soff[m / LDP]);
         mfma_one(1, m);
         __builtin_amdgcn_sched_barrier(0);
       });

@@ -335,134 +335,6 @@ __device__ __forceinline__ void reduce_rows_body(int bx, const float* __restrict
   *(lf_u32x2*)((uint16_t*)out + idx) = pack4<T>(v);
 }
 
-// ------------------------------------------------------------------------------- dys_dyb
-// grid (n_blocks, nsplit).  Each workgroup walks its N slice in 64-column tiles of dY:
-//   dS partial  [128 rows, R]  += dY_tile * B_tile            (accumulated over the slice)
-//   dB partial  [64 cols, R]    = dY_tile^T * S_block         (complete per tile)
-// LDS: two dY tiles, the S block [128][R] and two B tiles [64][R] (pitch 2R+32 bytes keeps the
-// 4-row transpose reads on distinct banks).
-template <typename T, int RT>
-__global__ void __launch_bounds__(256)
-lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __restrict__ ds_part,
-                    float* __restrict__ db_part, int M, int N, int R, int tiles_per_wg, const LfSegTable seg) {
-  constexpr int RP = RT * 32 + 32;
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  char* ys = lds;
-  char* ss = lds + 2 * TILE_BYTES;
-  char* bs = ss + ROWS * RP;
-
-  const int blk = blockIdx.x, ns = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int li = lane & 15, qq = lane >> 4, j4 = li >> 2, c4 = li & 3;
-  const BlockInfo bi = block_info(seg, blk, M);
-  const T* __restrict__ Bl = (const T*)seg.ptr[bi.seg];
-  const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
-  const int n_begin = ns * tiles_per_wg * 64;
-  const int ntiles = min(tiles_per_wg, N / 64 - ns * tiles_per_wg);  // the last slice may be shorter
-
-  auto load_b = [&](lf_u32x4 (&br)[(64 * RT * 2 + 255) / 256], int n0) {
-#pragma unroll
-    for (int i = 0; i < (64 * RT * 2 + 255) / 256; i++) {
-      const int g = i * 256 + tid;
-      const int row = g / (RT * 2), gc = g % (RT * 2);
-      lf_u32x4 v = {0, 0, 0, 0};
-      if (g < 64 * RT * 2 && gc * 8 < bi.rank) v = *(const lf_u32x4*)(Bl + (int64_t)(n0 + row) * bi.rank + gc * 8);
-      br[i] = v;
-    }
-  };
-  auto store_b = [&](const lf_u32x4 (&br)[(64 * RT * 2 + 255) / 256], char* dst) {
-#pragma unroll
-    for (int i = 0; i < (64 * RT * 2 + 255) / 256; i++) {
-      const int g = i * 256 + tid;
-      if (g < 64 * RT * 2) *(lf_u32x4*)(dst + (g / (RT * 2)) * RP + (g % (RT * 2)) * 16) = br[i];
-    }
-  };
-
-  TileRegs tr;
-  lf_u32x4 br[(64 * RT * 2 + 255) / 256];
-  tile_load(tr, dY, (const uint8_t*)nullptr, N, blk * ROWS, Mrows, n_begin, tid, false);
-  load_b(br, n_begin);
-  // S block -> LDS (rows beyond `valid` as zeros so they add nothing to dB)
-  for (int g = tid; g < ROWS * RT * 2; g += 256) {
-    const int row = g / (RT * 2), gc = g % (RT * 2);
-    lf_u32x4 v = {0, 0, 0, 0};
-    // S has R columns; R may be smaller than the RT * 16 columns of the register tiling (R = 48, 80, 96, 112)
-    if (row < bi.valid && gc * 8 < R) v = *(const lf_u32x4*)(S + (int64_t)(blk * ROWS + row) * R + gc * 8);
-    *(lf_u32x4*)(ss + row * RP + gc * 16) = v;
-  }
-  tile_store(tr, ys, tid, false);
-  store_b(br, bs);
-  if (ntiles > 1) {
-    tile_load(tr, dY, (const uint8_t*)nullptr, N, blk * ROWS, Mrows, n_begin + 64, tid, false);
-    load_b(br, n_begin + 64);
-  }
-  __syncthreads();
-
-  lf_f32x4 acc_ds[2][RT];
-#pragma unroll
-  for (int a = 0; a < 2; a++)
-#pragma unroll
-    for (int c = 0; c < RT; c++) acc_ds[a][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
-
-  for (int t = 0; t < ntiles; t++) {
-    const char* ycur = ys + (t & 1) * TILE_BYTES;
-    const char* bcur = bs + (t & 1) * 64 * RP;
-    // dS += dY_tile * B_tile : a = dY row fragment, b = B^T through the transpose read
-#pragma unroll
-    for (int step = 0; step < 2; step++) {
-      lf_u32x4 yf[2];
-#pragma unroll
-      for (int rt = 0; rt < 2; rt++) yf[rt] = tile_row_frag(ycur, wave * 32 + rt * 16 + li, step * 4 + qq);
-#pragma unroll
-      for (int c = 0; c < RT; c++) {
-        const lf_u32x4 bf = tr_read8(bcur + (step * 32 + qq * 8 + j4) * RP + (c * 16 + 4 * c4) * 2, RP);
-#pragma unroll
-        for (int rt = 0; rt < 2; rt++) acc_ds[rt][c] = Mfma16<T>::run(yf[rt], bf, acc_ds[rt][c]);
-      }
-    }
-    // dB tile: D[n][r] = sum_m dY[m][n] S[m][r]; wave w owns columns 16w..16w+15 of the tile
-    lf_f32x4 acc_db[RT];
-#pragma unroll
-    for (int c = 0; c < RT; c++) acc_db[c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < 4; kk++) {
-      const int mrow = kk * 32 + qq * 8 + j4;
-      const lf_u32x4 yt = tile_tr_frag(ycur, mrow, wave * 16 + 4 * c4);
-#pragma unroll
-      for (int c = 0; c < RT; c++) {
-        const lf_u32x4 sf = tr_read8(ss + mrow * RP + (c * 16 + 4 * c4) * 2, RP);
-        acc_db[c] = Mfma16<T>::run(yt, sf, acc_db[c]);
-      }
-    }
-    float* dbo = db_part + ((int64_t)blk * N + n_begin + t * 64) * R;
-#pragma unroll
-    for (int c = 0; c < RT; c++)
-#pragma unroll
-      for (int e = 0; e < 4; e++)
-        if (c * 16 < R) dbo[(int64_t)(wave * 16 + qq * 4 + e) * R + c * 16 + li] = acc_db[c][e];
-
-    if (t + 1 < ntiles) {
-      tile_store(tr, ys + ((t + 1) & 1) * TILE_BYTES, tid, false);
-      store_b(br, bs + ((t + 1) & 1) * 64 * RP);
-      if (t + 2 < ntiles) {
-        tile_load(tr, dY, (const uint8_t*)nullptr, N, blk * ROWS, Mrows, n_begin + (t + 2) * 64, tid, false);
-        load_b(br, n_begin + (t + 2) * 64);
-      }
-    }
-    __syncthreads();
-  }
-  float* dso = ds_part + (int64_t)ns * Mrows * R;
-#pragma unroll
-  for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-    for (int c = 0; c < RT; c++)
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const int row = blk * ROWS + wave * 32 + rt * 16 + qq * 4 + e;
-        if (row < Mrows && c * 16 < R) dso[(int64_t)row * R + c * 16 + li] = acc_ds[rt][c][e];
-      }
-}
-
 // Blocks [b0, b1) of segment s.
 __device__ __forceinline__ void segment_blocks(const LfSegTable& seg, int s, int M, int& b0, int& b1) {
   if (seg.table == nullptr) {
@@ -474,8 +346,186 @@ __device__ __forceinline__ void segment_blocks(const LfSegTable& seg, int s, int
   }
 }
 
+// ------------------------------------------------------------------------------- dys_dyb
+// grid (n_seg * max_chunks, nsplit).  Workgroup (s, ch, ns) owns the `group` consecutive 128-row blocks ch*group.. of
+// segment s and the N slice ns (tiles_per_wg <= TPW tiles of 64 columns); it walks its blocks, and per block the
+// tiles of the slice:
+//   dS partial  [128 rows, R]  += dY_tile * B_tile      (per block, over the slice; written once per block)
+//   dB partial  [64 cols, R]   += dY_tile^T * S_block    (per tile of the slice, kept in registers over ALL blocks of the
+//                                                         chunk; written once per workgroup)
+// so dB leaves the chip once per chunk of blocks, not once per block: at rank 64 and N = 28672 the per-block slabs
+// were as large as dY itself.  TPW bounds the registers of the dB accumulators (TPW * RT * 4).
+// LDS: two dY tiles, the S block [128][R] and two B tiles [64][R] (pitch 2R+32 bytes keeps the 4-row transpose reads on
+// distinct banks).  The S block is single-buffered: at a block switch one extra barrier separates its last readers
+// from the store of the next block's S (prefetched in registers one tile earlier).
+template <typename T, int RT, int TPW>
+__global__ void __launch_bounds__(256, RT == 1 ? 3 : RT <= 4 ? 2 : 1)   // waves per SIMD: the register budget follows the LDS footprint
+lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __restrict__ ds_part,
+                    float* __restrict__ db_part, int M, int N, int R, int tiles_per_wg, int group, int max_chunks,
+                    const LfSegTable seg) {
+  constexpr int RP = RT * 32 + 32;
+  constexpr int NBR = (64 * RT * 2 + 255) / 256;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* ys = lds;
+  char* ss = lds + 2 * TILE_BYTES;
+  char* bs = ss + ROWS * RP;
+
+  const int s = blockIdx.x / max_chunks, ch = blockIdx.x % max_chunks, ns = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 15, qq = lane >> 4, j4 = li >> 2, c4 = li & 3;
+  int b0, b1;
+  segment_blocks(seg, s, M, b0, b1);
+  const int bb0 = b0 + ch * group, bb1 = min(bb0 + group, b1);
+  if (bb0 >= b1) return;  // this segment has fewer chunks (uniform for the whole workgroup)
+  const int rank = seg.rank[s];
+  const T* __restrict__ Bl = (const T*)seg.ptr[s];
+  const int Mrows = seg.table ? seg.n_blocks * ROWS : M;
+  const int n_begin = ns * tiles_per_wg * 64;
+  const int ntiles = min(tiles_per_wg, N / 64 - ns * tiles_per_wg);  // the last slice may be shorter
+  const int total = (bb1 - bb0) * ntiles;                             // (block, tile) pairs, block-major
+
+  auto valid_rows = [&](int b) { return seg.table ? seg.table[3 * b + 1] : min(ROWS, M - b * ROWS); };
+  auto load_b = [&](lf_u32x4 (&br)[NBR], int n0) {
+#pragma unroll
+    for (int i = 0; i < NBR; i++) {
+      const int g = i * 256 + tid;
+      const int row = g / (RT * 2), gc = g % (RT * 2);
+      lf_u32x4 v = {0, 0, 0, 0};
+      if (g < 64 * RT * 2 && gc * 8 < rank) v = *(const lf_u32x4*)(Bl + (int64_t)(n0 + row) * rank + gc * 8);
+      br[i] = v;
+    }
+  };
+  auto store_b = [&](const lf_u32x4 (&br)[NBR], char* dst) {
+#pragma unroll
+    for (int i = 0; i < NBR; i++) {
+      const int g = i * 256 + tid;
+      if (g < 64 * RT * 2) *(lf_u32x4*)(dst + (g / (RT * 2)) * RP + (g % (RT * 2)) * 16) = br[i];
+    }
+  };
+  // S block of row block b (rows beyond its valid count as zeros, so they add nothing to dB).  S has R columns; R may
+  // be smaller than the RT * 16 columns of the register tiling (R = 48, 80, 96, 112)
+  auto load_s = [&](lf_u32x4 (&sr)[RT], int b) {
+    const int valid = valid_rows(b);
+#pragma unroll
+    for (int i = 0; i < RT; i++) {
+      const int g = i * 256 + tid;
+      const int row = g / (RT * 2), gc = g % (RT * 2);
+      lf_u32x4 v = {0, 0, 0, 0};
+      if (row < valid && gc * 8 < R) v = *(const lf_u32x4*)(S + (int64_t)(b * ROWS + row) * R + gc * 8);
+      sr[i] = v;
+    }
+  };
+  auto store_s = [&](const lf_u32x4 (&sr)[RT]) {
+#pragma unroll
+    for (int i = 0; i < RT; i++) {
+      const int g = i * 256 + tid;
+      *(lf_u32x4*)(ss + (g / (RT * 2)) * RP + (g % (RT * 2)) * 16) = sr[i];
+    }
+  };
+  // coordinates of pair q
+  auto blk_of = [&](int q) { return bb0 + q / ntiles; };
+  auto col_of = [&](int q) { return n_begin + (q % ntiles) * 64; };
+
+  TileRegs tr;
+  lf_u32x4 br[NBR], sr[RT];
+  tile_load(tr, dY, (const uint8_t*)nullptr, N, bb0 * ROWS, Mrows, n_begin, tid, false);
+  load_b(br, n_begin);
+  load_s(sr, bb0);
+  store_s(sr);
+  tile_store(tr, ys, tid, false);
+  store_b(br, bs);
+  if (total > 1) {
+    tile_load(tr, dY, (const uint8_t*)nullptr, N, blk_of(1) * ROWS, Mrows, col_of(1), tid, false);
+    load_b(br, col_of(1));
+    if (ntiles == 1) load_s(sr, blk_of(1));
+  }
+  __syncthreads();
+
+  lf_f32x4 acc_db[TPW][RT];
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int c = 0; c < RT; c++) acc_db[t][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  int q = 0;
+  for (int b = bb0; b < bb1; b++) {
+    lf_f32x4 acc_ds[2][RT];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+      for (int c = 0; c < RT; c++) acc_ds[a][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < TPW; t++) {
+      if (t < ntiles) {
+        const char* ycur = ys + (q & 1) * TILE_BYTES;
+        const char* bcur = bs + (q & 1) * 64 * RP;
+        // dS += dY_tile * B_tile : a = dY row fragment, b = B^T through the transpose read
+#pragma unroll
+        for (int step = 0; step < 2; step++) {
+          lf_u32x4 yf[2];
+#pragma unroll
+          for (int rt = 0; rt < 2; rt++) yf[rt] = tile_row_frag(ycur, wave * 32 + rt * 16 + li, step * 4 + qq);
+#pragma unroll
+          for (int c = 0; c < RT; c++) {
+            const lf_u32x4 bf = tr_read8(bcur + (step * 32 + qq * 8 + j4) * RP + (c * 16 + 4 * c4) * 2, RP);
+#pragma unroll
+            for (int rt = 0; rt < 2; rt++) acc_ds[rt][c] = Mfma16<T>::run(yf[rt], bf, acc_ds[rt][c]);
+          }
+        }
+        // dB tile: D[n][r] += sum_m dY[m][n] S[m][r]; wave w owns columns 16w..16w+15 of the tile
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+          const int mrow = kk * 32 + qq * 8 + j4;
+          const lf_u32x4 yt = tile_tr_frag(ycur, mrow, wave * 16 + 4 * c4);
+#pragma unroll
+          for (int c = 0; c < RT; c++) {
+            const lf_u32x4 sf = tr_read8(ss + mrow * RP + (c * 16 + 4 * c4) * 2, RP);
+            acc_db[t][c] = Mfma16<T>::run(yt, sf, acc_db[t][c]);
+          }
+        }
+        if (q + 1 < total) {
+          if (t + 1 == ntiles) {  // the next pair opens a new block: everyone is done with this block's S
+            __syncthreads();
+            store_s(sr);
+          }
+          tile_store(tr, ys + ((q + 1) & 1) * TILE_BYTES, tid, false);
+          store_b(br, bs + ((q + 1) & 1) * 64 * RP);
+          if (q + 2 < total) {
+            tile_load(tr, dY, (const uint8_t*)nullptr, N, blk_of(q + 2) * ROWS, Mrows, col_of(q + 2), tid, false);
+            load_b(br, col_of(q + 2));
+            if ((q + 2) % ntiles == 0) load_s(sr, blk_of(q + 2));
+          }
+        }
+        __syncthreads();
+        q++;
+      }
+    }
+    float* dso = ds_part + (int64_t)ns * Mrows * R;
+#pragma unroll
+    for (int rt = 0; rt < 2; rt++)
+#pragma unroll
+      for (int c = 0; c < RT; c++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int row = b * ROWS + wave * 32 + rt * 16 + qq * 4 + e;
+          if (row < Mrows && c * 16 < R) dso[(int64_t)row * R + c * 16 + li] = acc_ds[rt][c][e];
+        }
+  }
+  // C layout: column (r) = lane & 15, rows (n) = 4*(lane >> 4) + e
+  float* dbo = db_part + (((int64_t)s * max_chunks + ch) * N + n_begin) * R;
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+    if (t < ntiles) {
+#pragma unroll
+      for (int c = 0; c < RT; c++)
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (c * 16 < R) dbo[(int64_t)(t * 64 + wave * 16 + qq * 4 + e) * R + c * 16 + li] = acc_db[t][c][e];
+    }
+}
+
 // out_s = cast( mult * sum over parts of part[...] ) for segment s = blockIdx.y.
-//   transposed == 0 (dB): parts are the segment's blocks, part[b][n][R] -> out [rows, rank]
+//   transposed == 0 (dB): parts are the segment's chunks, part[(s*max_chunks + ch)][n][R] -> out [rows, rank]
 //   transposed == 1 (dA): parts are the segment's chunks, part[(s*max_chunks + ch)][R][rows] -> out [rank, rows]
 //   mult_mode 0: segment scale ; 1: 1/(1-p) of the segment ; 2: none (no keep-mask was given: no dropout).
 template <typename T>
@@ -496,12 +546,12 @@ __device__ __forceinline__ void reduce_segments_body(int bx, int s, const float*
                           : ((seg.block_p && seg.block_p[b0] > 0.f) ? 1.f / (1.f - seg.block_p[b0]) : 1.f);
   }
   lf_f32x4 v;
+  const int nch = (b1 - b0 + group - 1) / group;
   if (!transposed) {
     const int n = (int)(idx / rank), r = (int)(idx % rank);
-    v = sum_parts(part + (int64_t)b0 * rows * R + (int64_t)n * R + r, (int64_t)rows * R, b1 - b0);
+    v = sum_parts(part + (int64_t)s * max_chunks * rows * R + (int64_t)n * R + r, (int64_t)rows * R, nch);
   } else {
     const int r = (int)(idx / rows), k = (int)(idx % rows);
-    const int nch = (b1 - b0 + group - 1) / group;
     v = sum_parts(part + (int64_t)s * max_chunks * R * rows + (int64_t)r * rows + k, (int64_t)R * rows, nch);
   }
   *(lf_u32x2*)((uint16_t*)seg.out[s] + idx) = pack4<T>(v * mult);
@@ -519,13 +569,13 @@ reduce_segments_kernel(const float* __restrict__ part, int rows, int R, int tran
 template <typename T>
 __global__ void __launch_bounds__(256)
 reduce_ds_db_kernel(const float* __restrict__ ds_part, T* __restrict__ dS, int nparts, int M, int R, int nb_rows,
-                    const float* __restrict__ db_part, int N, int nb_seg, const LfSegTable seg) {
+                    const float* __restrict__ db_part, int N, int nb_seg, int group, int max_chunks, const LfSegTable seg) {
   const int b = blockIdx.x;
   if (b < nb_rows) {
     reduce_rows_body<T>(b, ds_part, dS, nparts, M, R, 1, seg);
   } else {
     const int c = b - nb_rows;
-    reduce_segments_body<T>(c % nb_seg, c / nb_seg, db_part, N, R, 0, 0, M, 1, 1, seg);
+    reduce_segments_body<T>(c % nb_seg, c / nb_seg, db_part, N, R, 0, 0, M, group, max_chunks, seg);
   }
 }
 
@@ -651,10 +701,45 @@ static int lds_slots(int smem_bytes) {
   return 256 * (per_cu > 0 ? per_cu : 1);
 }
 static int dys_smem(int rt) { return 2 * TILE_BYTES + ROWS * (rt * 32 + 32) + 2 * 64 * (rt * 32 + 32); }
-// 64-column dY tiles per workgroup; slices per row block = ceil((N/64) / t)
-static int dys_tiles_per_wg(int nblk, int N, int R) {
-  const int T = N / 64;
-  return pick_tiles_per_wg(T, lds_slots(dys_smem(rt_of(R))), [&](int t) { return (long)nblk * ((T + t - 1) / t); });
+// Shape of a dys_dyb launch: tiles per workgroup (<= the kernel's TPW), row blocks per chunk, chunks of the longest
+// segment.  Chosen by bytes moved: the dY stream counted in whole rounds of resident workgroups (a partly filled
+// round streams as long as a full one) plus the fp32 partial sums, written by the first stage and read by the second:
+// dS partials grow with the number of N slices, dB partials with the number of chunks.
+constexpr int dys_tpw(int rt) { return rt <= 2 ? 16 : rt == 4 ? 6 : 4; }   // dB accumulators: TPW * RT * 4 registers, next to 8 * RT of dS
+struct DysPlan { int tiles_per_wg, group, max_chunks, nsplit; };
+static DysPlan dys_plan(int M, int N, int R, const LfSegTable& seg) {
+  const int rt = rt_of(R), T = N / 64, nseg = seg.table ? seg.n_seg : 1;
+  const int nblk = n_row_blocks(M, seg);
+  const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
+  int blocks[LF_MAX_SEG];
+  for (int s = 0; s < nseg; s++) {
+    const int b0 = seg.table ? seg.first_block[s] : 0;
+    const int b1 = seg.table ? ((s + 1 < nseg) ? seg.first_block[s + 1] : seg.n_blocks) : nblk;
+    blocks[s] = b1 - b0;
+  }
+  // two workgroups per CU from rank 32 on (registers), else what the LDS footprint allows
+  const int slots = rt >= 8 ? 256 : rt >= 2 ? 512 : lds_slots(dys_smem(rt));
+  DysPlan best{1, 1, 1, T};
+  double best_cost = 1e300;
+  for (int t = 1; t <= dys_tpw(rt) && t <= T; t++) {
+    const int nsplit = (T + t - 1) / t;
+    for (int g = 1; g <= 32; g *= 2) {
+      long chunks = 0;
+      int max_chunks = 1;
+      for (int s = 0; s < nseg; s++) {
+        const int c = (blocks[s] + g - 1) / g;
+        chunks += c;
+        max_chunks = c > max_chunks ? c : max_chunks;
+      }
+      const long wgs = chunks * nsplit;
+      const double rounds = (double)((wgs + slots - 1) / slots);
+      const double stream = rounds * slots * g * t * (double)TILE_BYTES;
+      const double partial = 2.0 * 4.0 * R * ((double)nsplit * rows + (double)nseg * max_chunks * N);
+      const double cost = stream + partial;
+      if (cost < best_cost) { best_cost = cost; best = DysPlan{t, g, max_chunks, nsplit}; }
+    }
+  }
+  return best;
 }
 
 size_t lf_xa_workspace(int, int, int, const LfSegTable&) { return 0; }
@@ -698,48 +783,46 @@ int lf_launch_xa(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t
 size_t lf_dys_dyb_workspace(int M, int N, int R, const LfSegTable& seg) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  const int t = dys_tiles_per_wg(nblk, N, R);
-  const int nsl = (N / 64 + t - 1) / t;
-  return ((size_t)nsl * rows * R + (size_t)nblk * N * R) * sizeof(float);
+  const int nseg = seg.table ? seg.n_seg : 1;
+  const DysPlan pl = dys_plan(M, N, R, seg);
+  return ((size_t)pl.nsplit * rows * R + (size_t)nseg * pl.max_chunks * N * R) * sizeof(float);
 }
 
 template <typename T, int RT>
-static int dys_launch(const void* dY, const void* S, float* ds_part, float* db_part, int M, int N, int R, int tiles_per_wg,
+static int dys_launch(const void* dY, const void* S, float* ds_part, float* db_part, int M, int N, int R, const DysPlan& pl,
                       dim3 grid, const LfSegTable& seg, hipStream_t st) {
-  auto kern = lora_dys_dyb_kernel<T, RT>;
-  constexpr int RP = RT * 32 + 32;
+  auto kern = lora_dys_dyb_kernel<T, RT, dys_tpw(RT)>;
   const int smem = dys_smem(RT);
-  static_assert(RP == RT * 32 + 32, "");
   static LfLdsFlags lds_ok;
   if (!lf_allow_lds(kern, smem, lds_ok)) return LF_ELAUNCH;
-  return lf_launch(kern, grid, dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, tiles_per_wg, seg);
+  return lf_launch(kern, grid, dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R, pl.tiles_per_wg,
+                   pl.group, pl.max_chunks, seg);
 }
 
 template <typename T>
 static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M, int N, int R, const LfSegTable& seg, hipStream_t st) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
-  const int nslice = dys_tiles_per_wg(nblk, N, R);       // tiles per workgroup
-  const int split = (N / 64 + nslice - 1) / nslice;       // slices per row block = partial sums of dS
-  float* ds_part = (float*)ws;
-  float* db_part = ds_part + (int64_t)split * rows * R;
-  dim3 grid(nblk, split);
+  const int nseg = seg.table ? seg.n_seg : 1;
+  const DysPlan pl = dys_plan(M, N, R, seg);
+  float* ds_part = (float*)ws;                                   // [nsplit][rows][R]
+  float* db_part = ds_part + (int64_t)pl.nsplit * rows * R;      // [nseg * max_chunks][N][R]
+  dim3 grid(nseg * pl.max_chunks, pl.nsplit);
   int rc;
   switch (rt_of(R)) {
-    case 1: rc = dys_launch<T, 1>(dY, S, ds_part, db_part, M, N, R, nslice, grid, seg, st); break;
-    case 2: rc = dys_launch<T, 2>(dY, S, ds_part, db_part, M, N, R, nslice, grid, seg, st); break;
-    case 4: rc = dys_launch<T, 4>(dY, S, ds_part, db_part, M, N, R, nslice, grid, seg, st); break;
-    default: rc = dys_launch<T, 8>(dY, S, ds_part, db_part, M, N, R, nslice, grid, seg, st); break;
+    case 1: rc = dys_launch<T, 1>(dY, S, ds_part, db_part, M, N, R, pl, grid, seg, st); break;
+    case 2: rc = dys_launch<T, 2>(dY, S, ds_part, db_part, M, N, R, pl, grid, seg, st); break;
+    case 4: rc = dys_launch<T, 4>(dY, S, ds_part, db_part, M, N, R, pl, grid, seg, st); break;
+    default: rc = dys_launch<T, 8>(dY, S, ds_part, db_part, M, N, R, pl, grid, seg, st); break;
   }
   if (rc != LF_OK) return rc;
   const int64_t n = rows * R;
-  const int nseg = seg.table ? seg.n_seg : 1;
   int maxrank = 0;
   for (int s = 0; s < nseg; s++) maxrank = seg.rank[s] > maxrank ? seg.rank[s] : maxrank;
   const int64_t nout = (int64_t)N * maxrank;
   const int nb_rows = (int)((n + 1023) / 1024), nb_seg = (int)((nout + 1023) / 1024);  // four outputs per thread
   return lf_launch((reduce_ds_db_kernel<T>), dim3((unsigned)(nb_rows + nb_seg * nseg)), dim3(256), 0, st, (const float*)ds_part,
-                     (T*)dS, split, M, R, nb_rows, (const float*)db_part, N, nb_seg, seg);
+                     (T*)dS, pl.nsplit, M, R, nb_rows, (const float*)db_part, N, nb_seg, pl.group, pl.max_chunks, seg);
 }
 
 int lf_launch_dys_dyb(const void* dY, const void* S, void* dS, void* ws, size_t ws_bytes, int M, int N, int R,
