@@ -346,6 +346,16 @@ __device__ __forceinline__ void segment_blocks(const LfSegTable& seg, int s, int
   }
 }
 
+// Chunk ch of the blocks [b0, b1) when they are cut into ceil((b1 - b0) / group) chunks of nearly equal size (empty
+// beyond the last chunk).
+__device__ __forceinline__ void chunk_blocks(int b0, int b1, int group, int ch, int& bb0, int& bb1) {
+  const int n = b1 - b0, nch = (n + group - 1) / group;
+  if (n <= 0 || ch >= nch) { bb0 = bb1 = b1; return; }
+  const int base = n / nch, rem = n % nch;
+  bb0 = b0 + ch * base + min(ch, rem);
+  bb1 = bb0 + base + (ch < rem ? 1 : 0);
+}
+
 // ------------------------------------------------------------------------------- dys_dyb
 // grid (n_seg * max_chunks, nsplit).  Workgroup (s, ch, ns) owns the `group` consecutive 128-row blocks ch*group.. of
 // segment s and the N slice ns (tiles_per_wg <= TPW tiles of 64 columns); it walks its blocks, and per block the
@@ -673,6 +683,398 @@ lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const 
       if (c * 16 < R) po[(int64_t)(c * 16 + qq * 4 + e) * K + kt * 64 + wave * 16 + li] = acc[c][e];  // the partial has R rows
 }
 
+// ------------------------------------------------------------------ streaming through a ring of direct-to-LDS loads
+// The passes above keep one tile per workgroup in flight (it waits in registers between its load and its LDS store);
+// the LDS footprint allows two or three workgroups per CU, so a CU has 32-48 KB on order -- half of what the HBM
+// latency asks for, less at rank 64.  The kernels below (ranks up to 64) order their tiles as buffer loads that
+// write LDS themselves (no registers, no store instructions), NS - 1 tiles ahead of the one being consumed.
+//
+// A load group is waited for by count: vector memory operations complete in issue order, so "at most n younger
+// operations outstanding" means the group has landed.  The loop therefore contains no other vector memory
+// instruction (the compiler would count only its own and wait for everything), issues a group of the same size
+// every iteration (past the end: the last tile again, unconsumed), and drains the ring before the workgroup ends.
+// Rows past the end of a matrix are not clamped: every tile gets a buffer descriptor that ends where the matrix
+// ends, and lanes beyond it read zeros, which add nothing to a sum over rows.
+__device__ __forceinline__ uint32_t to_sgpr(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
+__device__ __forceinline__ lf_u32x4 window_rsrc(const void* base, int64_t bytes) {
+  const uint64_t a = (uint64_t)(uintptr_t)base;
+  const int64_t n = bytes > 0xffffffffll ? 0xffffffffll : bytes;   // (never negative: a window starts inside its matrix)
+  return lf_u32x4{to_sgpr((uint32_t)a), to_sgpr((uint32_t)(a >> 32)) & 0xffffu, to_sgpr((uint32_t)n), 0x00020000u};
+}
+// one wave instruction: lane l fetches 16 bytes at window offset `voff` into LDS byte lds_addr + 16 l
+__device__ __forceinline__ void dma16(const lf_u32x4& rsrc, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// at most `groups` groups of G operations each may still be outstanding
+template <int G>
+__device__ __forceinline__ void wait_groups(int groups) {
+  switch (groups) {
+    case 0: wait_vm<0>(); break;
+    case 1: wait_vm<G>(); break;
+    case 2: wait_vm<2 * G>(); break;
+    case 3: wait_vm<3 * G>(); break;
+    default: wait_vm<4 * G>(); break;
+  }
+}
+__device__ __forceinline__ void ring_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// Per-thread window offsets of a 128-row x 64-column tile of a 16-bit matrix with `ld` elements per row, in the LDS
+// layout the fragment readers expect (position p = i*256 + tid: row p>>3, slot p&7 holds granule slot ^ ((row>>1)&7)).
+__device__ __forceinline__ void tile_voffs(uint32_t (&v)[4], int64_t ld, int tid) {
+  const int srcg = (tid & 7) ^ ((tid >> 4) & 7);
+#pragma unroll
+  for (int i = 0; i < 4; i++) v[i] = (uint32_t)((int64_t)(i * 32 + (tid >> 3)) * ld * 2 + srcg * 16);
+}
+__device__ __forceinline__ void tile_dma(const lf_u32x4& rsrc, const uint32_t (&v)[4], uint32_t lds_tile, int wave) {
+#pragma unroll
+  for (int i = 0; i < 4; i++) dma16(rsrc, v[i], lds_tile + i * 4096 + wave * 1024);
+}
+// keep-mask bytes of the same tile: 128 rows of 64 bytes, row-major (position p = i*256 + tid: row p>>2, 16-byte chunk p&3)
+__device__ __forceinline__ void mask_voffs(uint32_t (&v)[2], int64_t ld, int tid) {
+#pragma unroll
+  for (int i = 0; i < 2; i++) v[i] = (uint32_t)((int64_t)(i * 64 + (tid >> 2)) * ld + (tid & 3) * 16);
+}
+__device__ __forceinline__ void mask_dma(const lf_u32x4& rsrc, const uint32_t (&v)[2], uint32_t lds_mask, int wave) {
+#pragma unroll
+  for (int i = 0; i < 2; i++) dma16(rsrc, v[i], lds_mask + i * 4096 + wave * 1024);
+}
+// keep-mask applied in place to a landed tile (any thread mapping; here each thread takes the positions p = i*256 + tid)
+__device__ __forceinline__ void tile_apply_mask(char* tile, const char* mtile, int tid) {
+  lf_u32x4 x[4];
+  lf_u32x2 m[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {   // all reads first: behind a store the compiler would not start the next read
+    const int p = i * 256 + tid, row = p >> 3, g = (p & 7) ^ ((row >> 1) & 7);
+    x[i] = *(const lf_u32x4*)(tile + p * 16);
+    m[i] = *(const lf_u32x2*)(mtile + row * 64 + g * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) *(lf_u32x4*)(tile + (i * 256 + tid) * 16) = apply_mask8(x[i], m[i]);
+}
+
+// A [rows x RT*16] side operand (S or dS block: 128 rows; B tile: 64 rows) in LDS: rows of RT*32 bytes, granule g of
+// row r at slot g ^ key(r).  A transpose read is served 16 lanes at a time: four consecutive rows, 32 bytes of each,
+// which the key puts on four different quarters of the 32 banks (at 32-byte rows they are there already).
+template <int RT>
+__device__ __forceinline__ int side_key(int row) { return RT >= 4 ? (row & 3) << 1 : RT == 2 ? ((row >> 1) & 1) << 1 : 0; }
+// window offsets of the granules this thread fetches: position p = i*256 + tid -> row p / (2 RT), slot p % (2 RT); a
+// granule beyond `cols` columns does not exist in memory: the first one is fetched instead (its products land in
+// rank columns that the reduce discards)
+template <int RT, int NI>
+__device__ __forceinline__ void side_voffs(uint32_t (&v)[NI], int pitch_elems, int cols, int tid) {
+#pragma unroll
+  for (int i = 0; i < NI; i++) {
+    const int p = i * 256 + tid, row = p / (RT * 2), g = (p % (RT * 2)) ^ side_key<RT>(row);
+    v[i] = (uint32_t)(row * pitch_elems * 2 + (g * 8 < cols ? g : 0) * 16);
+  }
+}
+template <int NI>
+__device__ __forceinline__ void side_dma(const lf_u32x4& rsrc, const uint32_t (&v)[NI], uint32_t lds_side, int wave) {
+#pragma unroll
+  for (int i = 0; i < NI; i++) dma16(rsrc, v[i], lds_side + i * 4096 + wave * 1024);
+}
+// transposed fragment: rows row..row+3 and row+4..row+7 of the lane's column among columns c*16 + 4*c4 .. (row and
+// row + 4 share their key)
+template <int RT>
+__device__ __forceinline__ lf_u32x4 side_tr8(const char* blk, int row, int c, int c4) {
+  const int g = c * 2 + (c4 >> 1);
+  return tr_read8(blk + row * (RT * 32) + ((g ^ side_key<RT>(row)) << 4) + (c4 & 1) * 8, RT * 32);
+}
+
+// ---- da.  grid (n_slices, max_chunks, n_seg).  Workgroup (ks, ch, s): the k-tiles of slice ks (at most TPW, at least
+// two: slices are balanced) and the `group` row blocks ch*group.. of segment s; pairs (block, tile) in block-major
+// order, the dS block of a row block is fetched once, with the block's first tile, into one of two buffers (a slice
+// of nt tiles keeps at most min(NS, nt + 1) stages of the ring busy, so a third block is never on order).
+//   D_j[r][k] += sum_m dS[m][r] * keep*X[m][k]   per tile j of the slice, in registers over all blocks of the chunk.
+// With a keep-mask the tile is masked in place one iteration before it is consumed.
+template <typename T, int RT, int TPW, int NS, bool MASK>
+__global__ void __launch_bounds__(256, 2)
+lora_da_ring_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const T* __restrict__ dS, float* __restrict__ part,
+                    int M, int K, int R, int n_slices, int group, int max_chunks, const LfSegTable seg) {
+  constexpr int STAGE = TILE_BYTES + (MASK ? ROWS * 64 : 0);
+  constexpr int SIDE = ROWS * RT * 32;
+  constexpr int G = 4 + (MASK ? 2 : 0);   // operations per load group and thread, not counting a dS block
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  char* ring = lds;
+  char* side = lds + NS * STAGE;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const int ks = blockIdx.x, ch = blockIdx.y, s = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = to_sgpr(tid >> 6);
+  const int li = lane & 15, qq = lane >> 4, j4 = li >> 2, c4 = li & 3;
+  int b0, b1, bb0, bb1;
+  segment_blocks(seg, s, M, b0, b1);
+  chunk_blocks(b0, b1, group, ch, bb0, bb1);
+  if (bb0 >= bb1) return;  // this segment has fewer chunks (uniform for the whole workgroup)
+  const float p = seg.table ? (seg.block_p ? seg.block_p[b0] : 0.f) : seg.p;
+  const bool use_mask = MASK && mask != nullptr && p > 0.f;
+  const int64_t Mrows = seg.table ? (int64_t)seg.n_blocks * ROWS : M;
+  const int T64 = K / 64;
+  const int kt0 = ks * (T64 / n_slices) + min(ks, T64 % n_slices);
+  const int nt = T64 / n_slices + (ks < T64 % n_slices ? 1 : 0);
+  const int ns = min(NS, nt + 1);   // stages in use
+
+  uint32_t xv[4], mv[2], dv[RT];
+  tile_voffs(xv, K, tid);
+  mask_voffs(mv, K, tid);
+  side_voffs<RT, RT>(dv, R, R, tid);
+
+  // Load group of the next pair into stage `ist`; behind the last pair the last tile is ordered again.  The windows
+  // move with the pair (byte pointers and bytes left up to the end of the matrix): a few scalar additions per group.
+  int ib = bb0, ij = 0, ist = 0;
+  const char* xb = (const char*)(X + (int64_t)bb0 * ROWS * K + (int64_t)kt0 * 64);
+  int64_t xleft = (((int64_t)Mrows - (int64_t)bb0 * ROWS) * K - (int64_t)kt0 * 64) * 2;
+  const char* sb = (const char*)(dS + (int64_t)bb0 * ROWS * R);
+  int64_t sleft = ((int64_t)Mrows - (int64_t)bb0 * ROWS) * R * 2;
+  const int64_t xnext = (int64_t)ROWS * K * 2 - (int64_t)nt * 128;   // from behind a block's last tile to the next block's first
+  auto issue = [&]() {
+    tile_dma(window_rsrc(xb, xleft), xv, lds0 + ist * STAGE, wave);
+    if constexpr (MASK) {
+      // the mask has one byte where X has two: same element offsets, half the byte offsets
+      const int64_t eoff = (xb - (const char*)X) >> 1;
+      mask_dma(window_rsrc(mask != nullptr ? (const char*)mask + eoff : (const char*)X, mask != nullptr ? (xleft >> 1) : 0), mv,
+               lds0 + ist * STAGE + TILE_BYTES, wave);
+    }
+    if (ij == 0 && ib < bb1) side_dma<RT>(window_rsrc(sb, sleft), dv, lds0 + NS * STAGE + ((ib - bb0) & 1) * SIDE, wave);
+    ist = ist + 1 == ns ? 0 : ist + 1;
+    if (ib < bb1) {
+      if (++ij < nt) {
+        xb += 128, xleft -= 128;
+      } else if (ib + 1 < bb1) {
+        ij = 0, ib++;
+        xb += 128 + xnext, xleft -= 128 + xnext;
+        sb += ROWS * R * 2, sleft -= ROWS * R * 2;
+      } else {
+        ib = bb1;   // the cursor stays on the last tile
+      }
+    }
+  };
+#pragma unroll 1
+  for (int i = 0; i < ns - 1; i++) issue();
+
+  lf_f32x4 acc[TPW][RT];
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int c = 0; c < RT; c++) acc[t][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  int cst = 0;   // stage of the pair being consumed
+  if constexpr (MASK) {
+    wait_groups<G>(ns - 2);
+    ring_barrier();
+    if (use_mask) tile_apply_mask(ring, ring + TILE_BYTES, tid);
+  }
+  for (int b = bb0; b < bb1; b++) {
+    const char* dcur = side + ((b - bb0) & 1) * SIDE;
+    lf_u32x4 df[4][RT];
+#pragma unroll
+    for (int t = 0; t < TPW; t++) {
+      if (t < nt) {
+        // MASK: the next pair's group has landed (it is masked during this iteration); else this pair's
+        wait_groups<G>(MASK ? ns - 3 : ns - 2);
+        ring_barrier();   // ... for every thread; and everyone is done with the previous pair's stage
+        issue();
+        if constexpr (MASK) {
+          const int nst = cst + 1 == ns ? 0 : cst + 1;
+          if (use_mask) tile_apply_mask(ring + nst * STAGE, ring + nst * STAGE + TILE_BYTES, tid);
+        }
+        const char* xcur = ring + cst * STAGE;
+        // all fragments of the tile first, then the MFMAs: with one or two waves per SIMD nothing else hides the LDS
+        // latency, and read-wait-multiply in turns costs a latency per MFMA
+        lf_u32x4 xt[4];
+        if (t == 0) {   // the dS fragments serve every tile of the block
+#pragma unroll
+          for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+            for (int c = 0; c < RT; c++) df[kk][c] = side_tr8<RT>(dcur, kk * 32 + qq * 8 + j4, c, c4);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) xt[kk] = tile_tr_frag(xcur, kk * 32 + qq * 8 + j4, wave * 16 + 4 * c4);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+          for (int c = 0; c < RT; c++) acc[t][c] = Mfma16<T>::run(df[kk][c], xt[kk], acc[t][c]);
+        __builtin_amdgcn_sched_barrier(0);
+        cst = cst + 1 == ns ? 0 : cst + 1;
+      }
+    }
+  }
+  wait_vm<0>();   // the unconsumed loads behind the last pair must not land in another workgroup's LDS
+  // C layout: column (k) = lane & 15, rows (r) = 4*(lane >> 4) + e
+  float* po = part + ((int64_t)s * max_chunks + ch) * R * K;
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+    if (t < nt) {
+#pragma unroll
+      for (int c = 0; c < RT; c++)
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (c * 16 < R) po[(int64_t)(c * 16 + qq * 4 + e) * K + (kt0 + t) * 64 + wave * 16 + li] = acc[t][c][e];
+    }
+}
+
+// ---- dys_dyb.  grid (n_seg * max_chunks, n_slices).  Workgroup (s, ch, ns): the tiles of N slice ns (balanced, 2 .. TPW
+// tiles) and chunk ch of segment s (chunks are balanced too); pairs (block, tile) in block-major order.  A load group
+// is the dY tile and its B tile [64, rank]; the S block of a row block comes with the block's first tile, into one of
+// two buffers.  Per pair:
+//   dS partial [128, R] += dY_tile * B_tile      (registers over the slice; stored when the block ends)
+//   dB partial [64, R]  += dY_tile^T * S_block    (registers over ALL blocks of the chunk; stored at the end)
+// The stores of a block's dS partial are vector memory operations like the loads: the group counts that follow them
+// wait for more than they must (the ring runs empty once per block), never for less.
+template <typename T, int RT, int TPW, int NS>
+__global__ void __launch_bounds__(256, RT >= 4 ? 1 : 2)
+lora_dys_dyb_ring_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __restrict__ ds_part, float* __restrict__ db_part,
+                         int M, int N, int R, int n_slices, int group, int max_chunks, const LfSegTable seg) {
+  constexpr int NIB = RT >= 2 ? RT / 2 : 1;         // B tile: 64 rows of RT*32 bytes (a 4 KB region at rank 16: all threads fetch)
+  constexpr int BT = NIB * 4096;
+  constexpr int STAGE = TILE_BYTES + BT;
+  constexpr int SIDE = ROWS * RT * 32;
+  constexpr int G = 4 + NIB;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  char* ring = lds;
+  char* side = lds + NS * STAGE;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const int s = blockIdx.x / max_chunks, ch = blockIdx.x % max_chunks, sl = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = to_sgpr(tid >> 6);
+  const int li = lane & 15, qq = lane >> 4, j4 = li >> 2, c4 = li & 3;
+  int b0, b1, bb0, bb1;
+  segment_blocks(seg, s, M, b0, b1);
+  chunk_blocks(b0, b1, group, ch, bb0, bb1);
+  if (bb0 >= bb1) return;  // this segment has fewer chunks (uniform for the whole workgroup)
+  const int rank = seg.rank[s];
+  const T* __restrict__ Bl = (const T*)seg.ptr[s];
+  const int64_t Mrows = seg.table ? (int64_t)seg.n_blocks * ROWS : M;
+  const int T64 = N / 64;
+  const int t0 = sl * (T64 / n_slices) + min(sl, T64 % n_slices);
+  const int nt = T64 / n_slices + (sl < T64 % n_slices ? 1 : 0);
+  const int ns = min(NS, nt + 1);   // stages in use
+
+  uint32_t yv[4], bv[NIB], sv[RT];
+  tile_voffs(yv, N, tid);
+  side_voffs<RT, NIB>(bv, rank, rank, tid);
+  side_voffs<RT, RT>(sv, R, R, tid);
+
+  // Load group of the next pair into stage `ist`; behind the last pair the last tile is ordered again.  The windows
+  // move with the pair (byte pointers and bytes left up to the end of the matrix): a few scalar additions per group.
+  int ib = bb0, ij = 0, ist = 0;
+  const char* yb = (const char*)(dY + (int64_t)bb0 * ROWS * N + (int64_t)t0 * 64);
+  int64_t yleft = (((int64_t)Mrows - (int64_t)bb0 * ROWS) * N - (int64_t)t0 * 64) * 2;
+  const char* bp = (const char*)(Bl + (int64_t)t0 * 64 * rank);
+  int64_t bleft = ((int64_t)N - (int64_t)t0 * 64) * rank * 2;
+  const char* sb = (const char*)(S + (int64_t)bb0 * ROWS * R);
+  int64_t sleft = ((int64_t)Mrows - (int64_t)bb0 * ROWS) * R * 2;
+  const int64_t ynext = (int64_t)ROWS * N * 2 - (int64_t)nt * 128;   // from behind a block's last tile to the next block's first
+  const int64_t bstep = (int64_t)64 * rank * 2;
+  auto issue = [&]() {
+    tile_dma(window_rsrc(yb, yleft), yv, lds0 + ist * STAGE, wave);
+    side_dma<NIB>(window_rsrc(bp, bleft), bv, lds0 + ist * STAGE + TILE_BYTES, wave);
+    if (ij == 0 && ib < bb1) side_dma<RT>(window_rsrc(sb, sleft), sv, lds0 + NS * STAGE + ((ib - bb0) & 1) * SIDE, wave);
+    ist = ist + 1 == ns ? 0 : ist + 1;
+    if (ib < bb1) {
+      if (++ij < nt) {
+        yb += 128, yleft -= 128;
+        bp += bstep, bleft -= bstep;
+      } else if (ib + 1 < bb1) {
+        ij = 0, ib++;
+        yb += 128 + ynext, yleft -= 128 + ynext;
+        bp -= (nt - 1) * bstep, bleft += (nt - 1) * bstep;
+        sb += ROWS * R * 2, sleft -= ROWS * R * 2;
+      } else {
+        ib = bb1;   // the cursor stays on the last tile
+      }
+    }
+  };
+#pragma unroll 1
+  for (int i = 0; i < ns - 1; i++) issue();
+
+  lf_f32x4 acc_db[TPW][RT];
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int c = 0; c < RT; c++) acc_db[t][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  int cst = 0;
+  for (int b = bb0; b < bb1; b++) {
+    const char* scur = side + ((b - bb0) & 1) * SIDE;
+    lf_f32x4 acc_ds[2][RT];
+    lf_u32x4 sf[4][RT];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+      for (int c = 0; c < RT; c++) acc_ds[a][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < TPW; t++) {
+      if (t < nt) {
+        wait_groups<G>(ns - 2);
+        ring_barrier();
+        issue();
+        const char* ycur = ring + cst * STAGE;
+        const char* bcur = ycur + TILE_BYTES;
+        // All fragments of the tile first, then the MFMAs (one wave per SIMD at rank 64: nothing else hides the LDS
+        // latency).  dS += dY_tile * B_tile: a = dY row fragment, b = B^T through the transpose read; dB tile:
+        // D[n][r] += sum_m dY[m][n] S[m][r], wave w owns columns 16w..16w+15 of the tile
+        lf_u32x4 yf[2][2], bf[2][RT], yt[4];
+        if (t == 0) {   // the S fragments serve every tile of the block
+#pragma unroll
+          for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+            for (int c = 0; c < RT; c++) sf[kk][c] = side_tr8<RT>(scur, kk * 32 + qq * 8 + j4, c, c4);
+        }
+#pragma unroll
+        for (int step = 0; step < 2; step++) {
+#pragma unroll
+          for (int rt = 0; rt < 2; rt++) yf[step][rt] = tile_row_frag(ycur, wave * 32 + rt * 16 + li, step * 4 + qq);
+#pragma unroll
+          for (int c = 0; c < RT; c++) bf[step][c] = side_tr8<RT>(bcur, step * 32 + qq * 8 + j4, c, c4);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+          const int mrow = kk * 32 + qq * 8 + j4;
+          yt[kk] = tile_tr_frag(ycur, mrow, wave * 16 + 4 * c4);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int step = 0; step < 2; step++)
+#pragma unroll
+          for (int c = 0; c < RT; c++)
+#pragma unroll
+            for (int rt = 0; rt < 2; rt++) acc_ds[rt][c] = Mfma16<T>::run(yf[step][rt], bf[step][c], acc_ds[rt][c]);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+          for (int c = 0; c < RT; c++) acc_db[t][c] = Mfma16<T>::run(yt[kk], sf[kk][c], acc_db[t][c]);
+        __builtin_amdgcn_sched_barrier(0);
+        cst = cst + 1 == ns ? 0 : cst + 1;
+      }
+    }
+    float* dso = ds_part + (int64_t)sl * Mrows * R;
+#pragma unroll
+    for (int rt = 0; rt < 2; rt++)
+#pragma unroll
+      for (int c = 0; c < RT; c++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int64_t row = (int64_t)b * ROWS + wave * 32 + rt * 16 + qq * 4 + e;
+          if (row < Mrows && c * 16 < R) dso[row * R + c * 16 + li] = acc_ds[rt][c][e];
+        }
+  }
+  wait_vm<0>();   // the unconsumed loads behind the last pair must not land in another workgroup's LDS
+  // C layout: column (r) = lane & 15, rows (n) = 4*(lane >> 4) + e
+  float* dbo = db_part + (((int64_t)s * max_chunks + ch) * N + (int64_t)t0 * 64) * R;
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+    if (t < nt) {
+#pragma unroll
+      for (int c = 0; c < RT; c++)
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (c * 16 < R) dbo[(int64_t)(t * 64 + wave * 16 + qq * 4 + e) * R + c * 16 + li] = acc_db[t][c][e];
+    }
+}
+
 int rt_of(int R) { return R <= 16 ? 1 : R <= 32 ? 2 : R <= 64 ? 4 : 8; }
 
 }  // namespace
@@ -742,6 +1144,69 @@ static DysPlan dys_plan(int M, int N, int R, const LfSegTable& seg) {
   return best;
 }
 
+// ---- work split of the ring kernels.  Workgroups (slice x chunk) of w tiles each run on `slots` resident slots; the
+// pass lasts about as long as its busiest slot.  Two upper bounds of that (in tiles): whole rounds of the largest
+// workgroup, and the list-scheduling bound sum / slots + largest; the smaller one is the estimate.
+struct RingSplit { long wgs; long chunks; int max_chunks; double span; };
+static RingSplit ring_split(const int* blocks, int nseg, int g, int T, int nsl, int slots) {
+  RingSplit r{0, 0, 1, 0.0};
+  const int t_max = (T + nsl - 1) / nsl;
+  long total = 0;
+  int big = 0;
+  for (int s = 0; s < nseg; s++) {
+    const int c = (blocks[s] + g - 1) / g;
+    if (c <= 0) continue;
+    r.chunks += c;
+    r.max_chunks = c > r.max_chunks ? c : r.max_chunks;
+    const int sz = (blocks[s] + c - 1) / c;
+    big = sz > big ? sz : big;
+    total += blocks[s];
+  }
+  r.wgs = r.chunks * nsl;
+  const double sum = (double)total * T / slots, largest = (double)big * t_max;
+  const double by_rounds = (double)((r.wgs + slots - 1) / slots) * largest, by_list = sum + largest;
+  r.span = by_rounds < by_list ? by_rounds : by_list;
+  if (r.span < sum) r.span = sum;
+  return r;
+}
+static void seg_block_counts(int M, const LfSegTable& seg, int* blocks, int& nseg) {
+  nseg = seg.table ? seg.n_seg : 1;
+  for (int s = 0; s < nseg; s++) {
+    const int b0 = seg.table ? seg.first_block[s] : 0;
+    const int b1 = seg.table ? ((s + 1 < nseg) ? seg.first_block[s + 1] : seg.n_blocks) : (M + ROWS - 1) / ROWS;
+    blocks[s] = b1 - b0;
+  }
+}
+static const int kGroups[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 64};
+
+constexpr int dysr_tpw(int rt) { return rt >= 2 ? 12 : 16; }
+constexpr int dysr_ns(int rt) { return rt >= 4 ? 5 : 3; }
+static int dysr_smem(int rt) { return dysr_ns(rt) * (TILE_BYTES + (rt >= 2 ? rt / 2 : 1) * 4096) + 2 * ROWS * rt * 32; }
+struct DysRingPlan { int n_slices, group, max_chunks; };
+// By bytes: the dY (+ B tile) stream over the busiest slot, the S blocks every workgroup fetches (from L2: half weight),
+// and the fp32 partials written here and read by the reduce (dS: one [rows, R] slab per slice; dB: one [N, R] slab per
+// chunk).
+static DysRingPlan dysr_plan(int M, int N, int R, const LfSegTable& seg) {
+  const int rt = rt_of(R), T = N / 64;
+  int blocks[LF_MAX_SEG], nseg;
+  seg_block_counts(M, seg, blocks, nseg);
+  const int64_t rows = seg.table ? (int64_t)seg.n_blocks * ROWS : M;
+  const int slots = lds_slots(dysr_smem(rt));
+  const double tile_bytes = TILE_BYTES + 64.0 * R * 2;
+  DysRingPlan best{1, 1, 1};
+  double best_cost = 1e300;
+  for (int nsl = 1; nsl <= T / 2; nsl++) {
+    if ((T + nsl - 1) / nsl > dysr_tpw(rt)) continue;
+    for (int g : kGroups) {
+      const RingSplit sp = ring_split(blocks, nseg, g, T, nsl, slots);
+      const double cost = sp.span * slots * tile_bytes + 0.5 * (double)sp.wgs * g * ROWS * R * 2 +
+                          2.0 * 4.0 * R * ((double)nsl * rows + (double)sp.chunks * N);
+      if (cost < best_cost) { best_cost = cost; best = DysRingPlan{nsl, g, sp.max_chunks}; }
+    }
+  }
+  return best;
+}
+
 size_t lf_xa_workspace(int, int, int, const LfSegTable&) { return 0; }
 
 template <typename T, int RT>
@@ -784,8 +1249,23 @@ size_t lf_dys_dyb_workspace(int M, int N, int R, const LfSegTable& seg) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
   const int nseg = seg.table ? seg.n_seg : 1;
+  if (rt_of(R) <= 4) {
+    const DysRingPlan pl = dysr_plan(M, N, R, seg);
+    return ((size_t)pl.n_slices * rows * R + (size_t)nseg * pl.max_chunks * N * R) * sizeof(float);
+  }
   const DysPlan pl = dys_plan(M, N, R, seg);
   return ((size_t)pl.nsplit * rows * R + (size_t)nseg * pl.max_chunks * N * R) * sizeof(float);
+}
+
+template <typename T, int RT>
+static int dysr_launch(const void* dY, const void* S, float* ds_part, float* db_part, int M, int N, int R, const DysRingPlan& pl,
+                       int nseg, const LfSegTable& seg, hipStream_t st) {
+  auto kern = lora_dys_dyb_ring_kernel<T, RT, dysr_tpw(RT), dysr_ns(RT)>;
+  const int smem = dysr_smem(RT);
+  static LfLdsFlags lds_ok;
+  if (!lf_allow_lds(kern, smem, lds_ok)) return LF_ELAUNCH;
+  return lf_launch(kern, dim3(nseg * pl.max_chunks, pl.n_slices), dim3(256), smem, st, (const T*)dY, (const T*)S, ds_part, db_part, M, N, R,
+                   pl.n_slices, pl.group, pl.max_chunks, seg);
 }
 
 template <typename T, int RT>
@@ -804,16 +1284,23 @@ static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
   const int nseg = seg.table ? seg.n_seg : 1;
-  const DysPlan pl = dys_plan(M, N, R, seg);
-  float* ds_part = (float*)ws;                                   // [nsplit][rows][R]
-  float* db_part = ds_part + (int64_t)pl.nsplit * rows * R;      // [nseg * max_chunks][N][R]
-  dim3 grid(nseg * pl.max_chunks, pl.nsplit);
-  int rc;
-  switch (rt_of(R)) {
-    case 1: rc = dys_launch<T, 1>(dY, S, ds_part, db_part, M, N, R, pl, grid, seg, st); break;
-    case 2: rc = dys_launch<T, 2>(dY, S, ds_part, db_part, M, N, R, pl, grid, seg, st); break;
-    case 4: rc = dys_launch<T, 4>(dY, S, ds_part, db_part, M, N, R, pl, grid, seg, st); break;
-    default: rc = dys_launch<T, 8>(dY, S, ds_part, db_part, M, N, R, pl, grid, seg, st); break;
+  float* ds_part = (float*)ws;   // [slices][rows][R], then the dB partials [nseg * max_chunks][N][R]
+  float* db_part;
+  int rc, nparts, group, max_chunks;
+  if (rt_of(R) <= 4) {
+    const DysRingPlan pl = dysr_plan(M, N, R, seg);
+    db_part = ds_part + (int64_t)pl.n_slices * rows * R;
+    nparts = pl.n_slices, group = pl.group, max_chunks = pl.max_chunks;
+    switch (rt_of(R)) {
+      case 1: rc = dysr_launch<T, 1>(dY, S, ds_part, db_part, M, N, R, pl, nseg, seg, st); break;
+      case 2: rc = dysr_launch<T, 2>(dY, S, ds_part, db_part, M, N, R, pl, nseg, seg, st); break;
+      default: rc = dysr_launch<T, 4>(dY, S, ds_part, db_part, M, N, R, pl, nseg, seg, st); break;
+    }
+  } else {
+    const DysPlan pl = dys_plan(M, N, R, seg);
+    db_part = ds_part + (int64_t)pl.nsplit * rows * R;
+    nparts = pl.nsplit, group = pl.group, max_chunks = pl.max_chunks;
+    rc = dys_launch<T, 8>(dY, S, ds_part, db_part, M, N, R, pl, dim3(nseg * pl.max_chunks, pl.nsplit), seg, st);
   }
   if (rc != LF_OK) return rc;
   const int64_t n = rows * R;
@@ -822,7 +1309,7 @@ static int dys_dyb_impl(const void* dY, const void* S, void* dS, void* ws, int M
   const int64_t nout = (int64_t)N * maxrank;
   const int nb_rows = (int)((n + 1023) / 1024), nb_seg = (int)((nout + 1023) / 1024);  // four outputs per thread
   return lf_launch((reduce_ds_db_kernel<T>), dim3((unsigned)(nb_rows + nb_seg * nseg)), dim3(256), 0, st, (const float*)ds_part,
-                     (T*)dS, pl.nsplit, M, R, nb_rows, (const float*)db_part, N, nb_seg, pl.group, pl.max_chunks, seg);
+                     (T*)dS, nparts, M, R, nb_rows, (const float*)db_part, N, nb_seg, group, max_chunks, seg);
 }
 
 int lf_launch_dys_dyb(const void* dY, const void* S, void* dS, void* ws, size_t ws_bytes, int M, int N, int R,
@@ -863,10 +1350,45 @@ static void da_shape(int M, int K, int R, const LfSegTable& seg, int& group, int
   if (max_chunks < 1) max_chunks = 1;
 }
 
+// Ring kernel shapes by rank tiles: tiles per slice (registers: TPW * RT * 4 accumulators) and ring depth (LDS: NS
+// stages of 16 KB, 24 KB with a keep-mask, plus two dS blocks of RT * 4 KB; two workgroups per CU where that fits).
+constexpr int da_tpw(int rt) { return rt >= 4 ? 8 : 16; }
+constexpr int da_ns(int rt, bool masked) { return masked ? (rt == 1 ? 3 : 5) : (rt == 4 ? 3 : 4); }
+static int da_ring_smem(int rt, bool masked) { return da_ns(rt, masked) * (TILE_BYTES + (masked ? ROWS * 64 : 0)) + 2 * ROWS * rt * 32; }
+struct DaPlan { int n_slices, group, max_chunks; };
+// Slices of the K axis (balanced, 2 .. TPW tiles each) x chunks of `group` row blocks per segment, by bytes moved: the
+// X stream in whole rounds of resident workgroups, the dS blocks every workgroup fetches, and the fp32 partials
+// (one [R, K] slab per chunk, written here and read by the reduce).
+static DaPlan da_plan(int M, int K, int R, bool masked, const LfSegTable& seg) {
+  const int rt = rt_of(R), T = K / 64;
+  int blocks[LF_MAX_SEG], nseg;
+  seg_block_counts(M, seg, blocks, nseg);
+  const int slots = lds_slots(da_ring_smem(rt, masked));
+  const double tile_bytes = TILE_BYTES + (masked ? ROWS * 64 : 0);
+  DaPlan best{1, 1, 1};
+  double best_cost = 1e300;
+  for (int nsl = 1; nsl <= T / 2; nsl++) {
+    if ((T + nsl - 1) / nsl > da_tpw(rt)) continue;
+    for (int g : kGroups) {
+      const RingSplit sp = ring_split(blocks, nseg, g, T, nsl, slots);
+      const double cost = sp.span * slots * tile_bytes + 0.5 * (double)sp.wgs * g * ROWS * R * 2 + 2.0 * 4.0 * R * K * (double)sp.chunks;
+      if (cost < best_cost) { best_cost = cost; best = DaPlan{nsl, g, sp.max_chunks}; }
+    }
+  }
+  return best;
+}
+
 size_t lf_da_workspace(int M, int K, int R, const LfSegTable& seg) {
-  int group, max_chunks;
-  da_shape(M, K, R, seg, group, max_chunks);
   const int nseg = seg.table ? seg.n_seg : 1;
+  int max_chunks;
+  if (rt_of(R) <= 4) {
+    // the launch plans with or without a keep-mask: room for either
+    const int a = da_plan(M, K, R, true, seg).max_chunks, b = da_plan(M, K, R, false, seg).max_chunks;
+    max_chunks = a > b ? a : b;
+  } else {
+    int group;
+    da_shape(M, K, R, seg, group, max_chunks);
+  }
   return (size_t)nseg * max_chunks * R * K * sizeof(float);
 }
 
@@ -881,19 +1403,42 @@ static int da_launch(const void* X, const uint8_t* mask, const void* dS, float* 
   return lf_launch(kern, grid, dim3(256), smem, st, (const T*)X, mask, (const T*)dS, part, M, K, R, group, max_chunks, seg);
 }
 
+template <typename T, int RT, bool MASK>
+static int da_ring_launch(const void* X, const uint8_t* mask, const void* dS, float* part, int M, int K, int R, const DaPlan& pl,
+                          int nseg, const LfSegTable& seg, hipStream_t st) {
+  auto kern = lora_da_ring_kernel<T, RT, da_tpw(RT), da_ns(RT, MASK), MASK>;
+  const int smem = da_ring_smem(RT, MASK);
+  static LfLdsFlags lds_ok;
+  if (!lf_allow_lds(kern, smem, lds_ok)) return LF_ELAUNCH;
+  return lf_launch(kern, dim3(pl.n_slices, pl.max_chunks, nseg), dim3(256), smem, st, (const T*)X, mask, (const T*)dS, part, M, K, R,
+                   pl.n_slices, pl.group, pl.max_chunks, seg);
+}
+
 template <typename T>
 static int da_impl(const void* X, const uint8_t* mask, const void* dS, void* ws, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
-  int group, max_chunks;
-  da_shape(M, K, R, seg, group, max_chunks);
   const int nseg = seg.table ? seg.n_seg : 1;
   float* part = (float*)ws;
-  dim3 grid(K / 64, max_chunks, nseg);
-  int rc;
-  switch (rt_of(R)) {
-    case 1: rc = da_launch<T, 1>(X, mask, dS, part, M, K, R, group, max_chunks, grid, seg, st); break;
-    case 2: rc = da_launch<T, 2>(X, mask, dS, part, M, K, R, group, max_chunks, grid, seg, st); break;
-    case 4: rc = da_launch<T, 4>(X, mask, dS, part, M, K, R, group, max_chunks, grid, seg, st); break;
-    default: rc = da_launch<T, 8>(X, mask, dS, part, M, K, R, group, max_chunks, grid, seg, st); break;
+  int group, max_chunks, rc;
+  if (rt_of(R) <= 4) {
+    const DaPlan pl = da_plan(M, K, R, mask != nullptr, seg);
+    group = pl.group;
+    max_chunks = pl.max_chunks;
+    if (mask != nullptr) {
+      switch (rt_of(R)) {
+        case 1: rc = da_ring_launch<T, 1, true>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
+        case 2: rc = da_ring_launch<T, 2, true>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
+        default: rc = da_ring_launch<T, 4, true>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
+      }
+    } else {
+      switch (rt_of(R)) {
+        case 1: rc = da_ring_launch<T, 1, false>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
+        case 2: rc = da_ring_launch<T, 2, false>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
+        default: rc = da_ring_launch<T, 4, false>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
+      }
+    }
+  } else {
+    da_shape(M, K, R, seg, group, max_chunks);
+    rc = da_launch<T, 8>(X, mask, dS, part, M, K, R, group, max_chunks, dim3(K / 64, max_chunks, nseg), seg, st);
   }
   if (rc != LF_OK) return rc;
   int maxrank = 0;
@@ -915,3 +1460,4 @@ int lf_launch_da(const void* X, const uint8_t* mask, const void* dS, void* ws, s
   if (dtype == LF_F16) return da_impl<_Float16>(X, mask, dS, ws, M, K, R, seg, st);
   return LF_EINVAL;
 }
+
