@@ -51,7 +51,7 @@ constexpr int PAIR_NN = 1024 + 32;
 template <bool NN> struct Lds {
   static constexpr int STAGE_B = NN ? 32 * PAIR_NN : BN * BK * 2;
   static constexpr int STAGE = STAGE_A + STAGE_B;
-  static constexpr int EP_OFF = 2 * STAGE, EP_WAVE = 4096, BYTES = EP_OFF + 4 * EP_WAVE;
+  static constexpr int EP_OFF = 2 * STAGE, EP_WAVE = 4608, BYTES = EP_OFF + 4 * EP_WAVE;
   static_assert(BYTES <= 160 * 1024, "two stages and the epilogue bands fit the LDS of a CU");
 };
 
@@ -66,6 +66,14 @@ template <> struct BigOp<__bf16> {
   static __device__ __forceinline__ void mfma(lf_f32x4& c, lf_u32x4 a, lf_u32x4 b) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
+  // d = a b into ordinary vector registers (for a product that vector instructions pick up next)
+  static __device__ __forceinline__ void mfma0(lf_f32x4& d, lf_u32x4 a, lf_u32x4 b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+  }
+  // c = a b: the first product of a tile needs no zeroed accumulator
+  static __device__ __forceinline__ void mfma_first(lf_f32x4& c, lf_u32x4 a, lf_u32x4 b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
     bf2 v = {(__bf16)lo, (__bf16)hi};
@@ -76,6 +84,12 @@ template <> struct BigOp<__bf16> {
 template <> struct BigOp<_Float16> {
   static __device__ __forceinline__ void mfma(lf_f32x4& c, lf_u32x4 a, lf_u32x4 b) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma0(lf_f32x4& d, lf_u32x4 a, lf_u32x4 b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma_first(lf_f32x4& c, lf_u32x4 a, lf_u32x4 b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -331,13 +345,16 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     };
 
     // ------------------------------------------------------------ LoRA seed: acc = mult * L Rop (masked), or zero
+    auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 8; i++)
+      for (int i = 0; i < 8; i++)
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
-        acc[i][j] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
-        asm volatile("" : "+a"(acc[i][j]));  // zeroed in the accumulation registers themselves
-      }
+        for (int j = 0; j < 8; j++) {
+          acc[i][j] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
+          asm volatile("" : "+a"(acc[i][j]));  // zeroed in the accumulation registers themselves
+        }
+    };
+    if (!(LORA && p.L != nullptr)) zero_acc();
     if (LORA && p.L != nullptr) {
       int sl = lane;
       asm volatile("" : "+v"(sl));   // as in the epilogue: keep the seed's address arithmetic inside the tile loop
@@ -353,10 +370,110 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       // The K loop's fragment registers are still dead here, which is where the room comes from.
       const bool sel = p.mult_mode == 1 && use_mask;
       const int n_chunks = (p.R + 31) / 32;
+      if (sel && n_chunks == 1) {
+        // ---- masked seed at ranks up to 32, one block row (16 rows) at a time: the product of a block row goes to
+        // ordinary vector registers (d = a b + 0), the keep-mask picks value or zero there, and the result is written
+        // into the accumulation registers -- three vector instructions per element (compare, select, write) where
+        // zeroing, multiplying into the accumulator and selecting in place take six (write; read, multiply, compare,
+        // select, write).  1/(1-p) goes into the 16-bit dS fragment, as the forward scale does (one rounding).
+        const int r0 = kg * 8;
+        const bool in_r = r0 < rank, in_R = r0 < p.R;
+        lf_u32x4 rf[8], lv[8], mq[16];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const int gn = n0 + wn * 128 + j * 16 + l16;
+          const int rc = in_r ? r0 : 0;
+          if constexpr (!NN) {
+            rf[j] = *(const lf_u32x4*)(rp + (int64_t)gn * rank + rc);
+          } else {
+            const uint32_t voff = (uint32_t)((rc * p.N + gn) * 2);
+            uint32_t e[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) e[k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcR, voff, k * p.N * 2, 0);
+            rf[j] = lf_u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) lv[i] = *(const lf_u32x4*)(Lp + (int64_t)(wrow0 + i * 16 + l16) * p.R + (in_R ? r0 : 0));
+        {
+          // keep-mask of the wave's 128x128 block, whole rows per instruction (lane -> row lane>>3, 16-byte chunk lane&7)
+          const uint8_t* mrow = p.mask + (int64_t)(wrow0 + (sl >> 3)) * p.ldmask + n0 + wn * 128 + (sl & 7) * 16;
+#pragma unroll
+          for (int q = 0; q < 16; q++) mq[q] = *(const lf_u32x4*)(mrow + (int64_t)q * 8 * p.ldmask);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+          for (int d = 0; d < 4; d++) rf[j][d] = in_r ? rf[j][d] : 0u;
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+          for (int d = 0; d < 4; d++) {
+            const uint32_t v = in_R ? lv[i][d] : 0u;
+            lv[i][d] = BigOp<T>::pack2(BigOp<T>::to_float((uint16_t)(v & 0xffffu)) * mult, BigOp<T>::to_float((uint16_t)(v >> 16)) * mult);
+          }
+        // vector results feed inline-assembly MFMAs: wait states, with the operands as in/outs (see the other path)
+        asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
+                                 "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]));
+        // Two slabs of the wave's LDS patch turn the mask rows to the accumulator layout (rows 144 bytes apart: a slab's
+        // 64 dword reads hit 64 banks).  Block row i+1 is written and multiplied while block row i is read and selected.
+        constexpr int MPITCH = 144, SLAB = 16 * MPITCH;
+        static_assert(2 * SLAB <= EP_WAVE, "two mask slabs fit a wave's patch");
+        const uint32_t mp_lds = lds0 + EP_OFF + wave * EP_WAVE;
+        const uint32_t mp_wr = mp_lds + (sl >> 3) * MPITCH + (sl & 7) * 16;
+        const uint32_t mp_rd = mp_lds + l16 * MPITCH + kg * 4;
+        lf_f32x4 tmp[2][8];
+        auto stage_row = [&](auto I) __attribute__((always_inline)) {
+          constexpr int i = I.value;
+          asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(mp_wr), "v"(mq[2 * i]), "n"((i & 1) * SLAB) : "memory");
+          asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(mp_wr), "v"(mq[2 * i + 1]), "n"((i & 1) * SLAB + 8 * MPITCH) : "memory");
+#pragma unroll
+          for (int j = 0; j < 8; j++) BigOp<T>::mfma0(tmp[i & 1][j], rf[j], lv[i]);
+        };
+        stage_row(integral_constant<int, 0>{});
+        sfor<8>([&](auto I) {
+          constexpr int i = I.value, so = (i & 1) * SLAB;
+          lgkm0();   // the slab of block row i is written
+          uint32_t k0, k1, k2, k3, k4, k5, k6, k7;
+          // (written out: inline-assembly operands inside a generic lambda's nested lambda do not compile with this clang)
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k0) : "v"(mp_rd), "n"(so) : "memory");
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k1) : "v"(mp_rd), "n"(so + 16) : "memory");
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k2) : "v"(mp_rd), "n"(so + 32) : "memory");
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k3) : "v"(mp_rd), "n"(so + 48) : "memory");
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k4) : "v"(mp_rd), "n"(so + 64) : "memory");
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k5) : "v"(mp_rd), "n"(so + 80) : "memory");
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k6) : "v"(mp_rd), "n"(so + 96) : "memory");
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k7) : "v"(mp_rd), "n"(so + 112) : "memory");
+          if constexpr (i + 1 < 8) stage_row(integral_constant<int, i + 1>{});
+          // The wait for the mask dwords (the two writes behind them may still be on their way) and the wait states
+          // between the MFMAs of this block row -- issued a block row ago; the nops cover the first -- and the vector
+          // instructions that read their results, in one statement that takes all of them as in/outs.
+          lf_f32x4(&tm)[8] = tmp[i & 1];
+          if constexpr (i + 1 < 8)
+            asm volatile("s_waitcnt lgkmcnt(2)\n\ts_nop 7"
+                         : "+v"(k0), "+v"(k1), "+v"(k2), "+v"(k3), "+v"(k4), "+v"(k5), "+v"(k6), "+v"(k7), "+v"(tm[0]), "+v"(tm[1]),
+                           "+v"(tm[2]), "+v"(tm[3]), "+v"(tm[4]), "+v"(tm[5]), "+v"(tm[6]), "+v"(tm[7])
+                         :: "memory");
+          else
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7"
+                         : "+v"(k0), "+v"(k1), "+v"(k2), "+v"(k3), "+v"(k4), "+v"(k5), "+v"(k6), "+v"(k7), "+v"(tm[0]), "+v"(tm[1]),
+                           "+v"(tm[2]), "+v"(tm[3]), "+v"(tm[4]), "+v"(tm[5]), "+v"(tm[6]), "+v"(tm[7])
+                         :: "memory");
+          const uint32_t mk[8] = {k0, k1, k2, k3, k4, k5, k6, k7};
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            lf_f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = ((mk[j] >> (8 * e)) & 0xffu) ? tm[j][e] : 0.f;
+            acc[i][j] = v;
+            asm volatile("" : "+a"(acc[i][j]));  // into the accumulation registers now
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      } else {
       // one MFMA k-step covers 32 rank columns; lanes whose 8 columns lie beyond R (or the rank) read the first
       // columns again and are zeroed by a select (branch-free)
-      mfma_fence();  // the accumulator was just zeroed by vector instructions
-      auto chunk = [&](int t) __attribute__((always_inline)) {
+      auto chunk = [&](int t, auto FIRST) __attribute__((always_inline)) {
         const int r0 = t * 32 + kg * 8;
         const bool in_r = r0 < rank, in_R = r0 < p.R;
         lf_u32x4 rf[8], lv[8];
@@ -400,11 +517,12 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
         for (int i = 0; i < 8; i++)
 #pragma unroll
-          for (int j = 0; j < 8; j++) BigOp<T>::mfma(acc[i][j], rf[j], lv[i]);
+          for (int j = 0; j < 8; j++) {
+            if constexpr (FIRST.value) BigOp<T>::mfma_first(acc[i][j], rf[j], lv[i]);   // writes the accumulators: no zeroing
+            else BigOp<T>::mfma(acc[i][j], rf[j], lv[i]);
+          }
         __builtin_amdgcn_sched_barrier(0);
       };
-      int t = 0;
-      for (; t + 1 < n_chunks; t++) chunk(t);
       // Keep-mask of the wave's 128x128 block: 16 KB.  A lane owns, in every 16x16 accumulator block, row l16 and four
       // consecutive columns (one dword of mask bytes), so loading "its" dwords directly is 64 instructions that each
       // touch 16 rows -- 16 cache lines for 256 bytes; measured 17 K cycles per tile, most of the seed.  Instead the
@@ -426,7 +544,8 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
 #endif
         }
       }
-      chunk(t);
+      chunk(0, std::true_type{});
+      for (int t = 1; t < n_chunks; t++) chunk(t, std::false_type{});
 #ifdef LF_ABL_NOSELECT
       if (sel && mult == 12345.f) {
 #else
@@ -471,6 +590,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
           }
           __builtin_amdgcn_sched_barrier(0);
         }
+      }
       }
       mfma_fence();
       route = route_of(nxt_tile.m0 + wm * 128);  // in flight during this tile's K loop
