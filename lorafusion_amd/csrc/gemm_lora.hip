@@ -688,23 +688,28 @@ static int choose_cfg(int M, int N, bool allow_big, double* cost_out = nullptr) 
   if (cost_out) *cost_out = best_cost;
   return best;
 }
-// Rows [0, m_main) in whole rounds of 256x256 tiles, the rest as a second launch with the tile
-// that spreads it best, when that beats one launch (a nearly empty last round of big tiles
-// costs a full tile time).  Returns m_main (0: single launch).
+// Rows [0, m_main) as 256x256 tiles, the rest as a second launch with the tile that spreads it best, when that beats
+// one launch (a nearly empty last round of big tiles costs a full tile time).  m_main is the multiple of 256 rows
+// with the lowest modelled cost of both launches: usually the one whose tiles fill whole rounds of the chip
+// (32 tile rows of 40 tiles are exactly five rounds; 30 rows of 40 are five rounds too, and leave a longer tail).
+// Returns m_main (0: single launch).
 static int choose_split(int M, int N, bool allow_big, int* cfg_head, int* cfg_tail) {
   constexpr double kLaunch = 4.0;  // a second launch
   const int grid_n = (N + 255) / 256;
   if (grid_n > 256) return 0;
-  const int rows_per_round = (256 / grid_n) * 256;
-  const int m_main = (M / rows_per_round) * rows_per_round;
-  if (m_main <= 0 || m_main >= M) return 0;
-  double single, tail;
-  choose_cfg(M, N, allow_big, &single);
-  *cfg_tail = choose_cfg(M - m_main, N, allow_big, &tail);
   const bool big = allow_big && N >= 256;
+  const TileCand& head = kCands[big ? 0 : 1];
+  double best;
+  choose_cfg(M, N, allow_big, &best);
+  int best_m = 0;
+  for (int r = 1; r * 256 < M; r++) {
+    double tail;
+    const int ct = choose_cfg(M - r * 256, N, allow_big, &tail);
+    const double cost = launch_cost(head, r * 256, N) + tail + kLaunch;
+    if (cost < best) { best = cost; best_m = r * 256; *cfg_tail = ct; }
+  }
   *cfg_head = big ? 7 : 1;
-  const double split = launch_cost(kCands[big ? 0 : 1], m_main, N) + tail + kLaunch;
-  return split < single ? m_main : 0;
+  return best_m;
 }
 
 static std::atomic<int> pinned_cfg{-1};
