@@ -14,12 +14,14 @@
 // therefore run-to-run deterministic.
 //
 // Streaming: the big operand moves as 128-row x 64-column tiles.  Global loads are coalesced
-// (8 consecutive lanes read one 128-byte row segment), the keep-mask is applied in registers,
-// and the tile is written to LDS with the same XOR swizzle as the GEMM (granule g of row r
-// at slot g ^ ((r>>1)&7)), from where both MFMA access patterns are bank-conflict free:
-// row fragments (ds_read_b128) and transposed fragments (ds_read_b64_tr_b16).  Loading MFMA
-// fragments straight from global memory would put every lane on a different row (one cache
-// line per lane) and runs at a quarter of the coalesced rate.
+// (8 consecutive lanes read one 128-byte row segment) and the tile sits in LDS with the same XOR
+// swizzle as the GEMM (granule g of row r at slot g ^ ((r>>1)&7)), from where both MFMA access
+// patterns are bank-conflict free: row fragments (ds_read_b128) and transposed fragments
+// (ds_read_b64_tr_b16).  Loading MFMA fragments straight from global memory would put every
+// lane on a different row (one cache line per lane) and runs at a quarter of the coalesced rate.
+// Two transports: through registers (load, keep-mask applied on the way, LDS store; xa, and
+// dys_dyb / da above rank 64), or as buffer loads that write LDS themselves, several tiles
+// ahead through a ring of stages (dys_dyb / da up to rank 64; second half of this file).
 //
 // MFMA 16x16x32 operand layout (64 lanes): lane l holds row/col (l & 15) and the 8
 // contraction elements of chunk (l >> 4).  Where the contraction index is the slow memory
@@ -1195,8 +1197,9 @@ static DysRingPlan dysr_plan(int M, int N, int R, const LfSegTable& seg) {
   const double tile_bytes = TILE_BYTES + 64.0 * R * 2;
   DysRingPlan best{1, 1, 1};
   double best_cost = 1e300;
-  for (int nsl = 1; nsl <= T / 2; nsl++) {
-    if ((T + nsl - 1) / nsl > dysr_tpw(rt)) continue;
+  for (int t = dysr_tpw(rt); t >= 2; t--) {   // tiles of the longest slice -> fewest slices that reach it
+    const int nsl = (T + t - 1) / t;
+    if (nsl > T / 2 || (T + nsl - 1) / nsl != t) continue;
     for (int g : kGroups) {
       const RingSplit sp = ring_split(blocks, nseg, g, T, nsl, slots);
       const double cost = sp.span * slots * tile_bytes + 0.5 * (double)sp.wgs * g * ROWS * R * 2 +
@@ -1367,8 +1370,9 @@ static DaPlan da_plan(int M, int K, int R, bool masked, const LfSegTable& seg) {
   const double tile_bytes = TILE_BYTES + (masked ? ROWS * 64 : 0);
   DaPlan best{1, 1, 1};
   double best_cost = 1e300;
-  for (int nsl = 1; nsl <= T / 2; nsl++) {
-    if ((T + nsl - 1) / nsl > da_tpw(rt)) continue;
+  for (int t = da_tpw(rt); t >= 2; t--) {   // tiles of the longest slice -> fewest slices that reach it
+    const int nsl = (T + t - 1) / t;
+    if (nsl > T / 2 || (T + nsl - 1) / nsl != t) continue;
     for (int g : kGroups) {
       const RingSplit sp = ring_split(blocks, nseg, g, T, nsl, slots);
       const double cost = sp.span * slots * tile_bytes + 0.5 * (double)sp.wgs * g * ROWS * R * 2 + 2.0 * 4.0 * R * K * (double)sp.chunks;
