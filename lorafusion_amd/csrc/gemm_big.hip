@@ -373,9 +373,9 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       if (sel && n_chunks == 1) {
         // ---- masked seed at ranks up to 32, one block row (16 rows) at a time: the product of a block row goes to
         // ordinary vector registers (d = a b + 0), the keep-mask picks value or zero there, and the result is written
-        // into the accumulation registers -- three vector instructions per element (compare, select, write) where
-        // zeroing, multiplying into the accumulator and selecting in place take six (write; read, multiply, compare,
-        // select, write).  1/(1-p) goes into the 16-bit dS fragment, as the forward scale does (one rounding).
+        // into the accumulation registers -- four vector instructions per element (multiply by 1/(1-p) in fp32,
+        // compare, select, write) where zeroing, accumulating and selecting in place take six (write; read,
+        // multiply, compare, select, write).
         const int r0 = kg * 8;
         const bool in_r = r0 < rank, in_R = r0 < p.R;
         lf_u32x4 rf[8], lv[8], mq[16];
@@ -408,10 +408,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
         for (int i = 0; i < 8; i++)
 #pragma unroll
-          for (int d = 0; d < 4; d++) {
-            const uint32_t v = in_R ? lv[i][d] : 0u;
-            lv[i][d] = BigOp<T>::pack2(BigOp<T>::to_float((uint16_t)(v & 0xffffu)) * mult, BigOp<T>::to_float((uint16_t)(v >> 16)) * mult);
-          }
+          for (int d = 0; d < 4; d++) lv[i][d] = in_R ? lv[i][d] : 0u;
         // vector results feed inline-assembly MFMAs: wait states, with the operands as in/outs (see the other path)
         asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
                                  "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]));
@@ -464,7 +461,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
           for (int j = 0; j < 8; j++) {
             lf_f32x4 v;
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = ((mk[j] >> (8 * e)) & 0xffu) ? tm[j][e] : 0.f;
+            for (int e = 0; e < 4; e++) v[e] = ((mk[j] >> (8 * e)) & 0xffu) ? tm[j][e] * mult : 0.f;   // 1/(1-p) in fp32
             acc[i][j] = v;
             asm volatile("" : "+a"(acc[i][j]));  // into the accumulation registers now
           }
