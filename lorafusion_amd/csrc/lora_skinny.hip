@@ -100,6 +100,17 @@ __device__ __forceinline__ lf_u32x4 tr_read8(const char* p, int pitch) {
 
 constexpr int TILE_BYTES = ROWS * 128;  // 128 rows x 64 columns of 16-bit
 
+// Swizzle key of a tile row: granule g of row r sits at slot g ^ tile_key(r).  LDS serves a 16-byte read 16 lanes at
+// a time and an 8-byte (transposed) read 32 lanes at a time, in both cases 256 bytes = all 64 banks.  Row fragments:
+// 16 consecutive rows, one granule each -- the 8 rows of one parity need 8 different keys.  Transposed fragments:
+// rows j, 8+j (j = 0..3), two neighbouring granules each -- the 4 rows of one parity (r>>1 = 0, 1, 4, 5 mod 8) need 4
+// different key>>1.  The three bits of r>>1 rotated by one do both (with the bits in place, 0/1 and 4/5 share key>>1:
+// every transposed read took two passes).
+__device__ __forceinline__ int tile_key(int row) {
+  const int x = (row >> 1) & 7;
+  return ((x & 1) << 2) | (x >> 1);
+}
+
 // One thread's share of a 128x64 tile: 4 granules of 8 elements (+ their 8 mask bytes each).
 struct TileRegs {
   lf_u32x4 x[4];
@@ -110,7 +121,7 @@ struct TileRegs {
 template <typename T>
 __device__ __forceinline__ void tile_load(TileRegs& r, const T* __restrict__ src, const uint8_t* __restrict__ mask,
                                           int64_t ld, int row0, int max_row, int col0, int tid, bool use_mask) {
-  const int srcg = (tid & 7) ^ ((tid >> 4) & 7);
+  const int srcg = (tid & 7) ^ tile_key(tid >> 3);   // rows i*32 + (tid>>3) share their key
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int row = min(row0 + i * 32 + (tid >> 3), max_row - 1);
@@ -128,15 +139,15 @@ __device__ __forceinline__ void tile_store(const TileRegs& r, char* tile, int ti
 
 // Row fragment: 8 consecutive columns (granule g) of `row`.
 __device__ __forceinline__ lf_u32x4 tile_row_frag(const char* tile, int row, int g) {
-  return *(const lf_u32x4*)(tile + row * 128 + ((g ^ ((row >> 1) & 7)) << 4));
+  return *(const lf_u32x4*)(tile + row * 128 + ((g ^ tile_key(row)) << 4));
 }
 
 // Transposed fragment: rows row..row+3 and row+4..row+7 of the lane's column; `col` is the first
 // of the 4 columns this lane addresses (multiple of 4).
 __device__ __forceinline__ lf_u32x4 tile_tr_frag(const char* tile, int row, int col) {
   const int g = col >> 3, within = (col & 7) * 2;
-  const char* p0 = tile + row * 128 + ((g ^ ((row >> 1) & 7)) << 4) + within;
-  const char* p1 = tile + (row + 4) * 128 + ((g ^ (((row + 4) >> 1) & 7)) << 4) + within;
+  const char* p0 = tile + row * 128 + ((g ^ tile_key(row)) << 4) + within;
+  const char* p1 = tile + (row + 4) * 128 + ((g ^ tile_key(row + 4)) << 4) + within;
   lf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(p0));
   lf_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(p1));
   lf_u32x2 a = __builtin_bit_cast(lf_u32x2, lo), b = __builtin_bit_cast(lf_u32x2, hi);
@@ -724,9 +735,9 @@ __device__ __forceinline__ void wait_groups(int groups) {
 __device__ __forceinline__ void ring_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Per-thread window offsets of a 128-row x 64-column tile of a 16-bit matrix with `ld` elements per row, in the LDS
-// layout the fragment readers expect (position p = i*256 + tid: row p>>3, slot p&7 holds granule slot ^ ((row>>1)&7)).
+// layout the fragment readers expect (position p = i*256 + tid: row p>>3, slot p&7 holds granule slot ^ tile_key(row)).
 __device__ __forceinline__ void tile_voffs(uint32_t (&v)[4], int64_t ld, int tid) {
-  const int srcg = (tid & 7) ^ ((tid >> 4) & 7);
+  const int srcg = (tid & 7) ^ tile_key(tid >> 3);
 #pragma unroll
   for (int i = 0; i < 4; i++) v[i] = (uint32_t)((int64_t)(i * 32 + (tid >> 3)) * ld * 2 + srcg * 16);
 }
@@ -749,7 +760,7 @@ __device__ __forceinline__ void tile_apply_mask(char* tile, const char* mtile, i
   lf_u32x2 m[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {   // all reads first: behind a store the compiler would not start the next read
-    const int p = i * 256 + tid, row = p >> 3, g = (p & 7) ^ ((row >> 1) & 7);
+    const int p = i * 256 + tid, row = p >> 3, g = (p & 7) ^ tile_key(row);
     x[i] = *(const lf_u32x4*)(tile + p * 16);
     m[i] = *(const lf_u32x2*)(mtile + row * 64 + g * 8);
   }
@@ -757,11 +768,17 @@ __device__ __forceinline__ void tile_apply_mask(char* tile, const char* mtile, i
   for (int i = 0; i < 4; i++) *(lf_u32x4*)(tile + (i * 256 + tid) * 16) = apply_mask8(x[i], m[i]);
 }
 
-// A [rows x RT*16] side operand (S or dS block: 128 rows; B tile: 64 rows) in LDS: rows of RT*32 bytes, granule g of
-// row r at slot g ^ key(r).  A transpose read is served 16 lanes at a time: four consecutive rows, 32 bytes of each,
-// which the key puts on four different quarters of the 32 banks (at 32-byte rows they are there already).
+// A [rows x RT*16] side operand (S or dS block: 128 rows; B tile: 64 rows) in LDS: rows of RT*32 bytes; granule g of
+// source row r at slot g ^ side_key(r) of LDS row side_row(r).  A transposed read is served 32 lanes at a time: rows
+// j, 8+j (j = 0..3), 32 bytes of each, which must land on eight different 32-byte groups of the 64 banks.  At 128-byte
+// rows the key separates (r>>3)&1 and (r>>1)&1 (the row's parity picks the half of the banks); at 64-byte rows
+// (r>>3)&1; at 32-byte rows no key can (a row is one group): rows 8..15 of every 16 swap their halves instead.
 template <int RT>
-__device__ __forceinline__ int side_key(int row) { return RT >= 4 ? (row & 3) << 1 : RT == 2 ? ((row >> 1) & 1) << 1 : 0; }
+__device__ __forceinline__ int side_key(int row) {
+  return RT >= 4 ? ((((row >> 3) & 1) << 1) | (((row >> 1) & 1) << 2)) : RT == 2 ? ((row >> 3) & 1) << 1 : 0;
+}
+template <int RT>
+__device__ __forceinline__ int side_row(int row) { return RT == 1 ? row ^ (((row >> 3) & 1) << 2) : row; }
 // window offsets of the granules this thread fetches: position p = i*256 + tid -> row p / (2 RT), slot p % (2 RT); a
 // granule beyond `cols` columns does not exist in memory: the first one is fetched instead (its products land in
 // rank columns that the reduce discards)
@@ -769,7 +786,7 @@ template <int RT, int NI>
 __device__ __forceinline__ void side_voffs(uint32_t (&v)[NI], int pitch_elems, int cols, int tid) {
 #pragma unroll
   for (int i = 0; i < NI; i++) {
-    const int p = i * 256 + tid, row = p / (RT * 2), g = (p % (RT * 2)) ^ side_key<RT>(row);
+    const int p = i * 256 + tid, row = side_row<RT>(p / (RT * 2)), g = (p % (RT * 2)) ^ side_key<RT>(row);   // side_row is its own inverse
     v[i] = (uint32_t)(row * pitch_elems * 2 + (g * 8 < cols ? g : 0) * 16);
   }
 }
@@ -778,12 +795,16 @@ __device__ __forceinline__ void side_dma(const lf_u32x4& rsrc, const uint32_t (&
 #pragma unroll
   for (int i = 0; i < NI; i++) dma16(rsrc, v[i], lds_side + i * 4096 + wave * 1024);
 }
-// transposed fragment: rows row..row+3 and row+4..row+7 of the lane's column among columns c*16 + 4*c4 .. (row and
-// row + 4 share their key)
+// transposed fragment: rows row..row+3 and row+4..row+7 (row % 8 < 4) of the lane's column among columns c*16 + 4*c4 ..
 template <int RT>
 __device__ __forceinline__ lf_u32x4 side_tr8(const char* blk, int row, int c, int c4) {
-  const int g = c * 2 + (c4 >> 1);
-  return tr_read8(blk + row * (RT * 32) + ((g ^ side_key<RT>(row)) << 4) + (c4 & 1) * 8, RT * 32);
+  const int g = c * 2 + (c4 >> 1), within = (c4 & 1) * 8;
+  const char* p0 = blk + side_row<RT>(row) * (RT * 32) + ((g ^ side_key<RT>(row)) << 4) + within;
+  const char* p1 = blk + side_row<RT>(row + 4) * (RT * 32) + ((g ^ side_key<RT>(row + 4)) << 4) + within;
+  lf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(p0));
+  lf_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(p1));
+  lf_u32x2 a = __builtin_bit_cast(lf_u32x2, lo), b = __builtin_bit_cast(lf_u32x2, hi);
+  return lf_u32x4{a[0], a[1], b[0], b[1]};
 }
 
 // ---- da.  grid (n_slices, max_chunks, n_seg).  Workgroup (ks, ch, s): the k-tiles of slice ks (at most TPW, at least
