@@ -170,10 +170,13 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
       for (int i = 0; i < NLB; i++) {
         // 32-byte unit u of LDS row r holds source unit u ^ key(r), key(r) = (r&3)*2 + ((r>>3)&1): the
         // 8 rows that 32 lanes of a transposed read touch (r, r+8 for four consecutive r) then cover
-        // all 64 banks
+        // all 64 banks.  Rows of 128 bytes (64-column tiles) hold four units and their parity already
+        // picks the half of the banks: there key(r) = ((r>>1)&1)*2 + ((r>>3)&1) separates the four
+        // rows of one parity (the general key, cut to two bits, left two of them on the same unit)
         int gid = i * NTHREADS + tid;
         int row = gid / GPR, g = gid % GPR;
-        int srcunit = (g >> 1) ^ ((((row & 3) << 1) | ((row >> 3) & 1)) & BKEY);
+        int srcunit = (g >> 1) ^ (BPITCH == 128 ? ((((row >> 1) & 1) << 1) | ((row >> 3) & 1))
+                                                : ((((row & 3) << 1) | ((row >> 3) & 1)) & BKEY));
         int col = min(n0 + (srcunit * 2 + (g & 1)) * 8, p.N - 8);
         bvoff[i] = (uint32_t)((int64_t)row * p.ldb * 2 + col * 2);
       }
@@ -374,7 +377,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     // receives column (lane&15), rows 0..3.  Group kg takes contraction rows kg*8.. (two reads).
     const int j4 = l16 >> 2, c = l16 & 3;
     const int row0 = kg * 8 + j4;
-    const int key = ((j4 << 1) | (kg & 1)) & BKEY;
+    const int key = BPITCH == 128 ? (((j4 >> 1) << 1) | (kg & 1)) : (((j4 << 1) | (kg & 1)) & BKEY);
 #pragma unroll
     for (int j = 0; j < TN; j++) {
       int colb = (wn * WN + j * 16 + 4 * c) * 2;  // byte offset within the row
