@@ -190,3 +190,45 @@ def test_reference_module_and_function_names_resolve():
         for s in syms:
             assert hasattr(m, s), f"lorafusion_amd.ops.{mod}.{s} is missing"
     assert importlib.import_module("lorafusion_amd.patch.patch_lora").apply_lora
+
+
+def test_workspace_sizes_of_the_rank_r_passes_stay_bounded():
+    """The scratch of the backward passes holds fp32 partial sums: one [rows, R] slab per slice of the streamed
+    matrix's columns and one [N, R] (or [R, K]) slab per chunk of an adapter's row blocks.  The split that sizes it is
+    host logic (no GPU): for every shape it must give a multiple of 256 bytes that is at least one slab of each kind
+    and stays below a few times the streamed operand (a split that cut every block into its own chunk did not)."""
+    import torch
+
+    from lorafusion_amd import _lib
+
+    lib = _lib.lib()
+
+    def routing(padded, ranks):
+        nb = sum(padded) // 128
+        table = torch.zeros((nb, 3), dtype=torch.int32)      # host pointers are only stored, never read on the CPU
+        scale = torch.ones(nb)
+        p = torch.zeros(nb)
+        return _lib.multi_routing(padded, ranks, table, scale, p, 128), (table, scale, p)
+
+    cases = []
+    for R in (16, 32, 48, 64, 128):
+        for (M, N, K) in ((1, 128, 128), (300, 256, 128), (2048, 4096, 4096), (8448, 4096, 4096), (16512, 28672, 4096),
+                          (8576, 57344, 8192), (8576, 8192, 28672)):
+            cases.append((_lib.single_routing(R, 2.0, 0.1), None, M, N, K, R, 1))
+    for padded, ranks in (([1152, 640, 1152, 768, 512, 896, 1920, 1536], [64] * 8), ([2688, 4480, 4608, 4736], [16] * 4),
+                          ([128] * 32, [16, 32] * 16), ([128, 8192, 128], [8, 64, 16])):
+        r, keep = routing(padded, ranks)
+        M, R = sum(padded), _lib.round_rank(max(ranks))
+        for (N, K) in ((4096, 4096), (57344, 8192), (128, 128)):
+            cases.append((r, keep, M, N, K, R, len(padded)))
+    for r, keep, M, N, K, R, nseg in cases:
+        rows = (M + 127) // 128 * 128
+        dys = lib.lf_workspace_bytes(_lib.LF_OP_DYS_DYB, M, N, K, R, ctypes.byref(r))
+        da = lib.lf_workspace_bytes(_lib.LF_OP_DA, M, N, K, R, ctypes.byref(r))
+        bwd = lib.lf_workspace_bytes(_lib.LF_OP_BWD, M, N, K, R, ctypes.byref(r))
+        assert dys % 256 == 0 and da % 256 == 0 and bwd == max(dys, da), (M, N, K, R)
+        assert dys >= (M * R + nseg * N * R) * 4 and da >= nseg * R * K * 4, (M, N, K, R, dys, da)
+        # partial sums written and read once stay within a few times the operand they are the sums of (tiny problems:
+        # a few slabs of each kind are the floor)
+        assert dys <= max(4 * rows * N * 2, 4 * (rows * R + nseg * N * R) * 4 + 4096), (M, N, K, R, dys)
+        assert da <= max(4 * rows * K * 3, 4 * nseg * R * K * 4 + 4096), (M, N, K, R, da)
