@@ -712,7 +712,9 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         }
         lgkm0();
 #pragma unroll
-        for (int rr = 0; rr < 4; rr++) *(lf_u32x4*)(crow + (int64_t)(i * 16 + rr * 4) * p.ldc) = v[rr];
+        // non-temporal: the output is not read again by this kernel; stored this way it leaves the L2 to the operand
+        // panels and its stores are acknowledged sooner (the next tile's first wait for memory is a wait for them)
+        for (int rr = 0; rr < 4; rr++) __builtin_nontemporal_store(v[rr], (lf_u32x4*)(crow + (int64_t)(i * 16 + rr * 4) * p.ldc));
         __builtin_amdgcn_sched_barrier(0);  // one band at a time: the scheduler otherwise reads all 256 accumulators up front
       }
     }
