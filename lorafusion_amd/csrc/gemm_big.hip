@@ -146,7 +146,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   auto tile_of = [&](int it) __attribute__((always_inline)) {
     int pid = it * G + wg;
     if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
-    constexpr int GROUP_M = 8;
+    const int GROUP_M = p.group_m;   // tile rows per group: 8, or 2 for a long K over few tile columns (see the launcher)
     const int width = GROUP_M * p.grid_n;
     const int group = pid / width;
     const int first_m = group * GROUP_M;
@@ -744,6 +744,12 @@ int launch_big(LfGemmParams p, const LfSegTable& seg, int max_wgs, hipStream_t s
   static LfLdsFlags lds_ok;
   constexpr int SMEM_BYTES = Lds<NN>::BYTES;
   if (!lf_allow_lds(kern, SMEM_BYTES, lds_ok)) return LF_ELAUNCH;
+  // Tile order: an XCD's 32 concurrent tiles form a block of group_m tile rows x 32 / group_m columns.  8 x 4 fetches
+  // the fewest operand panels (8 + 4).  With a long K and at most 16 tile columns the left operand does not fit the
+  // 256 MB memory-side cache and every pass over it is an HBM pass: 2 rows x 16 columns read it once per round
+  // (and as 16 neighbouring 128-byte pieces per row at a time) and leave the re-reads to the right operand, which the
+  // cache holds (16384x4096x14336: 1614 -> 1554 us; 16384x4096x28672: 3010 -> 2964 us; at K = 6144 it loses 8 %).
+  p.group_m = (p.K >= 8192 && p.grid_n <= 16) ? 2 : 8;
   const long total = (long)p.grid_m * p.grid_n;
   const int grid = (int)(total < max_wgs ? total : max_wgs);
   return lf_launch(kern, dim3(grid), dim3(256), SMEM_BYTES, st, p, seg);

@@ -50,6 +50,7 @@ struct LfGemmParams {
   int mult_mode;      // 0: LoRA term * scale ; 1: LoRA term * 1/(1-p), masked where p > 0
   int grid_m, grid_n;
   int row0;           // global row of local row 0 (routing lookup when a launch covers a row range)
+  int group_m;        // persistent kernel: tile rows per group of its tile order (set by its launcher)
 };
 
 // launchers (one per translation unit)
