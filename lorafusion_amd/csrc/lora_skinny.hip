@@ -155,7 +155,7 @@ __device__ __forceinline__ lf_u32x4 tile_tr_frag(const char* tile, int row, int 
 }
 
 // ------------------------------------------------------------------------------------ xa
-// One workgroup of 8 waves (fewer for ranks above 32) per 16 rows (32 from rank 48 on); no partial sums leave the workgroup.  The K range is dealt
+// One workgroup of 8 waves (2 above rank 64) per 16 rows (64 at ranks 48-64, 32 above); no partial sums leave the workgroup.  The K range is dealt
 // to the waves in 64-column steps (step s goes to wave s % waves), each wave streams its steps of the
 // 16 rows with coalesced 16-byte loads (8 lanes cover one 128-byte line), all loads of a batch
 // of steps in flight at once, applies the keep-mask in registers and turns the row-major
@@ -164,12 +164,15 @@ __device__ __forceinline__ lf_u32x4 tile_tr_frag(const char* tile, int row, int 
 // loads would put the four lanes of every quad on four different rows, a quarter of the
 // coalesced rate in the texture addresser.  The eight partial [16, R] accumulators are added in a fixed order through LDS,
 // scaled by 1/(1-p), zeroed in padded rows and beyond the adapter's rank, and stored as S.
-// Rows per workgroup: 16, or 32 from rank 48 on -- every workgroup reads the whole adapter matrix (from L2),
-// which at rank 64 is four times the bytes of its 16 rows of X; two row blocks share one set of A fragments.
-constexpr int xa_nb(int rt) { return rt >= 4 ? 2 : 1; }
+// Rows per workgroup: every workgroup reads the whole adapter matrix (from L2), which at rank 64 is four times the
+// bytes of 16 rows of X: with 32 rows per workgroup the pass ran at the L2's rate, not HBM's (268 workgroups x 1 MB of
+// A next to 140 MB of X at 8576 x 8192).  Ranks 48-64 take 64 rows (four row blocks share one set of A fragments)
+// and eight waves: 0.50 -> 0.40 ms over the four linears of the rank-64 layer.  At rank 16 two row blocks per
+// workgroup measured slower (0.27 -> 0.34 ms at the 8B layer: the registers of the second block cost loads in flight).
+constexpr int xa_nb(int rt) { return rt == 4 ? 4 : rt > 4 ? 2 : 1; }
 constexpr int xa_rows(int rt) { return 16 * xa_nb(rt); }
 // waves per workgroup and steps in flight per wave, by rank tiles (LDS: 2 KB * (1+RT) per wave; registers: 8 * RT per step)
-constexpr int xa_waves(int rt) { return rt <= 2 ? 8 : rt <= 4 ? 4 : 2; }
+constexpr int xa_waves(int rt) { return rt <= 4 ? 8 : 2; }
 constexpr int xa_unroll(int rt) { return rt <= 1 ? 4 : rt <= 2 ? 2 : 1; }
 
 // GEN: the keep-mask is not read but drawn here (Philox, the definition of the standalone mask
