@@ -92,7 +92,7 @@ def test_fused_ops_draw_their_mask_on_the_device():
     assert torch.equal(y, y_ref)
 
 
-@pytest.mark.parametrize("ranks", [[16, 16, 16, 16], [8, 64, 32, 128]])
+@pytest.mark.parametrize("ranks", [[16, 16, 16, 16], [8, 64, 32, 128], [64, 48, 16, 64], [32, 8, 24, 32]])
 def test_seeded_forward_draws_the_oracle_mask(ranks):
     """The rank-r forward kernel that draws its own mask writes exactly the oracle's bytes (per-block p,
     padded rows included) and produces the same S and Y, bit for bit, as the run fed that mask."""
