@@ -114,6 +114,76 @@ def test_layer_linears_from_descriptor(manager, monkeypatch):
     assert len(built) == 1, f"the routing of one micro-batch was built {len(built)} times for four linears"
 
 
+def test_linear_driven_by_a_schedule_file(manager, tmp_path):
+    """A JSON schedule of two micro-batches (grouped in one step, as the reference's planner groups them) is loaded
+    and drives a multi-adapter LoRA linear micro-batch by micro-batch: forward and backward of each against the
+    oracle, gradients accumulated over both, sample counts tallied by the manager."""
+    ml = manager
+    from lorafusion_amd.ops import schedule as sch
+    from lorafusion_amd.patch.patch_transformers import DecoderLayerLoRAProjections
+
+    cfgs = [SimpleNamespace(r=r, lora_alpha=al, lora_dropout=0.0) for r, al in ((16, 2.0), (64, 1.0), (8, 4.0))]
+    adapters = {f"lora_{i}": (c.r, c.lora_alpha, c.lora_dropout) for i, c in enumerate(cfgs)}
+    layer = DecoderLayerLoRAProjections.from_shapes(HIDDEN, KV, MLP, adapters, seed=7)
+    _randomise_lora(layer, seed=8)
+    lin = layer.linears()["down"]
+    K, N = lin.in_features, lin.out_features
+    steps = [{"micro_batch_infos": [
+        {"data_samples": [[2, 0, 0, 100], [0, 0, 1, 77], [2, 0, 2, 60], [1, 0, 3, 200]],
+         "max_microbatch_size": 1024, "adapter_padding_multiple": BLOCK, "micro_batch_idx": 0},
+        {"data_samples": [[1, 1, 4, 128], [1, 1, 5, 1]],
+         "max_microbatch_size": 1024, "adapter_padding_multiple": BLOCK, "micro_batch_idx": 1}]}]
+    path = tmp_path / "schedule.json"
+    path.write_text(__import__("json").dumps(steps))
+    mbs = sch.load_schedule(path)
+    assert [mb.padded_total_tokens for mb in mbs] == [256 + 128 + 256, 256]
+
+    mgr = ml.init_multi_lora_manager(cfgs, 1, 1024, [2, 2, 2])
+    g = torch.Generator().manual_seed(21)
+    exp_da = {i: torch.zeros(c.r, K) for i, c in enumerate(cfgs)}
+    exp_db = {i: torch.zeros(N, c.r) for i, c in enumerate(cfgs)}
+    w = lin.base_layer.weight.detach().cpu()
+    for mb in mbs:
+        info = ml.batch_info_from_micro_batch(mb, cfgs)
+        mgr.add_batch_info(info)
+        seq, padded = info.seq_len_list, info.padded_seq_len_list
+        assert seq == [mb.adapter_num_tokens_pairs[i] for i in info.lora_idx_list]
+        Mp = sum(padded)
+        assert Mp == mb.padded_total_tokens
+        x = torch.randn(Mp, K, generator=g).to(torch.bfloat16)
+        dy = torch.randn(Mp, N, generator=g).to(torch.bfloat16)
+        xd = x.cuda().reshape(1, Mp, K).requires_grad_(True)
+        mgr.mark_forward_pass_started()
+        y = lin(xd)
+        mgr.mark_backward_pass_started()
+        y.backward(dy.cuda().reshape(1, Mp, N))
+        torch.cuda.synchronize()
+        mgr.pop_oldest_batch_info()
+        a_list = [lin.lora_A[f"lora_{i}"].weight.detach().cpu() for i in info.lora_idx_list]
+        b_list = [lin.lora_B[f"lora_{i}"].weight.detach().cpu() for i in info.lora_idx_list]
+        scales = [cfgs[i].lora_alpha for i in info.lora_idx_list]
+        p_list = [0.0] * len(seq)
+        if len(seq) == 1:
+            # one active adapter: the reference takes the single-adapter op with the layer's own scaling
+            # (lora_alpha / r) over every row of the padded batch (lorafusion/patch/patch_lora.py:90-117)
+            sc = lin.scaling[f"lora_{info.lora_idx_list[0]}"]
+            ye, _ = lora_ref.linear_lora_fwd_fp32(x, w, a_list[0], b_list[0], sc)
+            dxe, da1, db1, _ = lora_ref.linear_lora_bwd_fp32(dy, x, w, a_list[0], b_list[0], sc)
+            dae, dbe = [da1], [db1]
+        else:
+            ye, _ = lora_ref.linear_multi_lora_fwd_fp32(x, w, a_list, b_list, seq, padded, scales, p_list, None)
+            dxe, dae, dbe, _ = lora_ref.linear_multi_lora_bwd_fp32(dy, x, w, a_list, b_list, seq, padded, scales, p_list, None)
+        _close(y[0], ye, f"micro-batch {mb.micro_batch_idx}: y")
+        _close(xd.grad[0], dxe, f"micro-batch {mb.micro_batch_idx}: dx")
+        for j, i in enumerate(info.lora_idx_list):
+            exp_da[i] += dae[j]
+            exp_db[i] += dbe[j]
+    for i in range(len(cfgs)):
+        _close(lin.lora_A[f"lora_{i}"].weight.grad, exp_da[i], f"accumulated da[{i}]")
+        _close(lin.lora_B[f"lora_{i}"].weight.grad, exp_db[i], f"accumulated db[{i}]")
+    assert mgr.adapter_sample_counts == {0: 1, 1: 3, 2: 2}
+
+
 def test_merged_projections_equal_the_separate_ones(manager):
     """qkv and gate/up as one GEMM each: the column slices are the separate projections' outputs (same base
     weights, no LoRA contribution with B = 0), bit for bit against the plain GEMM of each weight."""
