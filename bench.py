@@ -17,7 +17,9 @@ per linear 2*(2*M*K*N) + 6*M*r*(K+N).  `roofline` describes the dominant kernel 
 each timed live with HIP events on the launch stream.  `cpu_baseline` is the unfused PyTorch expression
 (the oracle's bf16 op-by-op arithmetic with autograd backward) on the host cores.  `workloads` holds the
 reference's other configurations (c1 single linear, c2 packed multi-LoRA linear, c3 NF4 linear, c5 70B-class
-NF4 layer), each with its own roofline entry, and `nf4_dequant` the standalone dequant kernel against HBM peak.
+NF4 layer), each with its own roofline entry, `nf4_dequant` the standalone dequant kernel against HBM peak, and
+`norm_act` the RMSNorm and SiLU-multiply kernels (the steps either side of the layer's linears) at the layer's
+shapes, each against HBM peak; they are measured on their own and are not part of `value`.
 """
 
 from __future__ import annotations
@@ -372,6 +374,52 @@ def nf4_dequant_block(dev) -> dict:
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "nf4_dequant_kernel"}}
 
 
+def norm_act_block(dev) -> dict:
+    """The elementwise steps either side of the 8B layer's linears on its 16512 rows: RMSNorm (hidden 4096) forward
+    and backward, SiLU(gate) * up on the merged [16512, 2 x 14336] projection output, forward and backward (which
+    writes the merged gradient).  Algorithmic bytes per element: 4 (norm forward: read x, write y), 6 (norm
+    backward: read dy and x, write dx), 6 (activation forward), 10 (activation backward)."""
+    from lorafusion_amd import _lib as L
+
+    lib = L.lib()
+    M, H, I = 16512, 4096, 14336
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(M, H, device=dev, generator=g).to(torch.bfloat16)
+    dy = torch.randn(M, H, device=dev, generator=g).to(torch.bfloat16)
+    w = torch.ones(H, device=dev, dtype=torch.bfloat16)
+    y, dx, dw = torch.empty_like(x), torch.empty_like(x), torch.empty_like(w)
+    rstd = torch.empty(M, device=dev)
+    n_ws = lib.lf_rmsnorm_bwd_workspace(M, H)
+    ws = torch.empty(n_ws, dtype=torch.uint8, device=dev)
+    gu = torch.randn(M, 2 * I, device=dev, generator=g).to(torch.bfloat16)
+    dc = torch.randn(M, I, device=dev, generator=g).to(torch.bfloat16)
+    c, dgu = torch.empty(M, I, device=dev, dtype=torch.bfloat16), torch.empty_like(gu)
+    st = L.stream_of(x)
+    calls = {
+        "rmsnorm_fwd": (4 * M * H + 4 * M, "rmsnorm_fwd_kernel", lambda: L.check(lib.lf_rmsnorm_fwd(
+            x.data_ptr(), w.data_ptr(), y.data_ptr(), rstd.data_ptr(), M, H, 1e-6, 0, st), "lf_rmsnorm_fwd")),
+        "rmsnorm_bwd_frozen_weight": (6 * M * H + 4 * M, "rmsnorm_bwd_kernel", lambda: L.check(lib.lf_rmsnorm_bwd(
+            dy.data_ptr(), x.data_ptr(), w.data_ptr(), rstd.data_ptr(), dx.data_ptr(), None, M, H, 0, None, 0, st),
+            "lf_rmsnorm_bwd")),
+        "rmsnorm_bwd_with_dw": (6 * M * H + 4 * M, "rmsnorm_bwd_kernel", lambda: L.check(lib.lf_rmsnorm_bwd(
+            dy.data_ptr(), x.data_ptr(), w.data_ptr(), rstd.data_ptr(), dx.data_ptr(), dw.data_ptr(), M, H, 0,
+            ws.data_ptr(), n_ws, st), "lf_rmsnorm_bwd")),
+        "silu_mul_fwd": (6 * M * I, "silu_mul_fwd_kernel", lambda: L.check(lib.lf_silu_mul_fwd(
+            gu.data_ptr(), gu[:, I:].data_ptr(), c.data_ptr(), M, I, 2 * I, 2 * I, I, 0, st), "lf_silu_mul_fwd")),
+        "silu_mul_bwd": (10 * M * I, "silu_mul_bwd_kernel", lambda: L.check(lib.lf_silu_mul_bwd(
+            dc.data_ptr(), gu.data_ptr(), gu[:, I:].data_ptr(), dgu.data_ptr(), dgu[:, I:].data_ptr(), M, I, I, 2 * I,
+            2 * I, 2 * I, 2 * I, 0, st), "lf_silu_mul_bwd")),
+    }
+    out = {"rows": M, "hidden": H, "intermediate": I}
+    for name, (nbytes, kernel, fn) in calls.items():
+        t = event_time_ms(fn, 50)
+        gbs = nbytes / (t * 1e-3) / 1e9
+        out[name] = {"launch_ms": round(t, 4), "bytes_per_launch": nbytes,
+                     "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                  "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": kernel}}
+    return out
+
+
 # --------------------------------------------------------------------------- the headline: the 8B layer
 
 def layer_c4(args, dev):
@@ -520,7 +568,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload (c4), its roofline and the CPU baseline")
-    ap.add_argument("--only", choices=sorted(WORKLOADS), default=None,
+    ap.add_argument("--only", choices=sorted(WORKLOADS) + ["norm_act"], default=None,
                     help="run one workload through the raw ops and print its entry alone (for profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -539,6 +587,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.only == "norm_act":
+        print(json.dumps({"metric": "norm_act", **norm_act_block(dev)}))
+        return
     if args.only is not None:
         print(json.dumps({"metric": METRIC, **raw_workload(args.only, args, dev, breakdown=not args.no_extras)}))
         return
@@ -568,6 +619,7 @@ def main():
     }
     if not args.no_extras:
         res["nf4_dequant"] = nf4_dequant_block(dev)
+        res["norm_act"] = norm_act_block(dev)
         small = argparse.Namespace(steps=max(5, args.steps // 2), warmup=max(2, args.warmup // 2))
         res["workloads"] = {name: raw_workload(name, args if name == "c2" else small, dev) for name in ("c1", "c2", "c3", "c5")}
     if not args.no_cpu_baseline:

@@ -239,6 +239,31 @@ int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const
  * (seed, element index) only. */
 int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream);
 
+/* RMSNorm and SiLU-multiply: the elementwise steps either side of the LoRA linears of a decoder layer.  The
+ * reference takes them from the liger-kernel package (apply_liger_kernel, lorafusion/utils/module.py:41-71;
+ * liger-kernel==0.5.6, requirements.txt:20); these stand in for that package's LigerRMSNormFunction ("llama"
+ * casting mode, offset 0) and LigerSiLUMulFunction.  HBM-bound streams; X, Y, dY, dX dense [M,H] and W [H] of one
+ * 16-bit dtype, 16-byte aligned, H % 8 == 0, H <= 8192 (LF_ELIMIT beyond).
+ *   forward:  rstd[m] = 1/sqrt(mean_h X[m,h]^2 + eps) (fp32, kept for the backward);
+ *             Y = round16(round16(X * rstd) * W)
+ *   backward: dX = rstd * (dY*W - X * rstd^2 * mean_h(dY*W*X));  dW = sum_m dY * round16(X * rstd) (fp32 sums,
+ *             summed in a fixed order: no atomics).  dX may alias dY.  dW == NULL skips the weight gradient (frozen
+ *             norm weights, the LoRA fine-tuning case) and needs no workspace; otherwise `workspace` holds
+ *             lf_rmsnorm_bwd_workspace(M, H) bytes. */
+int lf_rmsnorm_fwd(const void* X, const void* W, void* Y, float* rstd, int M, int H, float eps, int dtype,
+                   void* stream);
+size_t lf_rmsnorm_bwd_workspace(int M, int H);
+int lf_rmsnorm_bwd(const void* dY, const void* X, const void* W, const float* rstd, void* dX, void* dW, int M, int H,
+                   int dtype, void* workspace, size_t workspace_bytes, void* stream);
+/*   C = round16(round16(silu(A)) * B), silu in fp32;  dB = dC * silu(A),  dA = dC * (silu(A) * (1 - sig(A)) + sig(A)) * B.
+ * All operands [M,I] with their own row strides in elements (ld >= I, ld % 8 == 0, I % 8 == 0, 16-byte aligned
+ * bases), so A and B may be the two halves of a merged gate/up projection output [M,2I] and dA, dB the two halves
+ * of its gradient.  dA may alias A and dB may alias B. */
+int lf_silu_mul_fwd(const void* A, const void* B, void* C, int M, int I, int64_t lda, int64_t ldb, int64_t ldc,
+                    int dtype, void* stream);
+int lf_silu_mul_bwd(const void* dC, const void* A, const void* B, void* dA, void* dB, int M, int I, int64_t lddc,
+                    int64_t lda, int64_t ldb, int64_t ldda, int64_t lddb, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,7 @@ EXPORTS = (
     "lf_version", "lf_strerror", "lf_workspace_bytes", "lf_lora_xa", "lf_lora_xw_sb", "lf_lora_dys_dyb",
     "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant", "lf_dropout_mask",
     "lf_lora_xa_seeded", "lf_lora_fwd_seeded", "lf_nf4_lora_fwd", "lf_nf4_lora_bwd", "lf_lora_bwd_static", "lf_set_tile_cfg", "lf_gemm_plan",
+    "lf_rmsnorm_fwd", "lf_rmsnorm_bwd_workspace", "lf_rmsnorm_bwd", "lf_silu_mul_fwd", "lf_silu_mul_bwd",
 )
 
 
@@ -101,8 +102,15 @@ def lib() -> ctypes.CDLL:
     wp = ctypes.POINTER(NF4Weight)
     l.lf_nf4_lora_fwd.argtypes = [vp, wp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, rp, i, vp]
     l.lf_nf4_lora_bwd.argtypes = [vp, vp, wp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, rp, i, vp]
+    i64, f32 = ctypes.c_int64, ctypes.c_float
+    l.lf_rmsnorm_fwd.argtypes = [vp, vp, vp, vp, i, i, f32, i, vp]
+    l.lf_rmsnorm_bwd_workspace.restype = sz
+    l.lf_rmsnorm_bwd_workspace.argtypes = [i, i]
+    l.lf_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, vp, sz, vp]
+    l.lf_silu_mul_fwd.argtypes = [vp, vp, vp, i, i, i64, i64, i64, i, vp]
+    l.lf_silu_mul_bwd.argtypes = [vp, vp, vp, vp, vp, i, i, i64, i64, i64, i64, i64, i, vp]
     for name in EXPORTS:
-        if name not in ("lf_strerror", "lf_workspace_bytes"):
+        if name not in ("lf_strerror", "lf_workspace_bytes", "lf_rmsnorm_bwd_workspace"):
             getattr(l, name).restype = i
     _lib = l
     return l

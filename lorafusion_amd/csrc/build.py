@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB = os.path.join(PKG, "liblorafusion_hip.so")
-SOURCES = ["gemm_lora.hip", "gemm_big.hip", "lora_skinny.hip", "nf4_dequant.hip", "dropout_mask.hip", "lf_api.hip"]
+SOURCES = ["gemm_lora.hip", "gemm_big.hip", "lora_skinny.hip", "nf4_dequant.hip", "dropout_mask.hip", "norm_act.hip", "lf_api.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

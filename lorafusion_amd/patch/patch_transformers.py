@@ -5,8 +5,8 @@ The reference merges ``q_proj``/``k_proj``/``v_proj`` into one ``qkv_proj`` befo
 slices of one GEMM) so that a layer runs fewer, larger LoRA linears.  This module does the same without
 depending on ``transformers``: any attention / MLP object that holds ``nn.Linear``-like ``q_proj, k_proj,
 v_proj, o_proj`` / ``gate_proj, up_proj, down_proj`` can be converted, and ``gate``/``up`` are merged the
-same way (two GEMMs that share their input).  Attention itself, rotary embedding, norms and the
-activation stay with the caller: only the seven projections are on the fused path.
+same way (two GEMMs that share their input).  Attention itself, rotary embedding and norms stay with the
+caller; the default activation of the layer harness is the SiLU-multiply kernel on the merged gate/up output.
 
 ``LoRALinear`` carries the attributes ``patch_lora.lora_forward`` reads from a PEFT LoRA layer
 (``base_layer``, ``lora_A``, ``lora_B``, ``lora_dropout``, ``scaling``), so single adapter, packed
@@ -23,6 +23,7 @@ from typing import Callable, Iterable
 import torch
 from torch import nn
 
+from lorafusion_amd.ops.norm_act import silu_mul_merged
 from lorafusion_amd.patch.patch_lora import lora_forward
 
 
@@ -118,7 +119,7 @@ class DecoderLayerLoRAProjections(nn.Module):
     merged, N = q + 2 kv), ``o_proj``, ``gate_up_proj`` (N = 2 mlp) and ``down_proj``.
 
     ``forward(hidden, attention=..., activation=...)`` strings them together with the caller's attention
-    (``(q, k, v) -> [tokens, q]``) and activation (``(gate, up) -> [tokens, mlp]``, SwiGLU by default), without
+    (``(q, k, v) -> [tokens, q]``) and activation (``(gate, up) -> [tokens, mlp]``; by default SiLU(gate) * up, computed on the merged tensor), without
     norms or residuals: a harness for layer-shaped runs of the linears, not a transformer block.
     """
 
@@ -155,9 +156,14 @@ class DecoderLayerLoRAProjections(nn.Module):
         q, k, v = self.qkv_proj(hidden)
         ctx = attention(q, k, v) if attention is not None else q
         h = self.o_proj(ctx.contiguous())
-        gate, up = self.gate_up_proj(h)
-        z = activation(gate, up) if activation is not None else torch.nn.functional.silu(gate) * up
-        return self.down_proj(z.contiguous())
+        if activation is None:
+            # SiLU(gate) * up on the merged projection output: its two halves are read in place and the backward
+            # writes the gradient of the merged tensor, so there is no split / cat copy around the activation
+            z = silu_mul_merged(self.gate_up_proj.proj(h))
+        else:
+            gate, up = self.gate_up_proj(h)
+            z = activation(gate, up).contiguous()
+        return self.down_proj(z)
 
 
 def patch_module(model: nn.Module, from_type, transform: Callable, layer_indices: list[int] | None = None) -> nn.Module:
