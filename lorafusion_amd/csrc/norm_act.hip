@@ -236,8 +236,9 @@ rmsnorm_bwd_kernel(const lf_u32x4* __restrict__ dy, const lf_u32x4* __restrict__
   }
 }
 
-// dw[col] = sum over the partial rows in a fixed order: 16 strided groups, then the 16 group sums in order.
-constexpr int DWR_COLS = 64, DWR_GROUPS = 16;
+// dw[col] = sum over the partial rows in a fixed order: 64 strided groups, then the 64 group sums in order.
+// 16 columns per workgroup, so that a 4096-wide row gives every compute unit one workgroup.
+constexpr int DWR_COLS = 16, DWR_GROUPS = 64;
 template <typename T>
 __global__ void __launch_bounds__(DWR_COLS * DWR_GROUPS)
 rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int n_partial, int H, T* __restrict__ dw) {
