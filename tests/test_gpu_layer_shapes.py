@@ -121,9 +121,10 @@ def test_8b_layer_projections(K, N):
     _run_multi(16384, K, N, [16] * 4, [0.0, 0.05, 0.1, 0.1], [1.0, 2.0, 2.0, 4.0])
 
 
-@pytest.mark.parametrize("K,N", [(8192, 8192), (8192, 1024), (8192, 28672), (28672, 8192)])
+@pytest.mark.parametrize("K,N", [(8192, 8192), (8192, 1024), (8192, 10240), (8192, 28672), (8192, 57344), (28672, 8192)])
 def test_70b_layer_projections_nf4(K, N):
-    """8192 tokens, 8 adapters r=64, base weight quantised to NF4 and dequantised on the device."""
+    """8192 tokens, 8 adapters r=64, base weight quantised to NF4 and dequantised on the device; the separate
+    projections and the merged ones (q+k+v: N = 10240, gate+up: N = 57344)."""
     _run_multi(8192, K, N, [64] * 8, [0.0, 0.05, 0.1, 0.1, 0.0, 0.05, 0.1, 0.1], [1.0, 2.0, 2.0, 4.0] * 2, nf4=True)
 
 
