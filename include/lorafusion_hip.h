@@ -261,6 +261,24 @@ int lf_rmsnorm_bwd(const void* dY, const void* X, const void* W, const float* rs
  * of its gradient.  dA may alias A and dB may alias B. */
 int lf_silu_mul_fwd(const void* A, const void* B, void* C, int M, int I, int64_t lda, int64_t ldb, int64_t ldc,
                     int dtype, void* stream);
+/* SiLU-multiply as the prologue of the LoRA linear that follows it (the down projection of a SwiGLU MLP: liger-kernel's
+ * LigerSwiGLUMLP computes down_proj(silu(gate) * up), and the reference's patched down_proj then starts with the
+ * rank-r pass of lorafusion/ops/lora_v1.py:111-119 / multi_lora.py:502-513 on that product).  lf_lora_xa_silu_mul is
+ * lf_lora_xa / lf_lora_xa_seeded whose input X = round16(round16(silu(G)) * U) is computed on the fly from the gate and
+ * up tensors [M,K] (rows `ld` elements apart: the halves of a merged projection output, or two tensors; ld >= K,
+ * ld % 8 == 0, 16-byte aligned) and written once to X_out [M,K] for the base GEMM and the backward: the activation
+ * pass and the rank-r pass's own read of X disappear.  X_out is bit-identical to lf_silu_mul_fwd's output and S to
+ * lf_lora_xa's on it.  mask: explicit keep-mask [M,K] or NULL; mask_out != NULL: the mask is drawn from `seed` as
+ * lf_lora_xa_seeded draws it and written there (mask and mask_out exclude each other); both NULL: no dropout.
+ * lf_swiglu_lora_fwd adds the fused GEMM of lf_lora_xw_sb on X_out: Y = X_out W^T + scale S B^T + bias.
+ * The backward is lf_lora_bwd with X = X_out followed by lf_silu_mul_bwd on its dX. */
+int lf_lora_xa_silu_mul(const void* G, const void* U, int64_t ld, void* X_out, const uint8_t* mask, uint8_t* mask_out,
+                        uint64_t seed, const void* const* a_ptrs, void* S, int M, int K, int R, const lf_routing* routing,
+                        int dtype, void* stream);
+int lf_swiglu_lora_fwd(const void* G, const void* U, int64_t ld, void* X_out, const void* W, const void* bias,
+                       const uint8_t* mask, uint8_t* mask_out, uint64_t seed, const void* const* a_ptrs,
+                       const void* const* b_ptrs, void* Y, void* S_out, int M, int N, int K, int R,
+                       const lf_routing* routing, int dtype, void* stream);
 int lf_silu_mul_bwd(const void* dC, const void* A, const void* B, void* dA, void* dB, int M, int I, int64_t lddc,
                     int64_t lda, int64_t ldb, int64_t ldda, int64_t lddb, int dtype, void* stream);
 

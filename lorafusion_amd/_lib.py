@@ -25,6 +25,7 @@ EXPORTS = (
     "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant", "lf_dropout_mask",
     "lf_lora_xa_seeded", "lf_lora_fwd_seeded", "lf_nf4_lora_fwd", "lf_nf4_lora_bwd", "lf_lora_bwd_static", "lf_set_tile_cfg", "lf_gemm_plan",
     "lf_rmsnorm_fwd", "lf_rmsnorm_bwd_workspace", "lf_rmsnorm_bwd", "lf_silu_mul_fwd", "lf_silu_mul_bwd",
+    "lf_lora_xa_silu_mul", "lf_swiglu_lora_fwd",
 )
 
 
@@ -109,6 +110,8 @@ def lib() -> ctypes.CDLL:
     l.lf_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, vp, sz, vp]
     l.lf_silu_mul_fwd.argtypes = [vp, vp, vp, i, i, i64, i64, i64, i, vp]
     l.lf_silu_mul_bwd.argtypes = [vp, vp, vp, vp, vp, i, i, i64, i64, i64, i64, i64, i, vp]
+    l.lf_lora_xa_silu_mul.argtypes = [vp, vp, i64, vp, vp, vp, ctypes.c_uint64, vp, vp, i, i, i, rp, i, vp]
+    l.lf_swiglu_lora_fwd.argtypes = [vp, vp, i64, vp, vp, vp, vp, vp, ctypes.c_uint64, vp, vp, vp, vp, i, i, i, i, rp, i, vp]
     for name in EXPORTS:
         if name not in ("lf_strerror", "lf_workspace_bytes", "lf_rmsnorm_bwd_workspace"):
             getattr(l, name).restype = i

@@ -4,7 +4,8 @@
 
 int lf_launch_nf4_dequant(const uint8_t*, const void*, const float*, const float*, const float*, void*, int64_t,
                           int, int, int, hipStream_t);
-int lf_launch_xa(const void*, const uint8_t*, uint8_t*, uint64_t, void*, int, int, int, const LfSegTable&, int, hipStream_t);
+int lf_launch_xa(const void*, const void*, int64_t, void*, const uint8_t*, uint8_t*, uint64_t, void*, int, int, int, const LfSegTable&, int,
+                 hipStream_t);
 int lf_launch_dys_dyb(const void*, const void*, void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
 int lf_launch_da(const void*, const uint8_t*, const void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
 int lf_launch_dropout_mask(uint8_t*, int, int, float, const float*, int, uint64_t, hipStream_t);
@@ -122,7 +123,7 @@ int lf_lora_xa(const void* X, const uint8_t* mask, const void* const* a_ptrs, vo
   if (rc != LF_OK) return rc;
   for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
   (void)workspace; (void)ws_bytes;  // no partial sums leave the workgroups
-  return lf_launch_xa(X, mask, nullptr, 0, S, M, K, R, t, dtype, (hipStream_t)stream);
+  return lf_launch_xa(X, nullptr, 0, nullptr, mask, nullptr, 0, S, M, K, R, t, dtype, (hipStream_t)stream);
 }
 
 int lf_lora_xa_seeded(const void* X, uint8_t* mask_out, const void* const* a_ptrs, void* S, int M, int K, int R,
@@ -132,7 +133,28 @@ int lf_lora_xa_seeded(const void* X, uint8_t* mask_out, const void* const* a_ptr
   int rc = make_seg(routing, M, a_ptrs, nullptr, t);
   if (rc != LF_OK) return rc;
   for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
-  return lf_launch_xa(X, nullptr, mask_out, seed, S, M, K, R, t, dtype, (hipStream_t)stream);
+  return lf_launch_xa(X, nullptr, 0, nullptr, nullptr, mask_out, seed, S, M, K, R, t, dtype, (hipStream_t)stream);
+}
+
+int lf_lora_xa_silu_mul(const void* G, const void* U, int64_t ld, void* X_out, const uint8_t* mask, uint8_t* mask_out,
+                        uint64_t seed, const void* const* a_ptrs, void* S, int M, int K, int R, const lf_routing* routing,
+                        int dtype, void* stream) {
+  if (bad_dtype(dtype) || !a_ptrs || !G || !U || !X_out) return LF_EINVAL;
+  if (mask && mask_out) return LF_EINVAL;
+  LfSegTable t;
+  int rc = make_seg(routing, M, a_ptrs, nullptr, t);
+  if (rc != LF_OK) return rc;
+  for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
+  return lf_launch_xa(G, U, ld, X_out, mask, mask_out, seed, S, M, K, R, t, dtype, (hipStream_t)stream);
+}
+
+int lf_swiglu_lora_fwd(const void* G, const void* U, int64_t ld, void* X_out, const void* W, const void* bias,
+                       const uint8_t* mask, uint8_t* mask_out, uint64_t seed, const void* const* a_ptrs,
+                       const void* const* b_ptrs, void* Y, void* S_out, int M, int N, int K, int R,
+                       const lf_routing* routing, int dtype, void* stream) {
+  int rc = lf_lora_xa_silu_mul(G, U, ld, X_out, mask, mask_out, seed, a_ptrs, S_out, M, K, R, routing, dtype, stream);
+  if (rc != LF_OK) return rc;
+  return lf_lora_xw_sb(X_out, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype, stream);
 }
 
 int lf_lora_xw_sb(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs,

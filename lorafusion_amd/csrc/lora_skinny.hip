@@ -29,6 +29,7 @@
 // 4-row x 16-column patch; lane 4j+c addresses row j, columns 4c..4c+3; each lane receives
 // its column's 4 rows).
 #include "lf_common.h"
+#include "act_math.h"
 #include "philox.h"
 
 namespace {
@@ -169,8 +170,9 @@ __device__ __forceinline__ lf_u32x4 tile_tr_frag(const char* tile, int row, int 
 // A next to 140 MB of X at 8576 x 8192).  Ranks 48-64 take 64 rows (four row blocks share one set of A fragments)
 // and eight waves: 0.50 -> 0.40 ms over the four linears of the rank-64 layer.  At rank 16 two row blocks per
 // workgroup measured slower (0.27 -> 0.34 ms at the 8B layer: the registers of the second block cost loads in flight).
-constexpr int xa_nb(int rt) { return rt == 4 ? 4 : rt > 4 ? 2 : 1; }
-constexpr int xa_rows(int rt) { return 16 * xa_nb(rt); }
+// (with the activation prologue the up-half registers of four row blocks do not fit next to the rest at ranks 48-64: two)
+constexpr int xa_nb(int rt, bool act = false) { return rt == 4 ? (act ? 2 : 4) : rt > 4 ? 2 : 1; }
+constexpr int xa_rows(int rt, bool act = false) { return 16 * xa_nb(rt, act); }
 // waves per workgroup and steps in flight per wave, by rank tiles (LDS: 2 KB * (1+RT) per wave; registers: 8 * RT per step)
 constexpr int xa_waves(int rt) { return rt <= 4 ? 8 : 2; }
 constexpr int xa_unroll(int rt) { return rt <= 1 ? 4 : rt <= 2 ? 2 : 1; }
@@ -178,11 +180,17 @@ constexpr int xa_unroll(int rt) { return rt <= 1 ? 4 : rt <= 2 ? 2 : 1; }
 // GEN: the keep-mask is not read but drawn here (Philox, the definition of the standalone mask
 // kernel) from (seed, element index) and written to `mask_out` for the backward pass: the integer
 // work hides behind the X stream, and one launch and one 1-byte-per-element read disappear.
-template <typename T, int RT, bool GEN>
+// ACT: the rows of X do not exist yet: X = round16(round16(silu(G)) * U) is computed here from the gate and up halves of a
+// SwiGLU MLP (`X` = G, `U`, rows `ldx` elements apart: the two halves of one merged projection output, or two
+// tensors), written once to `act_out` [rows, K] (every element of X is loaded by exactly one lane of the grid) for the
+// base GEMM and the backward, and fed to the rank-r product from registers: the activation pass and this pass's own
+// read of X disappear.
+template <typename T, int RT, bool GEN, bool ACT>
 __global__ void __launch_bounds__(xa_waves(RT) * 64)
-lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_t* __restrict__ mask_out,
+lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T* __restrict__ act_out,
+               const uint8_t* __restrict__ mask, uint8_t* __restrict__ mask_out,
                uint32_t seed_lo, uint32_t seed_hi, T* __restrict__ S, int M, int K, int R, const LfSegTable seg) {
-  constexpr int XA_WAVES = xa_waves(RT), XA_U = xa_unroll(RT), NB = xa_nb(RT), XA_ROWS = xa_rows(RT);
+  constexpr int XA_WAVES = xa_waves(RT), XA_U = xa_unroll(RT), NB = xa_nb(RT, ACT), XA_ROWS = xa_rows(RT, ACT);
   // the partial accumulators of the final sum reuse the patches (a barrier separates the two uses): at
   // rank 64 the separate 16 KB pushed the workgroup over 40 KB, and a CU then holds two workgroups, not four
   constexpr int PATCH_BYTES = XA_WAVES * 2048 * (NB + RT), RED_BYTES = XA_WAVES * XA_ROWS * RT * 16 * 4;
@@ -204,16 +212,18 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
   const int lrow = lane >> 3, lg = lane & 7;
   const T* xrow[2 * NB];
   const uint8_t* mrow[2 * NB];
-  int64_t erow[2 * NB];    // GEN: element index of this lane's first column in each of its rows (two per 16-row block)
-  bool row_real[2 * NB];   // GEN: the row exists (is not a clamped duplicate): its mask bytes are written
+  int64_t erow[2 * NB];    // GEN, ACT: element index of this lane's first column in each of its rows (two per 16-row block)
+  bool row_real[2 * NB];   // GEN, ACT: the row exists (is not a clamped duplicate): its mask bytes / activations are written
 #pragma unroll
   for (int i = 0; i < 2 * NB; i++) {
     const int r = min(row0 + i * 8 + lrow, Mrows - 1);
-    xrow[i] = X + (int64_t)r * K + lg * 8;
+    xrow[i] = X + (int64_t)r * ldx + lg * 8;
     mrow[i] = mask + (int64_t)r * K + lg * 8;
     erow[i] = (int64_t)r * K + lg * 8;
     row_real[i] = row0 + i * 8 + lrow < Mrows;
   }
+  // ACT: the up half lies at one distance from the gate half for every row (a scalar, not a second set of row pointers)
+  const int64_t u_off = ACT ? (int64_t)((uintptr_t)U - (uintptr_t)X) : 0;
   const int wr_off[2] = {lrow * 128 + ((lg ^ ((lrow >> 1) & 7)) << 4), (8 + lrow) * 128 + ((lg ^ (((8 + lrow) >> 1) & 7)) << 4)};
   const int rd_row = li * 128, rd_key = (li >> 1) & 7;
 
@@ -225,6 +235,7 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
 
   // (a second register set to overlap the next batch's loads costs occupancy and measured slower)
   lf_u32x4 xv[1][XA_U][2 * NB], av[1][XA_U][RT][2];
+  lf_u32x4 uv[1][XA_U][ACT ? 2 * NB : 1];
   lf_u32x2 mv[1][XA_U][2 * NB];
   auto load_batch = [&](int b, int s0) {
 #pragma unroll
@@ -234,6 +245,7 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
 #pragma unroll
         for (int i = 0; i < 2 * NB; i++) {
           xv[b][u][i] = *((const lf_u32x4*)(xrow[i] + s * 64));
+          if constexpr (ACT) uv[b][u][i] = *((const lf_u32x4*)((const char*)(xrow[i] + s * 64) + u_off));
           if constexpr (!GEN) {
             if (use_mask) mv[b][u][i] = *((const lf_u32x2*)(mrow[i] + s * 64));
           }
@@ -257,6 +269,10 @@ lora_xa_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, uint8_
       if (s < nsteps) {
 #pragma unroll
         for (int i = 0; i < 2 * NB; i++) {
+          if constexpr (ACT) {
+            xv[b][u][i] = silu_mul8<T>(xv[b][u][i], uv[b][u][i]);
+            if (row_real[i]) *(lf_u32x4*)(act_out + erow[i] + s * 64) = xv[b][u][i];
+          }
           if constexpr (GEN) {
             uint32_t klo, khi;
             lf_keep8((uint64_t)(erow[i] + s * 64) >> 3, thr, seed_lo, seed_hi, klo, khi);
@@ -1237,38 +1253,52 @@ static DysRingPlan dysr_plan(int M, int N, int R, const LfSegTable& seg) {
 size_t lf_xa_workspace(int, int, int, const LfSegTable&) { return 0; }
 
 template <typename T, int RT>
-static int xa_launch(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t seed, void* S, int M, int K, int R,
-                     int64_t rows, const LfSegTable& seg, hipStream_t st) {
-  const unsigned grid = (unsigned)((rows + xa_rows(RT) - 1) / xa_rows(RT));
-  if (mask_out != nullptr)
-    return lf_launch((lora_xa_kernel<T, RT, true>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
-                       (uint32_t)seed, (uint32_t)(seed >> 32), (T*)S, M, K, R, seg);
-  return lf_launch((lora_xa_kernel<T, RT, false>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X, mask, mask_out,
-                       0u, 0u, (T*)S, M, K, R, seg);
+static int xa_launch(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out,
+                     uint64_t seed, void* S, int M, int K, int R, int64_t rows, const LfSegTable& seg, hipStream_t st) {
+  const bool gen = mask_out != nullptr, act = U != nullptr;
+  const int wg_rows = xa_rows(RT, act);
+  const unsigned grid = (unsigned)((rows + wg_rows - 1) / wg_rows);
+  const uint32_t lo = gen ? (uint32_t)seed : 0u, hi = gen ? (uint32_t)(seed >> 32) : 0u;
+#define LF_XA(GEN, ACT)                                                                                              \
+  return lf_launch((lora_xa_kernel<T, RT, GEN, ACT>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X,       \
+                   (const T*)U, ldx, (T*)act_out, mask, mask_out, lo, hi, (T*)S, M, K, R, seg)
+  if (gen && act) LF_XA(true, true);
+  if (gen) LF_XA(true, false);
+  if (act) LF_XA(false, true);
+  LF_XA(false, false);
+#undef LF_XA
 }
 
 template <typename T>
-static int xa_impl(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t seed, void* S, int M, int K, int R,
-                   const LfSegTable& seg, hipStream_t st) {
+static int xa_impl(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out,
+                   uint64_t seed, void* S, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
   switch (rt_of(R)) {
-    case 1: return xa_launch<T, 1>(X, mask, mask_out, seed, S, M, K, R, rows, seg, st);
-    case 2: return xa_launch<T, 2>(X, mask, mask_out, seed, S, M, K, R, rows, seg, st);
-    case 4: return xa_launch<T, 4>(X, mask, mask_out, seed, S, M, K, R, rows, seg, st);
-    default: return xa_launch<T, 8>(X, mask, mask_out, seed, S, M, K, R, rows, seg, st);
+    case 1: return xa_launch<T, 1>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, rows, seg, st);
+    case 2: return xa_launch<T, 2>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, rows, seg, st);
+    case 4: return xa_launch<T, 4>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, rows, seg, st);
+    default: return xa_launch<T, 8>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, rows, seg, st);
   }
 }
 
 // mask_out != nullptr: draw the keep-mask from `seed` (written to mask_out [rows, K]) instead of reading `mask`.
-int lf_launch_xa(const void* X, const uint8_t* mask, uint8_t* mask_out, uint64_t seed, void* S, int M, int K, int R,
-                 const LfSegTable& seg, int dtype, hipStream_t st) {
+// U != nullptr: X and U are the gate and up halves (rows ldx elements apart) and the pass's input
+// round16(round16(silu(X)) * U) is written to act_out [rows, K]; otherwise X [rows, K] is dense.
+int lf_launch_xa(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out,
+                 uint64_t seed, void* S, int M, int K, int R, const LfSegTable& seg, int dtype, hipStream_t st) {
   if (!X || !S || M <= 0 || K <= 0) return LF_EINVAL;
   if (K % 128 != 0 || R % 16 != 0 || R <= 0 || R > LF_MAX_RANK) return LF_ESHAPE;
   if (seg.table && seg.block_size_m != ROWS) return LF_ESHAPE;
   if (mask_out != nullptr && ((uintptr_t)mask_out & 7) != 0) return LF_ESHAPE;
-  if (dtype == LF_BF16) return xa_impl<__bf16>(X, mask, mask_out, seed, S, M, K, R, seg, st);
-  if (dtype == LF_F16) return xa_impl<_Float16>(X, mask, mask_out, seed, S, M, K, R, seg, st);
+  if (U != nullptr) {
+    if (!act_out) return LF_EINVAL;
+    if (ldx < K || ldx % 8 != 0 || (((uintptr_t)X | (uintptr_t)U | (uintptr_t)act_out) & 15) != 0) return LF_ESHAPE;
+  } else {
+    ldx = K;
+  }
+  if (dtype == LF_BF16) return xa_impl<__bf16>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, seg, st);
+  if (dtype == LF_F16) return xa_impl<_Float16>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, seg, st);
   return LF_EINVAL;
 }
 

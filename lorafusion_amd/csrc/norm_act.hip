@@ -16,41 +16,9 @@
 // SiLU-multiply takes row strides, so gate and up may be the two halves of one merged [M, 2I] projection output and
 // da / db the two halves of its gradient.
 #include "lf_common.h"
+#include "act_math.h"
 
 namespace {
-
-template <typename T> __device__ __forceinline__ void unpack8(const lf_u32x4& v, float f[8]);
-template <> __device__ __forceinline__ void unpack8<__bf16>(const lf_u32x4& v, float f[8]) {
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const uint32_t u = v[i];
-    f[2 * i] = __builtin_bit_cast(float, u << 16);
-    f[2 * i + 1] = __builtin_bit_cast(float, u & 0xffff0000u);
-  }
-}
-template <> __device__ __forceinline__ void unpack8<_Float16>(const lf_u32x4& v, float f[8]) {
-  typedef _Float16 v2 __attribute__((ext_vector_type(2)));
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const uint32_t u = v[i];  // a copy: bit_cast applied to the vector element itself reads element 0 for every i
-    const v2 h = __builtin_bit_cast(v2, u);
-    f[2 * i] = (float)h[0];
-    f[2 * i + 1] = (float)h[1];
-  }
-}
-
-template <typename T> __device__ __forceinline__ lf_u32x4 pack8(const float f[8]) {
-  typedef T v2 __attribute__((ext_vector_type(2)));
-  lf_u32x4 o;
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const v2 h = {(T)f[2 * i], (T)f[2 * i + 1]};
-    o[i] = __builtin_bit_cast(uint32_t, h);
-  }
-  return o;
-}
-
-template <typename T> __device__ __forceinline__ float round16(float v) { return (float)(T)v; }
 
 // Makes the compiler treat a packed vector as changed: the fp32 values unpacked from it cannot be kept alive across
 // this point (or hoisted out of a loop), only the packed registers are.  Emits no instruction.
@@ -258,8 +226,6 @@ rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int n_partial, int H
   }
 }
 
-// exp and reciprocal to one unit in the last place of fp32 each (the results are rounded to 16 bits)
-__device__ __forceinline__ float sigmoid_f32(float a) { return __builtin_amdgcn_rcpf(1.0f + __expf(-a)); }
 
 constexpr int ACT_THREADS = 256;
 
@@ -282,12 +248,7 @@ silu_mul_fwd_kernel(const lf_u32x4* __restrict__ a, const lf_u32x4* __restrict__
 #pragma unroll
   for (int i = 0; i < ROWS; i++)
     if (row0 + i < M) {
-      float fa[8], fb[8];
-      unpack8<T>(av[i], fa);
-      unpack8<T>(bv[i], fb);
-#pragma unroll
-      for (int e = 0; e < 8; e++) fa[e] = round16<T>(fa[e] * sigmoid_f32(fa[e])) * fb[e];
-      c[(int64_t)(row0 + i) * ldc + col] = pack8<T>(fa);
+      c[(int64_t)(row0 + i) * ldc + col] = silu_mul8<T>(av[i], bv[i]);
     }
 }
 

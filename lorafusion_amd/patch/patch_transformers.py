@@ -6,7 +6,8 @@ slices of one GEMM) so that a layer runs fewer, larger LoRA linears.  This modul
 depending on ``transformers``: any attention / MLP object that holds ``nn.Linear``-like ``q_proj, k_proj,
 v_proj, o_proj`` / ``gate_proj, up_proj, down_proj`` can be converted, and ``gate``/``up`` are merged the
 same way (two GEMMs that share their input).  Attention itself, rotary embedding and norms stay with the
-caller; the default activation of the layer harness is the SiLU-multiply kernel on the merged gate/up output.
+caller; the default activation of the layer harness is SiLU-multiply on the merged gate/up output, computed inside
+the first kernel of the down projection (``swiglu_lora_forward``).
 
 ``LoRALinear`` carries the attributes ``patch_lora.lora_forward`` reads from a PEFT LoRA layer
 (``base_layer``, ``lora_A``, ``lora_B``, ``lora_dropout``, ``scaling``), so single adapter, packed
@@ -23,8 +24,7 @@ from typing import Callable, Iterable
 import torch
 from torch import nn
 
-from lorafusion_amd.ops.norm_act import silu_mul_merged
-from lorafusion_amd.patch.patch_lora import lora_forward
+from lorafusion_amd.patch.patch_lora import lora_forward, swiglu_lora_forward
 
 
 @torch.no_grad()
@@ -157,13 +157,11 @@ class DecoderLayerLoRAProjections(nn.Module):
         ctx = attention(q, k, v) if attention is not None else q
         h = self.o_proj(ctx.contiguous())
         if activation is None:
-            # SiLU(gate) * up on the merged projection output: its two halves are read in place and the backward
-            # writes the gradient of the merged tensor, so there is no split / cat copy around the activation
-            z = silu_mul_merged(self.gate_up_proj.proj(h))
-        else:
-            gate, up = self.gate_up_proj(h)
-            z = activation(gate, up).contiguous()
-        return self.down_proj(z)
+            # SiLU(gate) * up on the merged projection output, as the prologue of the down projection's rank-r pass:
+            # the two halves are read in place, once, and the backward writes the gradient of the merged tensor
+            return swiglu_lora_forward(self.down_proj, self.gate_up_proj.proj(h), use_fused=self.down_proj.use_fused)
+        gate, up = self.gate_up_proj(h)
+        return self.down_proj(activation(gate, up).contiguous())
 
 
 def patch_module(model: nn.Module, from_type, transform: Callable, layer_indices: list[int] | None = None) -> nn.Module:
