@@ -377,8 +377,9 @@ def nf4_dequant_block(dev) -> dict:
 def norm_act_block(dev) -> dict:
     """The elementwise steps either side of the 8B layer's linears on its 16512 rows: RMSNorm (hidden 4096) forward
     and backward, SiLU(gate) * up on the merged [16512, 2 x 14336] projection output, forward and backward (which
-    writes the merged gradient).  Algorithmic bytes per element: 4 (norm forward: read x, write y), 6 (norm
-    backward: read dy and x, write dx), 6 (activation forward), 10 (activation backward)."""
+    writes the merged gradient), and the activation folded into the down projection's rank-r pass.  Algorithmic bytes per
+    element: 4 (norm forward: read x, write y), 6 (norm backward: read dy and x, write dx), 6 (activation forward),
+    10 (activation backward)."""
     from lorafusion_amd import _lib as L
 
     lib = L.lib()
@@ -410,6 +411,26 @@ def norm_act_block(dev) -> dict:
             dc.data_ptr(), gu.data_ptr(), gu[:, I:].data_ptr(), dgu.data_ptr(), dgu[:, I:].data_ptr(), M, I, I, 2 * I,
             2 * I, 2 * I, 2 * I, 0, st), "lf_silu_mul_bwd")),
     }
+    # the down projection's rank-r pass (4 adapters r=16, the layer's segments, keep-mask drawn in the kernel) with the
+    # activation as its prologue, next to the activation kernel followed by the plain pass.  Algorithmic bytes per
+    # element: 7 fused (read gate and up, write the product and the mask byte), 6 + 3 separate.
+    from lorafusion_amd.ops import multi_lora as ml
+
+    seq = segments(16384, 4, seed=0, longest=8192)
+    info = ml.prepare_multi_lora_batch_info(seq, [0, 1, 2, 3], [16] * 4, [0.0, 0.05, 0.1, 0.1], [1.0, 2.0, 2.0, 4.0], 128)
+    rt = info.routing(enable_dropout=True)
+    assert rt.M == M
+    a_list = [torch.randn(16, I, device=dev, generator=g).to(torch.bfloat16) * 0.01 for _ in range(4)]
+    a_ptrs = L.ptr_array(a_list)
+    s_out = torch.empty(M, 16, device=dev, dtype=torch.bfloat16)
+    mask_out = torch.empty(M, I, device=dev, dtype=torch.bool)
+    seed = ctypes.c_uint64(1234)
+    calls["down_xa_with_silu_mul_prologue"] = (7 * M * I, "lora_xa_kernel<.., seeded, activation>", lambda: L.check(
+        lib.lf_lora_xa_silu_mul(gu.data_ptr(), gu[:, I:].data_ptr(), 2 * I, c.data_ptr(), None, mask_out.data_ptr(), seed,
+                                a_ptrs, s_out.data_ptr(), M, I, 16, rt.c, 0, st), "lf_lora_xa_silu_mul"))
+    calls["down_xa_seeded_alone"] = (3 * M * I, "lora_xa_kernel<.., seeded>", lambda: L.check(
+        lib.lf_lora_xa_seeded(c.data_ptr(), mask_out.data_ptr(), a_ptrs, s_out.data_ptr(), M, I, 16, rt.c, seed, 0, st),
+        "lf_lora_xa_seeded"))
     out = {"rows": M, "hidden": H, "intermediate": I}
     for name, (nbytes, kernel, fn) in calls.items():
         t = event_time_ms(fn, 50)
@@ -417,6 +438,8 @@ def norm_act_block(dev) -> dict:
         out[name] = {"launch_ms": round(t, 4), "bytes_per_launch": nbytes,
                      "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                   "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": kernel}}
+    out["down_prologue_saving_ms"] = round(out["silu_mul_fwd"]["launch_ms"] + out["down_xa_seeded_alone"]["launch_ms"]
+                                           - out["down_xa_with_silu_mul_prologue"]["launch_ms"], 4)
     return out
 
 
