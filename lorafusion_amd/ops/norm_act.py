@@ -176,5 +176,15 @@ def silu_mul_merged(gate_up: torch.Tensor) -> torch.Tensor:
 
 def swiglu_mlp_forward(mlp: nn.Module, x: torch.Tensor) -> torch.Tensor:
     """``down_proj(silu(gate_proj(x)) * up_proj(x))`` of an HF Llama / Qwen2 MLP (what liger's ``LigerSwiGLUMLP``
-    computes), through whatever the three projections are (plain or LoRA linears)."""
-    return mlp.down_proj(silu_mul(mlp.gate_proj(x), mlp.up_proj(x)))
+    computes), through whatever the three projections are.  A ``down_proj`` that is a LoRA linear on the fused ops
+    (a PEFT layer under ``apply_lora``, or ``LoRALinear``) takes the activation as the prologue of its first kernel."""
+    from lorafusion_amd.patch import patch_lora
+
+    gate, up = mlp.gate_proj(x), mlp.up_proj(x)
+    down = mlp.down_proj
+    fused = getattr(down, "use_fused", None)
+    if fused is None:
+        fused = getattr(type(down), "_lorafusion_use_fused", None)
+    if fused and patch_lora._is_lora_linear(down) and gate.shape[-1] % 128 == 0:
+        return patch_lora.swiglu_lora_forward(down, gate, up, use_fused=True)
+    return down(silu_mul(gate, up))

@@ -135,21 +135,26 @@ def lora_forward(model, x: torch.Tensor, *args, use_fused: bool = True, **kwargs
     return result.to(result_dtype)
 
 
-def swiglu_lora_forward(model, gate_up: torch.Tensor, *, use_fused: bool = True) -> torch.Tensor:
+def swiglu_lora_forward(model, gate_up: torch.Tensor, up: "torch.Tensor | None" = None, *, use_fused: bool = True) -> torch.Tensor:
     """``lora_forward(model, silu(gate) * up)`` for the down projection of a SwiGLU MLP, with gate and up the two halves
-    of ``gate_up``: on the fused path the activation is the prologue of the linear's rank-r pass (one pass over the
+    of ``gate_up`` (or ``gate_up`` the gate tensor and ``up`` given separately): on the fused path the activation is the prologue of the linear's rank-r pass (one pass over the
     gate/up tensor instead of an activation pass plus a pass over its output).  Same adapter selection as
     ``lora_forward``; NF4 base weights and ``use_fused=False`` take the activation kernel followed by ``lora_forward``."""
-    from lorafusion_amd.ops.norm_act import silu_mul_merged
+    from lorafusion_amd.ops.norm_act import silu_mul, silu_mul_merged
     from lorafusion_amd.ops.swiglu_lora import fused_swiglu_linear_lora, fused_swiglu_linear_multi_lora
 
     if not _is_lora_linear(model):
         raise TypeError(f"model must be a LoRALinear, but got {type(model)}")
     weight = model.base_layer.weight
     if not use_fused or _nf4_state(weight) is not None or not gate_up.is_cuda:
-        return lora_forward(model, silu_mul_merged(gate_up) if gate_up.is_cuda else
-                            torch.nn.functional.silu(gate_up[..., : gate_up.shape[-1] // 2]) * gate_up[..., gate_up.shape[-1] // 2:],
-                            use_fused=use_fused)
+        if up is not None:
+            act = silu_mul(gate_up, up) if gate_up.is_cuda else torch.nn.functional.silu(gate_up) * up
+        elif gate_up.is_cuda:
+            act = silu_mul_merged(gate_up)
+        else:
+            half = gate_up.shape[-1] // 2
+            act = torch.nn.functional.silu(gate_up[..., :half]) * gate_up[..., half:]
+        return lora_forward(model, act, use_fused=use_fused)
     manager = get_multi_lora_manager()
     result_dtype = gate_up.dtype
     linear_bias = getattr(model.base_layer, "bias", None)
@@ -159,7 +164,8 @@ def swiglu_lora_forward(model, gate_up: torch.Tensor, *, use_fused: bool = True)
         lora_b = model.lora_B[adapter_key].weight
         p = float(getattr(model.lora_dropout[adapter_key], "p", 0.0)) if model.training else 0.0
         return fused_swiglu_linear_lora(_cast_input(model, gate_up, lora_a.dtype), weight, lora_a, lora_b,
-                                        model.scaling[adapter_key], dropout_p=p, linear_bias=linear_bias)
+                                        model.scaling[adapter_key], dropout_p=p, linear_bias=linear_bias,
+                                        up=None if up is None else _cast_input(model, up, lora_a.dtype))
 
     if manager is None:
         if len(model.lora_A) > 1:
@@ -179,7 +185,8 @@ def swiglu_lora_forward(model, gate_up: torch.Tensor, *, use_fused: bool = True)
         if g.shape[0] != 1:
             raise ValueError("currently, we only support batch size 1 for multi-linear LoRA")
     return fused_swiglu_linear_multi_lora(g, weight, lora_a_list, lora_b_list, info.routing(enable_dropout=enable_dropout),
-                                          linear_bias=linear_bias).to(result_dtype)
+                                          linear_bias=linear_bias,
+                                          up=None if up is None else _cast_input(model, up, lora_a_list[0].dtype)).to(result_dtype)
 
 
 def apply_lora(*, use_fused: bool = True, target_cls=None) -> None:
@@ -192,3 +199,4 @@ def apply_lora(*, use_fused: bool = True, target_cls=None) -> None:
         return lora_forward(self, x, *args, use_fused=use_fused, **kwargs)
 
     cls.forward = forward_wrapper
+    cls._lorafusion_use_fused = use_fused   # read by the SwiGLU MLP forward to pick the prologue path for down_proj

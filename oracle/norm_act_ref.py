@@ -87,4 +87,4 @@ def ulp16_err(actual: torch.Tensor, expected: torch.Tensor) -> float:
     e = expected.double()
     mag = e.abs().clamp_min(torch.finfo(actual.dtype).tiny)
     spacing = torch.exp2(torch.floor(torch.log2(mag)) - (bits - 1))
-    return float(((actual.double() - e).abs() / spacing).max())
+    return float(((actual.detach().double() - e).abs() / spacing).max())

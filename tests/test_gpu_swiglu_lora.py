@@ -209,3 +209,67 @@ def test_argument_errors():
     with pytest.raises(ValueError, match="multiple of 256"):
         fused_swiglu_linear_lora(gu[:, :384].contiguous(), torch.zeros(128, 192, dtype=torch.bfloat16, device="cuda"), a[:, :192], 
                                  torch.zeros(128, 16, dtype=torch.bfloat16, device="cuda"), 1.0)
+
+
+def test_separate_gate_and_up_tensors_and_the_patched_hf_mlp():
+    """gate and up as two tensors (what HF's ``LlamaMLP`` produces): the same results as the merged layout, bit for
+    bit; and an HF ``LlamaMLP`` whose ``down_proj`` is a LoRA linear takes the prologue path under
+    ``apply_liger_kernel`` and matches the unpatched module."""
+    from transformers.models.llama import modeling_llama as mlm
+    from transformers.models.llama.configuration_llama import LlamaConfig
+
+    from lorafusion_amd import _lib as L
+    from lorafusion_amd.ops.swiglu_lora import fused_swiglu_linear_lora
+    from lorafusion_amd.patch.patch_transformers import LoRALinear
+    from lorafusion_amd.utils.module import apply_liger_kernel, restore_liger_kernel
+
+    M, K, N, r = 260, 512, 384, 32
+    d = single_inputs(M, K, N, r, p=0.1, seed=3)
+    gu = _gate_up(M, K, torch.bfloat16, 4).cuda()
+
+    def run(separate):
+        a, b = d["a"].cuda().requires_grad_(True), d["b"].cuda().requires_grad_(True)
+        if separate:
+            g, u = gu[:, :K].contiguous().requires_grad_(True), gu[:, K:].contiguous().requires_grad_(True)
+            y = fused_swiglu_linear_lora(g, d["w"].cuda(), a, b, 2.0, dropout_p=0.1, dropout_mask=d["mask"].cuda(), up=u)
+        else:
+            g = gu.clone().requires_grad_(True)
+            y = fused_swiglu_linear_lora(g, d["w"].cuda(), a, b, 2.0, dropout_p=0.1, dropout_mask=d["mask"].cuda())
+        y.backward(d["dy"].cuda())
+        dg = torch.cat([g.grad, u.grad], dim=1) if separate else g.grad
+        return y.detach(), dg, a.grad, b.grad
+
+    for got, exp in zip(run(True), run(False)):
+        assert torch.equal(got, exp)
+
+    H, I = 256, 512
+    cfg = LlamaConfig(hidden_size=H, intermediate_size=I, num_hidden_layers=1, num_attention_heads=4,
+                      num_key_value_heads=4, vocab_size=32)
+    torch.manual_seed(0)
+    mlp = mlm.LlamaMLP(cfg).to("cuda", torch.bfloat16)
+    mlp.down_proj = LoRALinear(mlp.down_proj, {"default": (16, 32.0, 0.0)})
+    torch.nn.init.normal_(mlp.down_proj.lora_B["default"].weight, std=0.02)
+    x = torch.randn(200, H, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).cuda()
+    ref = mlp(x)
+    calls = []
+    real_lib = L.lib()
+
+    class _Lib:
+        def __getattr__(self, name):
+            if name == "lf_swiglu_lora_fwd":
+                calls.append(1)
+            return getattr(real_lib, name)
+
+    apply_liger_kernel("all")
+    try:
+        import unittest.mock as mock
+
+        with mock.patch.object(L, "lib", lambda: _Lib()):
+            xr = x.clone().requires_grad_(True)
+            out = mlp(xr)
+            out.float().square().mean().backward()
+    finally:
+        restore_liger_kernel()
+    assert len(calls) == 1
+    _close(out, ref.detach().float().cpu(), "patched MLP with a LoRA down projection")
+    assert torch.isfinite(xr.grad.float()).all() and mlp.down_proj.lora_A["default"].weight.grad is not None
