@@ -53,3 +53,54 @@ def test_forward_backward_replay_matches_eager():
         torch.cuda.synchronize()
         for k, (g, e) in enumerate(zip(got, want)):
             assert torch.equal(g, e), f"replay {replay}: output {k} differs from the eager call"
+
+
+def test_norm_activation_and_prologue_replay_matches_eager():
+    """RMSNorm forward / backward (with dw: two kernels and a workspace), SiLU-multiply, and the down projection with
+    the activation as its prologue, captured once and replayed on fresh values."""
+    from lorafusion_amd.ops import norm_act
+    from lorafusion_amd.ops.swiglu_lora import fused_swiglu_linear_lora
+
+    M, H, I, N, r = 300, 512, 768, 256, 16
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn(M, H, device="cuda", generator=g).to(torch.bfloat16)
+    dyn = torch.randn(M, H, device="cuda", generator=g).to(torch.bfloat16)
+    wn = (1 + 0.1 * torch.randn(H, device="cuda", generator=g)).to(torch.bfloat16)
+    gu = torch.randn(M, 2 * I, device="cuda", generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, I, device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+    a = (torch.randn(r, I, device="cuda", generator=g) * 0.03).to(torch.bfloat16)
+    b = (torch.randn(N, r, device="cuda", generator=g) * 0.01).to(torch.bfloat16)
+    dy = torch.randn(M, N, device="cuda", generator=g).to(torch.bfloat16)
+
+    def run():
+        xs, ws = x.detach().requires_grad_(True), wn.detach().requires_grad_(True)
+        y = norm_act.rms_norm(xs, ws, 1e-5)
+        y.backward(dyn)
+        gs, a_, b_ = gu.detach().requires_grad_(True), a.detach().requires_grad_(True), b.detach().requires_grad_(True)
+        z = fused_swiglu_linear_lora(gs, w, a_, b_, 2.0, seed=11, dropout_p=0.1)
+        z.backward(dy)
+        return [y.detach(), xs.grad, ws.grad, z.detach(), gs.grad, a_.grad, b_.grad]
+
+    run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        run()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            outs = run()
+    torch.cuda.synchronize()
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    for replay in range(3):
+        x.copy_(torch.randn(x.shape, generator=gen, device="cuda").to(x.dtype))
+        gu.copy_(torch.randn(gu.shape, generator=gen, device="cuda").to(gu.dtype))
+        dy.copy_(torch.randn(dy.shape, generator=gen, device="cuda").to(dy.dtype))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        want = run()
+        torch.cuda.synchronize()
+        for k, (g_, e_) in enumerate(zip(got, want)):
+            assert torch.equal(g_, e_), f"replay {replay}: output {k} differs from the eager call"
