@@ -35,6 +35,7 @@ PUBLIC = {
     "lorafusion/ops/triton_ops/dequantize_nf4.py": ("lorafusion_amd.ops.triton_ops.dequantize_nf4", ["dequantize_nf4_triton"]),
     "lorafusion/ops/triton_ops/config.py": ("lorafusion_amd.ops.triton_ops.config", ["get_lora_kernel_config"]),
     "lorafusion/patch/patch_lora.py": ("lorafusion_amd.patch.patch_lora", ["lora_forward", "apply_lora"]),
+    "lorafusion/utils/module.py": ("lorafusion_amd.utils.module", ["apply_liger_kernel"]),
 }
 
 

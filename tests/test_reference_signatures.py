@@ -22,7 +22,10 @@ with open(os.path.join(HERE, "golden", "reference_signatures.json")) as f:
 
 
 def _default_value(src: str):
-    return eval(src, {"torch": torch})  # noqa: S307 - literals and torch dtypes typed into the fixture
+    from lorafusion_amd.utils.module import LigerKernelLevel
+
+    # literals, torch dtypes and the level enum typed into the fixture
+    return eval(src, {"torch": torch, "LigerKernelLevel": LigerKernelLevel})  # noqa: S307
 
 
 @pytest.mark.parametrize("ref", SIGS, ids=[f"{s['module'].rsplit('.', 1)[1]}.{s['name']}" for s in SIGS])
