@@ -1,8 +1,11 @@
 """RMSNorm and SiLU-multiply HIP kernels against the oracle (GPU), through the C ABI and the autograd layer.
 
-Tolerances.  Forward outputs are compared with the oracle that rounds where the algorithm rounds: at most one
-16-bit spacing apart (the kernel's fp32 ``rstd`` / sigmoid may differ from the CPU's in the last place, which moves a
-value across a rounding boundary now and then), and with the exact fp64 value: at most 1.51 spacings (two roundings).
+Tolerances.  Forward outputs are two roundings of an exact value: the first is at most half a spacing of the
+intermediate, i.e. at most one spacing of the result in relative terms, the second half a spacing more -- at most 1.51
+spacings from the fp64 value, which is asserted.  Against the oracle that rounds where the algorithm rounds the outputs
+are equal except where the kernel's fp32 ``rstd`` / sigmoid differs from the CPU's in the last place and the
+intermediate rounds to the neighbouring value (under 0.2 % of the elements, asserted): one spacing of the intermediate
+is at most two of the result, and each side then rounds once more -- at most 3 spacings apart.
 Gradients are compared with the fp64 closed forms: |err| <= 1e-2 |e| + 1e-2 rms(e), the bar of the LoRA kernels, and
 those of SiLU-multiply, single roundings of fp32 values, to 0.51 spacings (plus the fp32 error where silu' cancels).
 """
@@ -87,7 +90,7 @@ def test_rmsnorm_forward_backward(shape, dtype):
     yo, rstdo = R.rms_norm_fwd(x, w, eps)
     ye, rstde = R.rms_norm_fwd_exact(x, w, eps)
     assert torch.allclose(rstd.cpu().double(), rstde, rtol=2e-6, atol=0)
-    assert R.ulp16_err(y.cpu(), yo.double()) <= 2.0 and float((y.cpu() != yo).float().mean()) < 2e-3
+    assert R.ulp16_err(y.cpu(), yo.double()) <= 3.0 and float((y.cpu() != yo).float().mean()) < 2e-3
     assert R.ulp16_err(y.cpu(), ye) <= 1.51
     dx, dw = _rms_bwd_abi(dy.cuda(), x.cuda(), w.cuda(), rstd)
     torch.cuda.synchronize()
@@ -113,7 +116,7 @@ def test_rmsnorm_layer_size_and_scale_invariance():
     y, rstd = _rms_fwd_abi(xd, wd, 1e-6)
     rows = torch.arange(0, M, 397)
     yo, _ = R.rms_norm_fwd(x[rows], w, 1e-6)
-    assert R.ulp16_err(y[rows.cuda()].cpu(), yo.double()) <= 2.0
+    assert R.ulp16_err(y[rows.cuda()].cpu(), yo.double()) <= 3.0
     dx, dw = _rms_bwd_abi(dyd, xd, wd, rstd)
     dxe, _ = R.rms_norm_bwd_exact(dy[rows], x[rows], w, 1e-6)
     _close(dx[rows.cuda()], dxe, "dx")
@@ -152,7 +155,7 @@ def test_silu_mul_forward_backward(shape, dtype, merged):
     c = _silu_fwd_abi(ad, bd, I)
     torch.cuda.synchronize()
     co = R.silu_mul_fwd(a, b)
-    assert R.ulp16_err(c.cpu(), co.double()) <= 2.0 and float((c.cpu() != co).float().mean()) < 2e-3
+    assert R.ulp16_err(c.cpu(), co.double()) <= 3.0 and float((c.cpu() != co).float().mean()) < 2e-3
     assert R.ulp16_err(c.cpu(), R.silu_mul_fwd_exact(a, b)) <= 1.51
     dg = torch.empty((M, 2 * I), dtype=dtype, device="cuda")
     da, db = (dg[:, :I], dg[:, I:]) if merged else (torch.empty_like(ad), torch.empty_like(bd))
@@ -187,7 +190,7 @@ def test_silu_mul_layer_size_is_linear_in_up():
     c = _silu_fwd_abi(gu[:, :I], gu[:, I:], I)
     rows = torch.arange(0, M, 1031, device="cuda")
     co = R.silu_mul_fwd(gu[rows, :I].cpu(), gu[rows, I:].cpu())
-    assert R.ulp16_err(c[rows].cpu(), co.double()) <= 2.0
+    assert R.ulp16_err(c[rows].cpu(), co.double()) <= 3.0
     gu2 = gu.clone()
     gu2[:, I:] *= 2
     c2 = _silu_fwd_abi(gu2[:, :I], gu2[:, I:], I)
@@ -215,7 +218,7 @@ def test_autograd_layer_and_hf_patch():
     w = norm.weight.detach().cpu()
     yo, _ = R.rms_norm_fwd(x.reshape(M, H), w, 1e-5)
     dxe, dwe = R.rms_norm_bwd_exact(dy.reshape(M, H), x.reshape(M, H), w, 1e-5)
-    assert y.shape == x.shape and R.ulp16_err(y.reshape(M, H).cpu(), yo.double()) <= 2.0
+    assert y.shape == x.shape and R.ulp16_err(y.reshape(M, H).cpu(), yo.double()) <= 3.0
     _close(xd.grad.reshape(M, H), dxe, "dx")
     _close(norm.weight.grad, dwe, "dw")
     # frozen weight: no dw is computed, dx is the same
@@ -259,7 +262,7 @@ def test_autograd_layer_and_hf_patch():
     # and the activation inside is the oracle's
     gate, up = mlp.gate_proj(hn(xm)), mlp.up_proj(hn(xm))
     co = R.silu_mul_fwd(gate.detach().cpu(), up.detach().cpu())
-    assert R.ulp16_err(norm_act.silu_mul(gate, up).detach().cpu(), co.double()) <= 2.0
+    assert R.ulp16_err(norm_act.silu_mul(gate, up).detach().cpu(), co.double()) <= 3.0
 
 
 def test_rejected_shapes_enqueue_nothing():

@@ -71,7 +71,7 @@ def test_prologue_equals_activation_then_xa_single(rank, mode, dtype):
     assert torch.equal(s, s_ref)
     # and against the oracle: S = drop(c) A^T (1/(1-p) applied), c the rounded activation
     co = R.silu_mul_fwd(gu[:, :K].cpu(), gu[:, K:].cpu())
-    assert R.ulp16_err(x.cpu(), co.double()) <= 2.0
+    assert R.ulp16_err(x.cpu(), co.double()) <= 3.0
     _, s_exp = lora_ref.linear_lora_fwd_fp32(x.cpu(), torch.zeros(8, K), a.cpu(), torch.zeros(8, rank), 1.0,
                                              mask.cpu() if mask is not None else None, use_p)
     _close(s[:, :rank], s_exp, "S")

@@ -106,7 +106,7 @@ def test_silu_mul_forward_is_hf_mlp_activation(dtype):
     else:
         # torch's half silu divides (x / (1 + exp(-x))) where the algorithm multiplies by the sigmoid: the fp32
         # values differ in the last place and a few of them round to the neighbouring half
-        assert float((got != exp).float().mean()) < 5e-3 and R.ulp16_err(got, exp.double()) <= 2.0  # 2: a step across a power of two
+        assert float((got != exp).float().mean()) < 5e-3 and R.ulp16_err(got, exp.double()) <= 3.0  # a neighbouring intermediate: two spacings of the result, and a rounding each
     exact = R.silu_mul_fwd_exact(a, b)
     assert torch.allclose(exact, torch.nn.functional.silu(a.double()) * b.double(), rtol=1e-14, atol=1e-300)
     assert R.ulp16_err(got, exact) <= 1.51
