@@ -281,3 +281,32 @@ def test_rejected_shapes_enqueue_nothing():
     with pytest.raises(ValueError, match="dtype"):
         norm_act.rms_norm(x[:, :64].contiguous(), w[:64].float())
     assert ctypes.sizeof(ctypes.c_void_p) == 8
+
+
+def test_empty_three_dimensional_and_strided_inputs():
+    from lorafusion_amd.ops import norm_act
+
+    w = torch.ones(64, dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    # no rows: nothing is launched, shapes and gradients are still right
+    x0 = torch.empty(0, 64, dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    y0 = norm_act.rms_norm(x0, w, 1e-6)
+    y0.sum().backward()
+    assert y0.shape == (0, 64) and x0.grad.shape == (0, 64) and torch.count_nonzero(w.grad) == 0
+    g0 = torch.empty(2, 0, 128, dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    c0 = norm_act.silu_mul_merged(g0)
+    c0.sum().backward()
+    assert c0.shape == (2, 0, 64) and g0.grad.shape == g0.shape
+    # [batch, seq, hidden] with a transposed (non-contiguous) batch/seq layout, and column slices as operands
+    x = _rand((5, 7, 64), torch.bfloat16, 40, scale=2.0)
+    xt = x.cuda().transpose(0, 1)                     # [7, 5, 64], strides (64, 448, 1)
+    y = norm_act.rms_norm(xt, w.detach(), 1e-5)
+    yo, _ = R.rms_norm_fwd(x.transpose(0, 1).reshape(35, 64), torch.ones(64, dtype=torch.bfloat16), 1e-5)
+    assert y.shape == (7, 5, 64) and R.ulp16_err(y.reshape(35, 64).cpu(), yo.double()) <= 3.0
+    big = _rand((33, 400), torch.bfloat16, 41, scale=2.0).cuda()
+    a, b = big[:, 8:136], big[:, 200:328]               # 128 columns each, row stride 400, 16-byte aligned starts
+    c = norm_act.silu_mul(a, b)
+    co = R.silu_mul_fwd(a.cpu(), b.cpu())
+    assert R.ulp16_err(c.cpu(), co.double()) <= 3.0
+    a2, b2 = big[:, 4:132], big[:, 204:332]             # starts that are not 16-byte aligned: copied, same result rule
+    c2 = norm_act.silu_mul(a2, b2)
+    assert R.ulp16_err(c2.cpu(), R.silu_mul_fwd(a2.cpu(), b2.cpu()).double()) <= 3.0
