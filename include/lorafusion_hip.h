@@ -82,6 +82,10 @@ typedef struct lf_routing {
 
 int lf_version(void);
 const char* lf_strerror(int code);
+/* Bytes of `workspace` the entry point(s) behind `op` need for this shape.  0 also for a shape or routing
+ * the entry point itself would refuse (M <= 0, R not a multiple of 16 in 16..128, a tiled dimension
+ * -- N for DYS_DYB / BWD / NF4_*, K for XA / DA / FWD / BWD / NF4_* -- that is not a positive multiple
+ * of 128, bad routing): the size query never fails harder than the call. */
 size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* routing);
 
 /* S = drop(X) A^T.  Stands in for seeded_dropout + `masked_scaled_x @ lora_a.T`

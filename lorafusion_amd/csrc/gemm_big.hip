@@ -116,8 +116,10 @@ __device__ __forceinline__ void sfor(F&& f) {
 #ifdef LF_BIG_TIMING
 __device__ unsigned long long lf_big_timing[16];  // cycles: seed, k loop, epilogue, wall (100 MHz), tiles
 #define LF_TICK(var) const long long var = __builtin_readcyclecounter()
+#define LF_MT(var) const unsigned long long var = __builtin_amdgcn_s_memtime()
 #else
 #define LF_TICK(var)
+#define LF_MT(var)
 #endif
 
 // LORA = false: the instance for calls without a LoRA term (the seed code is compiled out, which also keeps that
@@ -633,6 +635,10 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     // loads that nothing consumes keep the step body uniform).  Gap schedule of a step (one MFMA = one gap of three
     // issue slots): sub-step 0: a fragment read every third gap, the scalar offset of one load of the coming stage
     // every fourth; sub-step 1: a fragment read every third gap, M0 in gap 4i, load i in gap 4i+1.
+#ifdef LF_BIG_TIMING
+    unsigned tm_vm = 0, tm_bar = 0, tm_lg = 0, tm_s0 = 0, tm_s1 = 0;
+    unsigned long long mt_prev = __builtin_amdgcn_s_memtime();
+#endif
     auto k_step = [&](int s, const LoadSrc& ld, int lk) __attribute__((always_inline)) {
       const int cs = (par + s) & 1;
       const uint32_t cur = cs * STAGE, nxt = STAGE - cur;
@@ -647,8 +653,17 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         mfma_one(0, m);
         __builtin_amdgcn_sched_barrier(0);
       });
+      LF_MT(mt_a);
+#ifndef LF_ABL_NOVMWAIT
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads of step s+1 (issued a sub-step ago) have landed
+#endif
+      LF_MT(mt_b);
+#ifndef LF_ABL_NOBAR
       barrier();
+#else
+      __builtin_amdgcn_sched_barrier(0); lgkm0(); __builtin_amdgcn_sched_barrier(0);
+#endif
+      LF_MT(mt_c);
       sfor<64>([&](auto MM) {
         constexpr int m = MM.value;
         if constexpr (m % RDS == 0 && m / RDS < 16) read_one(S0{}, S0{}, nxt, integral_constant<int, (m / RDS + 8) & 15>{});
@@ -661,8 +676,14 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         __builtin_amdgcn_sched_barrier(0);
       });
       __builtin_amdgcn_sched_barrier(0);
+      LF_MT(mt_d);
       lgkm0();
       __builtin_amdgcn_sched_barrier(0);
+      LF_MT(mt_e);
+#ifdef LF_BIG_TIMING
+      tm_vm += (unsigned)(mt_b - mt_a); tm_bar += (unsigned)(mt_c - mt_b); tm_lg += (unsigned)(mt_e - mt_d);
+      tm_s0 += (unsigned)(mt_a - mt_prev); tm_s1 += (unsigned)(mt_d - mt_c); mt_prev = mt_e;
+#endif
     };
     {
       int s = 0;
@@ -727,6 +748,11 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       atomicAdd(&lf_big_timing[2], (unsigned long long)(tk3 - tk2));
       atomicAdd(&lf_big_timing[3], (unsigned long long)(wall_clock64() - tw0));
       atomicAdd(&lf_big_timing[4], 1ull);
+      atomicAdd(&lf_big_timing[7], (unsigned long long)tm_vm);
+      atomicAdd(&lf_big_timing[8], (unsigned long long)tm_bar);
+      atomicAdd(&lf_big_timing[9], (unsigned long long)tm_lg);
+      atomicAdd(&lf_big_timing[10], (unsigned long long)tm_s0);
+      atomicAdd(&lf_big_timing[11], (unsigned long long)tm_s1);
     }
 #endif
     tile = nxt_tile;

@@ -73,6 +73,10 @@ int make_seg(const lf_routing* r, int M, const void* const* ptrs, void* const* o
 
 bool bad_dtype(int d) { return d != LF_BF16 && d != LF_F16; }
 
+// What the rank-r passes and their planners assume of a dimension they tile (N of dys_dyb, K of xa / da) and of R.
+bool bad_tiled_dim(int v) { return v <= 0 || v % 128 != 0; }
+bool bad_rank_cols(int R) { return R <= 0 || R % 16 != 0 || R > LF_MAX_RANK; }
+
 }  // namespace
 
 extern "C" {
@@ -96,6 +100,12 @@ size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* 
   LfSegTable t;
   const void* dummy_ptrs[LF_MAX_SEG] = {};
   if (make_seg(routing, M, dummy_ptrs, nullptr, t) != LF_OK) return 0;
+  // shapes the launch itself would refuse need no workspace; the planners are only asked about shapes they tile
+  if (M <= 0 || bad_rank_cols(R)) return 0;
+  const bool reads_n = op == LF_OP_DYS_DYB || op == LF_OP_BWD || op == LF_OP_NF4_BWD || op == LF_OP_NF4_FWD;
+  const bool reads_k = op == LF_OP_XA || op == LF_OP_DA || op == LF_OP_FWD || op == LF_OP_BWD || op == LF_OP_NF4_FWD ||
+                       op == LF_OP_NF4_BWD;
+  if ((reads_n && bad_tiled_dim(N)) || (reads_k && bad_tiled_dim(K))) return 0;
   switch (op) {
     case LF_OP_XA: return align256(lf_xa_workspace(M, K, R, t));
     case LF_OP_DYS_DYB: return align256(lf_dys_dyb_workspace(M, N, R, t));
@@ -245,10 +255,13 @@ int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8
                        const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
                        void* const* db_ptrs, void* dS_out, int M, int N, int K, int R, const lf_routing* routing,
                        int dtype, void* stream) {
+  if (bad_dtype(dtype) || !dY || !X || !S || !b_ptrs || !da_ptrs || !db_ptrs || !dS_out) return LF_EINVAL;
+  if (dX && (!W || !a_ptrs)) return LF_EINVAL;
+  if (M <= 0 || N <= 0 || K <= 0 || R <= 0) return LF_EINVAL;
+  if (bad_tiled_dim(N) || bad_tiled_dim(K) || bad_rank_cols(R)) return LF_ESHAPE;
   LfSegTable t;
   int rc = make_seg(routing, M, nullptr, nullptr, t);
   if (rc != LF_OK) return rc;
-  if (M <= 0 || N <= 0 || K <= 0 || R <= 0) return LF_EINVAL;
   const size_t a = lf_dys_dyb_workspace(M, N, R, t), b = lf_da_workspace(M, K, R, t);
   const size_t need = align256(a > b ? a : b);
   if (need > (size_t)LF_STATIC_SCRATCH_BYTES) return LF_ESTATIC;

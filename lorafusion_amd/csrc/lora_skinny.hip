@@ -1236,6 +1236,7 @@ static DysRingPlan dysr_plan(int M, int N, int R, const LfSegTable& seg) {
   const int slots = lds_slots(dysr_smem(rt));
   const double tile_bytes = TILE_BYTES + 64.0 * R * 2;
   DysRingPlan best{1, 1, 1};
+  if (T < 2) return best;   // fewer than two column tiles: nothing to split (and no division by a zero slice count)
   double best_cost = 1e300;
   for (int t = dysr_tpw(rt); t >= 2; t--) {   // tiles of the longest slice -> fewest slices that reach it
     const int nsl = (T + t - 1) / t;
@@ -1423,6 +1424,7 @@ static DaPlan da_plan(int M, int K, int R, bool masked, const LfSegTable& seg) {
   const int slots = lds_slots(da_ring_smem(rt, masked));
   const double tile_bytes = TILE_BYTES + (masked ? ROWS * 64 : 0);
   DaPlan best{1, 1, 1};
+  if (T < 2) return best;   // as in dysr_plan
   double best_cost = 1e300;
   for (int t = da_tpw(rt); t >= 2; t--) {   // tiles of the longest slice -> fewest slices that reach it
     const int nsl = (T + t - 1) / t;

@@ -83,10 +83,11 @@ rmsnorm_fwd_kernel(const lf_u32x4* __restrict__ x, const lf_u32x4* __restrict__ 
 // Widest rows with dw: the weight vector is read from LDS instead (registers go to the row, its gradient and the sums).
 constexpr bool bwd_w_in_regs(int ch, bool dw) { return !(dw && ch >= 12); }
 
-// dX may alias dY: a wave holds the whole row of dY in registers before it writes that row of dX.
+// dX may alias dY: a wave holds the whole row of dY in registers before it writes that row of dX (neither pointer
+// is restrict-qualified, so the compiler may not move a load of dY below a store to dX either).
 template <typename T, int CH, bool DW, bool FULL>
 __global__ void __launch_bounds__(NORM_THREADS)
-rmsnorm_bwd_kernel(const lf_u32x4* __restrict__ dy, const lf_u32x4* __restrict__ x, const lf_u32x4* __restrict__ w,
+rmsnorm_bwd_kernel(const lf_u32x4* dy, const lf_u32x4* __restrict__ x, const lf_u32x4* __restrict__ w,
                    const float* __restrict__ rstd, lf_u32x4* dx, float* __restrict__ dw_partial /* [gridDim.x, H] */,
                    int M, int hc, float h) {
   // LDS: one row of fp32 partial sums (DW), then the weight vector where it is not kept in registers

@@ -37,17 +37,31 @@ _MODELS = {
 _saved: dict[tuple[type, str], object] = {}
 
 
+def _original_forward(module):
+    """HF's own forward of the patched class `module` belongs to -- found along the MRO, so that a subclass of a
+    patched class (which inherits the patched forward but is no key of `_saved` itself) falls back correctly."""
+    for cls in type(module).__mro__:
+        fn = _saved.get((cls, "forward"))
+        if fn is not None:
+            return fn
+    raise RuntimeError(f"{type(module).__name__}: no saved forward (apply_liger_kernel did not patch this class)")
+
+
 def _rms_norm_forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
-    if not hidden_states.is_cuda or hidden_states.dtype != self.weight.dtype or hidden_states.dtype == torch.float32:
-        # fp32 activations or mixed dtypes: HF's own arithmetic (the kernels are 16-bit)
-        return _saved[(type(self), "forward")](self, hidden_states)
+    h = hidden_states.shape[-1]
+    if (not hidden_states.is_cuda or hidden_states.dtype != self.weight.dtype or hidden_states.dtype == torch.float32
+            or h % 8 != 0 or h > 8192):
+        # fp32 activations, mixed dtypes, or a width the kernel does not take (rows of 16-byte pieces, at most 8192
+        # wide): HF's own arithmetic
+        return _original_forward(self)(self, hidden_states)
     return rms_norm(hidden_states, self.weight, self.variance_epsilon)
 
 
 def _mlp_forward(self, x: torch.Tensor) -> torch.Tensor:
     act = getattr(getattr(self, "config", None), "hidden_act", "silu")
-    if act not in ("silu", "swish") or not x.is_cuda or x.dtype == torch.float32:
-        return _saved[(type(self), "forward")](self, x)
+    inter = getattr(getattr(self, "gate_proj", None), "out_features", 0)
+    if act not in ("silu", "swish") or not x.is_cuda or x.dtype == torch.float32 or inter % 8 != 0:
+        return _original_forward(self)(self, x)
     return swiglu_mlp_forward(self, x)
 
 

@@ -75,6 +75,38 @@ def test_argument_validation_without_gpu():
     assert lib.lf_lora_xa(one, None, ptrs, one, one, 1 << 20, 128, 128, 16, bad2, 0, None) == -5
 
 
+def test_size_query_and_static_backward_refuse_untiled_shapes():
+    """A tiled dimension below the tile (or R the passes do not take) must come back as a code, not as a host crash:
+    the planners divide by the number of 64-column tiles."""
+    from lorafusion_amd import _lib
+
+    lib = _lib.lib()
+    r = _lib.single_routing(16, 1.0, 0.0)
+    for bad in (0, 32, 64, 192):
+        assert lib.lf_workspace_bytes(_lib.LF_OP_BWD, 256, bad, 256, 16, r) == 0
+        assert lib.lf_workspace_bytes(_lib.LF_OP_BWD, 256, 256, bad, 16, r) == 0
+        assert lib.lf_workspace_bytes(_lib.LF_OP_DYS_DYB, 256, bad, 0, 16, r) == 0
+        assert lib.lf_workspace_bytes(_lib.LF_OP_DA, 256, 0, bad, 16, r) == 0
+        assert lib.lf_workspace_bytes(_lib.LF_OP_NF4_BWD, 256, bad, 256, 16, r) == 0
+    # the dimension an op does not tile may be anything
+    assert lib.lf_workspace_bytes(_lib.LF_OP_DYS_DYB, 256, 256, 0, 16, r) > 0
+    assert lib.lf_workspace_bytes(_lib.LF_OP_DA, 256, 0, 256, 16, r) > 0
+    for bad_r in (0, 8, 24, 144):
+        assert lib.lf_workspace_bytes(_lib.LF_OP_BWD, 256, 256, 256, bad_r, r) == 0
+    assert lib.lf_workspace_bytes(_lib.LF_OP_BWD, 0, 256, 256, 16, r) == 0
+    one = ctypes.c_void_p(256)
+    ptrs = (ctypes.c_void_p * 1)(256)
+    call = lambda M, N, K, R, dt=0, dy=one: lib.lf_lora_bwd_static(dy, one, one, None, one, ptrs, ptrs, one, ptrs, ptrs, one, M, N, K, R, r, dt, None)
+    for bad in (32, 64, 192):
+        assert call(256, bad, 256, 16) == _lib.LF_ESHAPE
+        assert call(256, 256, bad, 16) == _lib.LF_ESHAPE
+    assert call(256, 256, 256, 24) == _lib.LF_ESHAPE
+    assert call(256, 256, 256, 144) == _lib.LF_ESHAPE
+    assert call(256, 0, 256, 16) == _lib.LF_EINVAL
+    assert call(256, 256, 256, 16, dt=7) == _lib.LF_EINVAL       # dtype and pointers are looked at first
+    assert call(256, 256, 256, 16, dy=None) == _lib.LF_EINVAL
+
+
 def test_python_layer_refuses_cpu_tensors():
     from lorafusion_amd.ops.lora_v1 import fused_linear_lora
     from lorafusion_amd.ops.nf4 import QuantState, dequantize_nf4_triton

@@ -176,6 +176,20 @@ def test_ops_refuse_cpu_tensors_and_bad_levels():
     n = ml.LlamaRMSNorm(64)
     x = torch.randn(3, 64)
     patched = n(x)
+
+    # a subclass inherits the patched forward; its fallback is found along the MRO
+    class MyNorm(ml.LlamaRMSNorm):
+        pass
+
+    class MyMLP(ml.LlamaMLP):
+        pass
+
+    sub = MyNorm(64)
+    sub_patched = sub(x)
+    cfg = ml.LlamaConfig(hidden_size=64, intermediate_size=96, hidden_act="silu")
+    mlp = MyMLP(cfg)
+    mlp_patched = mlp(x)
     restore_liger_kernel()
     assert (ml.LlamaRMSNorm.forward, ml.LlamaMLP.forward) == before
     assert torch.equal(patched, n(x))
+    assert torch.equal(sub_patched, sub(x)) and torch.equal(mlp_patched, mlp(x))

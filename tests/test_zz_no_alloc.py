@@ -109,3 +109,10 @@ def test_static_scratch_rejects_oversized_call():
     assert b"static" in lib.lf_strerror(rc)
     torch.cuda.synchronize()
     assert float(t.float().abs().sum()) == 0.0
+    # shapes the rank-r passes do not tile are refused before anything is planned or launched
+    for n, k, r in ((64, 256, 16), (256, 32, 16), (256, 256, 24)):
+        rc = lib.lf_lora_bwd_static(L.ptr(t), L.ptr(t), L.ptr(t), None, L.ptr(t), arr, arr, L.ptr(t), arr, arr, L.ptr(t),
+                                    256, n, k, r, L.single_routing(16, 1.0, 0.0), L.LF_BF16, L.stream_of(t))
+        assert rc == L.LF_ESHAPE, (n, k, r, rc)
+    torch.cuda.synchronize()
+    assert float(t.float().abs().sum()) == 0.0
