@@ -25,6 +25,18 @@
  * (non-zero = keep), R = max rank rounded up to 16.  Wherever an entry point takes a keep-mask,
  * mask == NULL means "no dropout" for the whole call: p of the routing is then ignored and
  * nothing is rescaled by 1/(1-p).
+ *
+ * Keep-mask formats.  Every keep-mask argument (read or written) comes in one of two formats, chosen
+ * per call by OR-ing LF_MASK_BITS into `dtype`:
+ *  - bytes (default): uint8 [M,K], one byte per element, non-zero = keep -- the reference's bool
+ *    tensor (lorafusion/ops/triton_ops/dropout.py:79, read back by
+ *    fused_lora_dyw_dsa.py:144-153);
+ *  - bits (dtype | LF_MASK_BITS): uint8 [M,K/8], element k of a row = bit (k & 7) of byte (k >> 3)
+ *    of that row, 1 = keep; rows K/8 bytes apart, base 16-byte aligned.  An eighth of the traffic in
+ *    every kernel that touches the mask; the format the Python layer uses for masks the library
+ *    draws itself.  lf_mask_pack / lf_mask_unpack convert.  The large-shape GEMM kernel reads
+ *    bits only: a dX call with a byte mask (or with more than 32 rank columns) runs on the older
+ *    eight-wave tile, a few per cent slower.
  */
 #ifndef LORAFUSION_HIP_H
 #define LORAFUSION_HIP_H
@@ -46,6 +58,7 @@ extern "C" {
 
 #define LF_BF16 0
 #define LF_F16 1
+#define LF_MASK_BITS 0x100 /* OR into dtype: the call's keep-masks are bit-packed (see above) */
 
 #define LF_MAX_SEG 32
 
@@ -242,6 +255,13 @@ int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const
  * the 128 output bits, low half of a word first), kept when draw >= floor(p * 2^16): a function of
  * (seed, element index) only. */
 int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream);
+
+/* Keep-mask format conversion: bytes [M,K] (non-zero = keep) -> bits [M,K/8] and back (to 0/1
+ * bytes); K % 128 == 0, both buffers 16-byte aligned.  The reference has one format only (its bool
+ * tensor, lorafusion/ops/triton_ops/dropout.py:79); these exist so that a caller holding such a
+ * tensor can use the bit-packed entry points, and read back a mask the library drew. */
+int lf_mask_pack(const uint8_t* mask_bytes, uint8_t* mask_bits, int M, int K, void* stream);
+int lf_mask_unpack(const uint8_t* mask_bits, uint8_t* mask_bytes, int M, int K, void* stream);
 
 /* RMSNorm and SiLU-multiply: the elementwise steps either side of the LoRA linears of a decoder layer.  The
  * reference takes them from the liger-kernel package (apply_liger_kernel, lorafusion/utils/module.py:41-71;

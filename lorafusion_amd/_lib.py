@@ -15,6 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liblorafusion_hip.so")
 
 LF_BF16, LF_F16 = 0, 1
+LF_MASK_BITS = 0x100  # OR into dtype: the call's keep-masks are bit-packed ([M, K/8] bytes, element k = bit k & 7 of byte k >> 3)
 LF_MAX_SEG = 32
 LF_OP_XA, LF_OP_DYS_DYB, LF_OP_DA, LF_OP_FWD, LF_OP_BWD, LF_OP_NF4_FWD, LF_OP_NF4_BWD = range(7)
 LF_OK, LF_EINVAL, LF_ESHAPE, LF_EWORKSPACE, LF_ELAUNCH, LF_ELIMIT, LF_ESTATIC = 0, -1, -2, -3, -4, -5, -6
@@ -25,7 +26,7 @@ EXPORTS = (
     "lf_lora_da", "lf_lora_dyw_dsa", "lf_lora_fwd", "lf_lora_bwd", "lf_gemm", "lf_nf4_dequant", "lf_dropout_mask",
     "lf_lora_xa_seeded", "lf_lora_fwd_seeded", "lf_nf4_lora_fwd", "lf_nf4_lora_bwd", "lf_lora_bwd_static", "lf_set_tile_cfg", "lf_gemm_plan",
     "lf_rmsnorm_fwd", "lf_rmsnorm_bwd_workspace", "lf_rmsnorm_bwd", "lf_silu_mul_fwd", "lf_silu_mul_bwd",
-    "lf_lora_xa_silu_mul", "lf_swiglu_lora_fwd",
+    "lf_lora_xa_silu_mul", "lf_swiglu_lora_fwd", "lf_mask_pack", "lf_mask_unpack",
 )
 
 
@@ -112,6 +113,8 @@ def lib() -> ctypes.CDLL:
     l.lf_silu_mul_bwd.argtypes = [vp, vp, vp, vp, vp, i, i, i64, i64, i64, i64, i64, i, vp]
     l.lf_lora_xa_silu_mul.argtypes = [vp, vp, i64, vp, vp, vp, ctypes.c_uint64, vp, vp, i, i, i, rp, i, vp]
     l.lf_swiglu_lora_fwd.argtypes = [vp, vp, i64, vp, vp, vp, vp, vp, ctypes.c_uint64, vp, vp, vp, vp, i, i, i, i, rp, i, vp]
+    l.lf_mask_pack.argtypes = [vp, vp, i, i, vp]
+    l.lf_mask_unpack.argtypes = [vp, vp, i, i, vp]
     for name in EXPORTS:
         if name not in ("lf_strerror", "lf_workspace_bytes", "lf_rmsnorm_bwd_workspace"):
             getattr(l, name).restype = i

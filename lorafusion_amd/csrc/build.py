@@ -21,6 +21,20 @@ FLAGS = [
 ]
 
 
+# sources whose kernels issue memory instructions from inline assembly: their generated code is checked for the
+# hazards the compiler does not resolve there (asm_lint.py)
+LINTED = ["gemm_big.hip", "gemm_lora.hip", "lora_skinny.hip"]
+
+
+def _assembly(src: str) -> str:
+    out = os.path.join(HERE, "build", src.replace(".hip", ".s"))
+    cmd = ["hipcc", *FLAGS, "-S", "--cuda-device-only", os.path.join(HERE, src), "-o", out]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc -S failed on {src}:\n{res.stderr}")
+    return out
+
+
 def _compile(src: str) -> str:
     obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
     cmd = ["hipcc", *FLAGS, "-c", os.path.join(HERE, src), "-o", obj]
@@ -35,8 +49,14 @@ def _compile(src: str) -> str:
 
 def build(verbose: bool = True) -> str:
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    from lorafusion_amd.csrc.asm_lint import lint
+
     with ThreadPoolExecutor(max_workers=6) as ex:
+        asm = [ex.submit(_assembly, s) for s in LINTED]
         objs = list(ex.map(_compile, SOURCES))
+        hazards = [v for a in asm for v in lint(a.result())]
+    if hazards:
+        raise RuntimeError("hazards in generated code that inline assembly hides from the compiler:\n" + "\n".join(hazards))
     res = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-z,defs", "-o", LIB, *objs],
                          capture_output=True, text=True)
     if res.returncode != 0:

@@ -32,7 +32,48 @@ dropout_mask_kernel(uint8_t* __restrict__ mask, int64_t n16, int K, uint32_t thr
   *(lf_u32x4*)(mask + e0) = o;
 }
 
+// Keep-mask formats: one byte per element (the reference's bool tensor, lorafusion/ops/triton_ops/dropout.py:79) and
+// one bit per element (element k of a row = bit k & 7 of byte k >> 3).  Each thread converts 16 elements.
+__global__ void __launch_bounds__(256)
+mask_pack_kernel(const lf_u32x4* __restrict__ bytes, uint16_t* __restrict__ bits, int64_t n16) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= n16) return;
+  const lf_u32x4 v = bytes[t];
+  uint32_t o = 0;
+#pragma unroll
+  for (int d = 0; d < 4; d++) {
+    // any nonzero byte keeps: normalise to 0/1, then one multiply gathers the four bits (no carries: see lf_keep8)
+    const uint32_t w = v[d];
+    const uint32_t nz = ((w | ((w & 0x7f7f7f7fu) + 0x7f7f7f7fu)) >> 7) & 0x01010101u;
+    o |= ((nz * 0x01020408u) >> 24) << (4 * d);
+  }
+  bits[t] = (uint16_t)o;
+}
+
+__global__ void __launch_bounds__(256)
+mask_unpack_kernel(const uint16_t* __restrict__ bits, lf_u32x4* __restrict__ bytes, int64_t n16) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= n16) return;
+  const uint32_t b = bits[t];
+  lf_u32x4 o;
+#pragma unroll
+  for (int d = 0; d < 4; d++) o[d] = (((b >> (4 * d)) & 0xfu) * 0x00204081u) & 0x01010101u;
+  bytes[t] = o;
+}
+
 }  // namespace
+
+int lf_launch_mask_pack(const uint8_t* bytes, uint8_t* bits, int64_t n, hipStream_t st) {
+  const int64_t n16 = n / 16, blocks = (n16 + 255) / 256;
+  if (blocks > 0x7fffffffLL) return LF_ELIMIT;
+  return lf_launch(mask_pack_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const lf_u32x4*)bytes, (uint16_t*)bits, n16);
+}
+
+int lf_launch_mask_unpack(const uint8_t* bits, uint8_t* bytes, int64_t n, hipStream_t st) {
+  const int64_t n16 = n / 16, blocks = (n16 + 255) / 256;
+  if (blocks > 0x7fffffffLL) return LF_ELIMIT;
+  return lf_launch(mask_unpack_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t*)bits, (lf_u32x4*)bytes, n16);
+}
 
 int lf_launch_dropout_mask(uint8_t* mask, int M, int K, float p, const float* block_p, int block_size_m, uint64_t seed,
                            hipStream_t st) {

@@ -51,7 +51,9 @@ constexpr int PAIR_NN = 1024 + 32;
 template <bool NN> struct Lds {
   static constexpr int STAGE_B = NN ? 32 * PAIR_NN : BN * BK * 2;
   static constexpr int STAGE = STAGE_A + STAGE_B;
-  static constexpr int EP_OFF = 2 * STAGE, EP_WAVE = 4608, BYTES = EP_OFF + 4 * EP_WAVE;
+  // per wave behind the stages: the epilogue's band buffer (4.5 KB), before that the landing area of a tile's LoRA
+  // operands (dX product: 4 KB of A_i rows + 2 KB of keep bits)
+  static constexpr int EP_OFF = 2 * STAGE, EP_WAVE = 6144, BYTES = EP_OFF + 4 * EP_WAVE;
   static_assert(BYTES <= 160 * 1024, "two stages and the epilogue bands fit the LDS of a CU");
 };
 
@@ -74,6 +76,17 @@ template <> struct BigOp<__bf16> {
   static __device__ __forceinline__ void mfma_first(lf_f32x4& c, lf_u32x4 a, lf_u32x4 b) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
   }
+  // the LoRA term: 16 rank columns per step (two registers per operand), into the accumulators / into (d = a b) and
+  // onto (d += a b) ordinary vector registers
+  static __device__ __forceinline__ void mfma16(lf_f32x4& c, lf_u32x2 a, lf_u32x2 b) {
+    asm volatile("v_mfma_f32_16x16x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma16_v0(lf_f32x4& d, lf_u32x2 a, lf_u32x2 b) {
+    asm volatile("v_mfma_f32_16x16x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma16_v(lf_f32x4& d, lf_u32x2 a, lf_u32x2 b) {
+    asm volatile("v_mfma_f32_16x16x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
     bf2 v = {(__bf16)lo, (__bf16)hi};
@@ -90,6 +103,15 @@ template <> struct BigOp<_Float16> {
   }
   static __device__ __forceinline__ void mfma_first(lf_f32x4& c, lf_u32x4 a, lf_u32x4 b) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma16(lf_f32x4& c, lf_u32x2 a, lf_u32x2 b) {
+    asm volatile("v_mfma_f32_16x16x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma16_v0(lf_f32x4& d, lf_u32x2 a, lf_u32x2 b) {
+    asm volatile("v_mfma_f32_16x16x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma16_v(lf_f32x4& d, lf_u32x2 a, lf_u32x2 b) {
+    asm volatile("v_mfma_f32_16x16x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -116,10 +138,8 @@ __device__ __forceinline__ void sfor(F&& f) {
 #ifdef LF_BIG_TIMING
 __device__ unsigned long long lf_big_timing[16];  // cycles: seed, k loop, epilogue, wall (100 MHz), tiles
 #define LF_TICK(var) const long long var = __builtin_readcyclecounter()
-#define LF_MT(var) const unsigned long long var = __builtin_amdgcn_s_memtime()
 #else
 #define LF_TICK(var)
-#define LF_MT(var)
 #endif
 
 // LORA = false: the instance for calls without a LoRA term (the seed code is compiled out, which also keeps that
@@ -268,7 +288,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   Tile tile = tile_of(0);
   LoadSrc src = src_of(tile);
   load_stage(src, 0, 0);
-  load_stage(src, nk > 1 ? 1 : 0, 1);
+  load_stage(src, 1, 1);
 
   // Adapter of a wave's 128 rows: rank, skinny operand, multiplier, whether a keep-mask applies.  With a routing table
   // these are two dependent scalar loads (table row, then the segment's pointer), so a tile's lookup is issued while
@@ -299,16 +319,21 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     }
     return r;
   };
+  constexpr bool has_lora = LORA;   // the launcher picks the LORA instance exactly when there is a term (p.L != nullptr)
   Route route{};
-  if (LORA && p.L != nullptr) route = route_of(tile.m0 + wm * 128);
+  if (has_lora) route = route_of(tile.m0 + wm * 128);
+  const int n16 = p.R >> 4;   // chunks of 16 rank columns (one 16x16x16 MFMA step each)
 
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the first tile's two stages (later tiles: waited for before the epilogue's stores)
   int par = 0;  // LDS stage of the current tile's K step 0 (tiles follow each other through the two stages without a gap)
   for (int it = 0; it < n_my; it++) {
-    // everything below is scoped to one tile: fragments, accumulators and seed operands do not live across tiles
+    // everything below is scoped to one tile: fragments, accumulators and LoRA operands do not live across tiles
     const Tile nxt_tile = it + 1 < n_my ? tile_of(it + 1) : tile;
     const LoadSrc nxt_src = src_of(nxt_tile);
     const int m0 = tile.m0, n0 = tile.n0;
     const int wrow0 = m0 + wm * 128;
+    const Route rt = route;
+    if (has_lora) route = route_of(nxt_tile.m0 + wm * 128);  // in flight during this tile's K loop
 
     LF_TICK(tk0);
 #ifdef LF_BIG_TIMING
@@ -316,7 +341,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
 #endif
     lf_u32x4 fa[2][8], fb[2][8];
     lf_f32x4 acc[8][8];
-    uint32_t fa_off[2], fb_off[2];  // fragment addresses: set after the seed, so they are not live across it
+    uint32_t fa_off[2], fb_off[2];
     // one fragment read of sub-step KS of the stage at LDS byte offset `st`: idx < 8: A fragment idx; else B fragment idx-8
     auto read_one = [&](auto SET, auto KS, uint32_t st, auto IDX) __attribute__((always_inline)) {
       constexpr int idx = IDX.value, set = SET.value, ks = KS.value;
@@ -341,263 +366,75 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         fb[set][idx - 8] = lf_u32x4{lo[0], lo[1], hi[0], hi[1]};
       }
     };
-    auto mfma_one = [&](int set, int m) __attribute__((always_inline)) {
+    // FIRST: the first MFMA into an accumulator block of a tile takes the constant 0 as its addend and writes the
+    // block: no zeroing pass, and nothing of the previous tile has to be cleared
+    auto mfma_one = [&](int set, int m, auto FIRST) __attribute__((always_inline)) {
       const int i = m >> 3, j = m & 7;
-      BigOp<T>::mfma(acc[i][j], fb[set][j], fa[set][i]);
+      if constexpr (FIRST.value) BigOp<T>::mfma_first(acc[i][j], fb[set][j], fa[set][i]);
+      else BigOp<T>::mfma(acc[i][j], fb[set][j], fa[set][i]);
     };
 
-    // ------------------------------------------------------------ LoRA seed: acc = mult * L Rop (masked), or zero
-    auto zero_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-      for (int i = 0; i < 8; i++)
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-          acc[i][j] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
-          asm volatile("" : "+a"(acc[i][j]));  // zeroed in the accumulation registers themselves
-        }
-    };
-    if (!(LORA && p.L != nullptr)) zero_acc();
-    if (LORA && p.L != nullptr) {
+    // ------------------------------------------------------------ operands of the LoRA term
+    // The term is added at the END of a tile (masked: inside the epilogue's conversion).  Nothing of it may be
+    // requested behind the epilogue's stores: loads and stores share one counter and complete out of order with
+    // respect to each other, so a wait for such a load would be a wait for the 128 KB of output stored just before.
+    // The dX product (NN) therefore requests, during the tile's first K sub-step (the texture addresser is idle
+    // there), what it cannot fetch quickly afterwards -- the keep-mask bits of the wave's 128x128 block, which come
+    // from HBM, and the first 16 rows of A_i over the wave's columns, which the MFMA needs transposed -- as
+    // direct-to-LDS loads into the wave's own 6 KB behind the stages (the epilogue's band buffer, idle until then):
+    // no registers are involved, and the data has landed by the vmcnt(0) of the tile's second K step (K >= 128).
+    // The L fragments and the forward's B_i fragments are plain 8-byte loads issued right behind the K loop; they come
+    // from L2, and their wait coincides with the wait for the next tile's stages that precedes the first store anyway.
+    const bool sel = NN && LORA && p.mult_mode == 1 && rt.use_mask;   // keep-mask applies to this wave's rows
+    const uint32_t area = lds0 + EP_OFF + wave * EP_WAVE;               // this wave's 6 KB
+    uint32_t rfl_voff = 0, mk_voff = 0;
+    lf_u32x4 rsrcR{}, rsrcM{};
+    int rfl_s0 = 0, rfl_step = 0, mk_step = 0;
+    if constexpr (NN && LORA) {
       int sl = lane;
-      asm volatile("" : "+v"(sl));   // as in the epilogue: keep the seed's address arithmetic inside the tile loop
-      const int l16 = sl & 15, kg = sl >> 4;
-      const T* rp = route.rp;
-      const int rank = route.rank;
-      const bool use_mask = route.use_mask;
-      const float mult = route.mult;
-      const __amdgpu_buffer_rsrc_t rsrcR = __builtin_amdgcn_make_buffer_rsrc((void*)rp, 0, 0x7fffffff, 0x00020000);
-      // Everything the seed reads is requested up front -- per chunk of 32 rank columns the 8 + 8 operand fragments
-      // and, together with the last chunk's, the keep-mask bytes of the wave's 128x128 block (one dword per
-      // accumulator block and lane) -- so that a tile pays the memory latency once per chunk, not once per block row.
-      // The K loop's fragment registers are still dead here, which is where the room comes from.
-      const bool sel = p.mult_mode == 1 && use_mask;
-      const int n_chunks = (p.R + 31) / 32;
-      if (sel && n_chunks == 1) {
-        // ---- masked seed at ranks up to 32, one block row (16 rows) at a time: the product of a block row goes to
-        // ordinary vector registers (d = a b + 0), the keep-mask picks value or zero there, and the result is written
-        // into the accumulation registers -- four vector instructions per element (multiply by 1/(1-p) in fp32,
-        // compare, select, write) where zeroing, accumulating and selecting in place take six (write; read,
-        // multiply, compare, select, write).
-        const int r0 = kg * 8;
-        const bool in_r = r0 < rank, in_R = r0 < p.R;
-        lf_u32x4 rf[8], lv[8], mq[16];
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-          const int gn = n0 + wn * 128 + j * 16 + l16;
-          const int rc = in_r ? r0 : 0;
-          if constexpr (!NN) {
-            rf[j] = *(const lf_u32x4*)(rp + (int64_t)gn * rank + rc);
-          } else {
-            const uint32_t voff = (uint32_t)((rc * p.N + gn) * 2);
-            uint32_t e[8];
-#pragma unroll
-            for (int k = 0; k < 8; k++) e[k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcR, voff, k * p.N * 2, 0);
-            rf[j] = lf_u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) lv[i] = *(const lf_u32x4*)(Lp + (int64_t)(wrow0 + i * 16 + l16) * p.R + (in_R ? r0 : 0));
-        {
-          // keep-mask of the wave's 128x128 block, whole rows per instruction (lane -> row lane>>3, 16-byte chunk lane&7)
-          const uint8_t* mrow = p.mask + (int64_t)(wrow0 + (sl >> 3)) * p.ldmask + n0 + wn * 128 + (sl & 7) * 16;
-#pragma unroll
-          for (int q = 0; q < 16; q++) mq[q] = *(const lf_u32x4*)(mrow + (int64_t)q * 8 * p.ldmask);
-        }
-#pragma unroll
-        for (int j = 0; j < 8; j++)
-#pragma unroll
-          for (int d = 0; d < 4; d++) rf[j][d] = in_r ? rf[j][d] : 0u;
-#pragma unroll
-        for (int i = 0; i < 8; i++)
-#pragma unroll
-          for (int d = 0; d < 4; d++) lv[i][d] = in_R ? lv[i][d] : 0u;
-        // vector results feed inline-assembly MFMAs: wait states, with the operands as in/outs (see the other path)
-        asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
-                                 "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]));
-        // Two slabs of the wave's LDS patch turn the mask rows to the accumulator layout (rows 144 bytes apart: a slab's
-        // 64 dword reads hit 64 banks).  Block row i+1 is written and multiplied while block row i is read and selected.
-        constexpr int MPITCH = 144, SLAB = 16 * MPITCH;
-        static_assert(2 * SLAB <= EP_WAVE, "two mask slabs fit a wave's patch");
-        const uint32_t mp_lds = lds0 + EP_OFF + wave * EP_WAVE;
-        const uint32_t mp_wr = mp_lds + (sl >> 3) * MPITCH + (sl & 7) * 16;
-        const uint32_t mp_rd = mp_lds + l16 * MPITCH + kg * 4;
-        lf_f32x4 tmp[2][8];
-        auto stage_row = [&](auto I) __attribute__((always_inline)) {
-          constexpr int i = I.value;
-          asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(mp_wr), "v"(mq[2 * i]), "n"((i & 1) * SLAB) : "memory");
-          asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(mp_wr), "v"(mq[2 * i + 1]), "n"((i & 1) * SLAB + 8 * MPITCH) : "memory");
-#pragma unroll
-          for (int j = 0; j < 8; j++) BigOp<T>::mfma0(tmp[i & 1][j], rf[j], lv[i]);
-        };
-        stage_row(integral_constant<int, 0>{});
-        sfor<8>([&](auto I) {
-          constexpr int i = I.value, so = (i & 1) * SLAB;
-          lgkm0();   // the slab of block row i is written
-          uint32_t k0, k1, k2, k3, k4, k5, k6, k7;
-          // (written out: inline-assembly operands inside a generic lambda's nested lambda do not compile with this clang)
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k0) : "v"(mp_rd), "n"(so) : "memory");
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k1) : "v"(mp_rd), "n"(so + 16) : "memory");
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k2) : "v"(mp_rd), "n"(so + 32) : "memory");
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k3) : "v"(mp_rd), "n"(so + 48) : "memory");
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k4) : "v"(mp_rd), "n"(so + 64) : "memory");
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k5) : "v"(mp_rd), "n"(so + 80) : "memory");
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k6) : "v"(mp_rd), "n"(so + 96) : "memory");
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(k7) : "v"(mp_rd), "n"(so + 112) : "memory");
-          if constexpr (i + 1 < 8) stage_row(integral_constant<int, i + 1>{});
-          // The wait for the mask dwords (the two writes behind them may still be on their way) and the wait states
-          // between the MFMAs of this block row -- issued a block row ago; the nops cover the first -- and the vector
-          // instructions that read their results, in one statement that takes all of them as in/outs.
-          lf_f32x4(&tm)[8] = tmp[i & 1];
-          if constexpr (i + 1 < 8)
-            asm volatile("s_waitcnt lgkmcnt(2)\n\ts_nop 7"
-                         : "+v"(k0), "+v"(k1), "+v"(k2), "+v"(k3), "+v"(k4), "+v"(k5), "+v"(k6), "+v"(k7), "+v"(tm[0]), "+v"(tm[1]),
-                           "+v"(tm[2]), "+v"(tm[3]), "+v"(tm[4]), "+v"(tm[5]), "+v"(tm[6]), "+v"(tm[7])
-                         :: "memory");
-          else
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7"
-                         : "+v"(k0), "+v"(k1), "+v"(k2), "+v"(k3), "+v"(k4), "+v"(k5), "+v"(k6), "+v"(k7), "+v"(tm[0]), "+v"(tm[1]),
-                           "+v"(tm[2]), "+v"(tm[3]), "+v"(tm[4]), "+v"(tm[5]), "+v"(tm[6]), "+v"(tm[7])
-                         :: "memory");
-          const uint32_t mk[8] = {k0, k1, k2, k3, k4, k5, k6, k7};
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            lf_f32x4 v;
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = ((mk[j] >> (8 * e)) & 0xffu) ? tm[j][e] * mult : 0.f;   // 1/(1-p) in fp32
-            acc[i][j] = v;
-            asm volatile("" : "+a"(acc[i][j]));  // into the accumulation registers now
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      } else {
-      // one MFMA k-step covers 32 rank columns; lanes whose 8 columns lie beyond R (or the rank) read the first
-      // columns again and are zeroed by a select (branch-free)
-      auto chunk = [&](int t, auto FIRST) __attribute__((always_inline)) {
-        const int r0 = t * 32 + kg * 8;
-        const bool in_r = r0 < rank, in_R = r0 < p.R;
-        lf_u32x4 rf[8], lv[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-          const int gn = n0 + wn * 128 + j * 16 + l16;
-          const int rc = in_r ? r0 : 0;
-          if constexpr (!NN) {
-            rf[j] = *(const lf_u32x4*)(rp + (int64_t)gn * rank + rc);
-          } else {
-            // eight rows of one column of Rop [rank, N]: 16-bit buffer loads that share a per-lane offset
-            const uint32_t voff = (uint32_t)(((rc - t * 32) * p.N + gn) * 2);
-            uint32_t e[8];
-#pragma unroll
-            for (int k = 0; k < 8; k++) e[k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcR, voff, (t * 32 + k) * p.N * 2, 0);
-            rf[j] = lf_u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) lv[i] = *(const lf_u32x4*)(Lp + (int64_t)(wrow0 + i * 16 + l16) * p.R + (in_R ? r0 : 0));
-#pragma unroll
-        for (int j = 0; j < 8; j++)
-#pragma unroll
-          for (int d = 0; d < 4; d++) rf[j][d] = in_r ? rf[j][d] : 0u;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-#pragma unroll
-          for (int d = 0; d < 4; d++) lv[i][d] = in_R ? lv[i][d] : 0u;
-          if (p.mult_mode == 0 && mult != 1.f) {
-            // the forward scale goes into the 16-bit L fragment (fp32 product, one rounding; exact for powers of two)
-#pragma unroll
-            for (int d = 0; d < 4; d++)
-              lv[i][d] = BigOp<T>::pack2(BigOp<T>::to_float((uint16_t)(lv[i][d] & 0xffffu)) * mult, BigOp<T>::to_float((uint16_t)(lv[i][d] >> 16)) * mult);
-          }
-        }
-        // The MFMAs are inline assembly, which the compiler's hazard recogniser does not see: a vector ALU result
-        // (the selects and the scaling above) needs wait states before an MFMA reads it.  The nop takes the operands
-        // as in/outs, so every instruction that produces them stays in front of it and every MFMA behind.
-        asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
-                                 "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]));
-#pragma unroll
-        for (int i = 0; i < 8; i++)
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            if constexpr (FIRST.value) BigOp<T>::mfma_first(acc[i][j], rf[j], lv[i]);   // writes the accumulators: no zeroing
-            else BigOp<T>::mfma(acc[i][j], rf[j], lv[i]);
-          }
-        __builtin_amdgcn_sched_barrier(0);
-      };
-      // Keep-mask of the wave's 128x128 block: 16 KB.  A lane owns, in every 16x16 accumulator block, row l16 and four
-      // consecutive columns (one dword of mask bytes), so loading "its" dwords directly is 64 instructions that each
-      // touch 16 rows -- 16 cache lines for 256 bytes; measured 17 K cycles per tile, most of the seed.  Instead the
-      // block is read with whole rows per instruction (lane -> row lane>>3, 16-byte chunk lane&7: 8 rows x 128 bytes,
-      // 16 instructions) and each 16-row slab is turned to the accumulator layout through the wave's LDS patch (rows
-      // 144 bytes apart: the 64 dword reads of a slab then hit 64 different banks).  The loads are issued whether or
-      // not a mask applies (without one: 16 times the head of L): defined under a condition and used under another,
-      // the compiler spills the values one by one, each behind its own wait.
-      lf_u32x4 mq[16];
-      {
-        const uint8_t* mrow = sel ? p.mask + (int64_t)(wrow0 + (sl >> 3)) * p.ldmask + n0 + wn * 128 + (sl & 7) * 16 : (const uint8_t*)Lp;
-        const int64_t qstride = sel ? 8 * p.ldmask : 0;
-#pragma unroll
-        for (int q = 0; q < 16; q++) {
-#ifndef LF_ABL_NOMASKLOAD
-          mq[q] = *(const lf_u32x4*)(mrow + q * qstride);
-#else
-          mq[q] = lf_u32x4{0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u + (uint32_t)qstride};
-#endif
-        }
-      }
-      chunk(0, std::true_type{});
-      for (int t = 1; t < n_chunks; t++) chunk(t, std::false_type{});
-#ifdef LF_ABL_NOSELECT
-      if (sel && mult == 12345.f) {
-#else
-      if (sel) {
-#endif
-        mfma_fence();
-        // keep-mask select and 1/(1-p) in fp32, one block row (16-row slab) at a time
-        constexpr int MPITCH = 144;
-        const uint32_t mp_lds = lds0 + EP_OFF + wave * EP_WAVE;
-        const uint32_t mp_wr = mp_lds + (sl >> 3) * MPITCH + (sl & 7) * 16;   // + 8 rows for the slab's second load
-        const uint32_t mp_rd = mp_lds + l16 * MPITCH + kg * 4;                // + 16 per accumulator block
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-          asm volatile("ds_write_b128 %0, %1" ::"v"(mp_wr), "v"(mq[2 * i]) : "memory");
-          asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(mp_wr), "v"(mq[2 * i + 1]), "n"(8 * MPITCH) : "memory");
-          lgkm0();
-          uint32_t mk[8];
-          {
-            // (written out: inline-assembly operands inside a generic lambda do not compile with this clang)
-            uint32_t k0, k1, k2, k3, k4, k5, k6, k7;
-            asm volatile("ds_read_b32 %0, %1" : "=v"(k0) : "v"(mp_rd) : "memory");
-            asm volatile("ds_read_b32 %0, %1 offset:16" : "=v"(k1) : "v"(mp_rd) : "memory");
-            asm volatile("ds_read_b32 %0, %1 offset:32" : "=v"(k2) : "v"(mp_rd) : "memory");
-            asm volatile("ds_read_b32 %0, %1 offset:48" : "=v"(k3) : "v"(mp_rd) : "memory");
-            asm volatile("ds_read_b32 %0, %1 offset:64" : "=v"(k4) : "v"(mp_rd) : "memory");
-            asm volatile("ds_read_b32 %0, %1 offset:80" : "=v"(k5) : "v"(mp_rd) : "memory");
-            asm volatile("ds_read_b32 %0, %1 offset:96" : "=v"(k6) : "v"(mp_rd) : "memory");
-            asm volatile("ds_read_b32 %0, %1 offset:112" : "=v"(k7) : "v"(mp_rd) : "memory");
-            lgkm0();
-            // the waits are assembly too: the values are used only behind this point
-            asm volatile("" : "+v"(k0), "+v"(k1), "+v"(k2), "+v"(k3), "+v"(k4), "+v"(k5), "+v"(k6), "+v"(k7));
-            mk[0] = k0; mk[1] = k1; mk[2] = k2; mk[3] = k3; mk[4] = k4; mk[5] = k5; mk[6] = k6; mk[7] = k7;
-          }
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            // a definition right in front of the use: the copies out of the accumulation registers cannot rise above
-            // it (without it, all 256 are read up front)
-            asm volatile("" : "+a"(acc[i][j]));
-#pragma unroll
-            for (int e = 0; e < 4; e++) acc[i][j][e] = ((mk[j] >> (8 * e)) & 0xffu) ? acc[i][j][e] * mult : 0.f;
-            asm volatile("" : "+a"(acc[i][j]));  // back into the accumulation registers now, not at the next use
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      }
-      mfma_fence();
-      route = route_of(nxt_tile.m0 + wm * 128);  // in flight during this tile's K loop
+      asm volatile("" : "+v"(sl));   // lane-dependent offsets are derived inside the tile loop (not hoisted and spilled)
+      // A_i [rank, N]: load q covers rank rows 4q .. 4q+3 (lane>>4) x 128 columns (16 bytes per lane); rows beyond
+      // the adapter's rank lie beyond the buffer's end and read as zeros
+      const uint64_t rb = (uint64_t)(uintptr_t)rt.rp;
+      rsrcR = lf_u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)rb), (uint32_t)__builtin_amdgcn_readfirstlane((int)(rb >> 32)) & 0xffffu,
+                       (uint32_t)__builtin_amdgcn_readfirstlane(rt.rank * p.N * 2), 0x00020000u};
+      rfl_voff = (uint32_t)(((sl >> 4) * p.N + (sl & 15) * 8) * 2);
+      rfl_s0 = (n0 + wn * 128) * 2;
+      rfl_step = 4 * p.N * 2;
+      // keep bits: load q covers rows 64q + lane, 16 bytes (128 columns) each.  Without a mask the two loads read the
+      // head of L (an inline-assembly statement under a run-time condition does not compile inside a generic lambda)
+      const uint64_t mb = sel ? (uint64_t)(uintptr_t)(p.mask + (int64_t)wrow0 * p.ldmask + ((n0 + wn * 128) >> 3)) : (uint64_t)(uintptr_t)Lp;
+      rsrcM = lf_u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)mb), (uint32_t)__builtin_amdgcn_readfirstlane((int)(mb >> 32)) & 0xffffu, 0x7fffffffu, 0x00020000u};
+      mk_voff = sel ? (uint32_t)(sl * (int)p.ldmask) : 0u;
+      mk_step = sel ? 64 * (int)p.ldmask : 0;
     }
+    constexpr int N_LORA_LOADS = (NN && LORA) ? 6 : 0;
+    // load `q` of the list above, issued in gaps 2q (M0) and 2q+1 of the tile's first sub-step
+    auto lora_m0 = [&](auto Q) __attribute__((always_inline)) {
+      set_m0(area, integral_constant<int, Q.value * 1024>{});
+    };
+    auto lora_load = [&](auto Q) __attribute__((always_inline)) {
+      constexpr int q = Q.value;
+      // named once outside inline assembly: this clang does not capture a variable that a generic lambda uses in
+      // assembly operands only.  The nop in front of each load: its scalar operands may have been restored from a
+      // vector register lane (v_readlane) by the instruction before, and a scalar register written by the vector ALU
+      // needs five wait states before a memory instruction reads it -- a hazard the compiler resolves for its own
+      // instructions but cannot see inside inline assembly (the load would go out with the register's old value: a
+      // wild address).  The K loop's loads take their scalar operands from scalar arithmetic only.
+      const uint32_t rfl_voff_ = rfl_voff, mk_voff_ = mk_voff;
+      const lf_u32x4 rsrcR_ = rsrcR, rsrcM_ = rsrcM;
+      if constexpr (q < 4) {
+        const int so = rfl_s0 + q * rfl_step;
+        asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(rfl_voff_), "s"(rsrcR_), "s"(so) : "memory");
+      } else {
+        const int so = (q - 4) * mk_step;
+        asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(mk_voff_), "s"(rsrcM_), "s"(so) : "memory");
+      }
+    };
 
     // ------------------------------------------------------------ fragment addresses
     // A (and NT B): lane reads granule ks*4+kg of row l16 of a 16-row block; blocks are 2048 bytes apart.  Derived
-    // from an opaque copy of the lane id, every tile: four registers fewer live across the seed
+    // from an opaque copy of the lane id, every tile
     {
       int fl = lane;
       asm volatile("" : "+v"(fl));
@@ -621,9 +458,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
 
     // ------------------------------------------------------------ K loop
     LF_TICK(tk1);
-    mfma_fence();
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // both stages requested so far (and the seed operands) have landed
-    barrier();
+    barrier();   // both stages of this tile's first two K steps are in LDS (every wave has waited for its loads)
     {
       const uint32_t st = par * STAGE;
       sfor<16>([&](auto I) { read_one(S0{}, S0{}, st, integral_constant<int, (I.value + 8) & 15>{}); });
@@ -634,12 +469,12 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     // last two steps prefetch the first two steps of the next tile instead (of this tile again when none follows:
     // loads that nothing consumes keep the step body uniform).  Gap schedule of a step (one MFMA = one gap of three
     // issue slots): sub-step 0: a fragment read every third gap, the scalar offset of one load of the coming stage
-    // every fourth; sub-step 1: a fragment read every third gap, M0 in gap 4i, load i in gap 4i+1.
-#ifdef LF_BIG_TIMING
-    unsigned tm_vm = 0, tm_bar = 0, tm_lg = 0, tm_s0 = 0, tm_s1 = 0;
-    unsigned long long mt_prev = __builtin_amdgcn_s_memtime();
-#endif
-    auto k_step = [&](int s, const LoadSrc& ld, int lk) __attribute__((always_inline)) {
+    // every fourth (first step of a tile: a load of the LoRA operands in every gap that has one); sub-step 1: a
+    // fragment read every third gap, M0 in gap 4i, load i in gap 4i+1.
+    // FIRST (a tile's step 0): its MFMAs of sub-step 0 write the accumulators, and there is nothing to wait for at the
+    // barrier -- step 1's stage was waited for before the previous tile's stores; a vmcnt(0) here would wait for those
+    // stores, which by the second step's wait have long been acknowledged.
+    auto k_step = [&](int s, const LoadSrc& ld, int lk, auto FIRST) __attribute__((always_inline)) {
       const int cs = (par + s) & 1;
       const uint32_t cur = cs * STAGE, nxt = STAGE - cur;
       int ka, kb;
@@ -650,20 +485,15 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         constexpr int m = MM.value;
         if constexpr (m % RDS == 0 && m / RDS < 16) read_one(S1{}, S1{}, cur, integral_constant<int, (m / RDS + 8) & 15>{});
         if constexpr (m % 4 == 2) soff[m / 4] = (m / 4 < 8 ? ka : kb) + istr[m / 4];
-        mfma_one(0, m);
+        if constexpr (FIRST.value && m < 2 * N_LORA_LOADS) {
+          if constexpr (m % 2 == 0) lora_m0(integral_constant<int, m / 2>{});
+          else lora_load(integral_constant<int, m / 2>{});
+        }
+        mfma_one(0, m, FIRST);
         __builtin_amdgcn_sched_barrier(0);
       });
-      LF_MT(mt_a);
-#ifndef LF_ABL_NOVMWAIT
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads of step s+1 (issued a sub-step ago) have landed
-#endif
-      LF_MT(mt_b);
-#ifndef LF_ABL_NOBAR
+      if constexpr (!FIRST.value) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads of step s+1 (issued a sub-step ago) have landed
       barrier();
-#else
-      __builtin_amdgcn_sched_barrier(0); lgkm0(); __builtin_amdgcn_sched_barrier(0);
-#endif
-      LF_MT(mt_c);
       sfor<64>([&](auto MM) {
         constexpr int m = MM.value;
         if constexpr (m % RDS == 0 && m / RDS < 16) read_one(S0{}, S0{}, nxt, integral_constant<int, (m / RDS + 8) & 15>{});
@@ -672,30 +502,143 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
           else set_m0(mb, integral_constant<int, (m / LDP - 8) * M0B_STEP>{});
         }
         if constexpr (m % LDP == 1 && m / LDP < 16) issue_load(m / LDP < 8 ? ld.ra : ld.rb, m / LDP < 8 ? a_voff : b_voff, soff[m / LDP]);
-        mfma_one(1, m);
+        mfma_one(1, m, std::false_type{});
         __builtin_amdgcn_sched_barrier(0);
       });
       __builtin_amdgcn_sched_barrier(0);
-      LF_MT(mt_d);
       lgkm0();
       __builtin_amdgcn_sched_barrier(0);
-      LF_MT(mt_e);
-#ifdef LF_BIG_TIMING
-      tm_vm += (unsigned)(mt_b - mt_a); tm_bar += (unsigned)(mt_c - mt_b); tm_lg += (unsigned)(mt_e - mt_d);
-      tm_s0 += (unsigned)(mt_a - mt_prev); tm_s1 += (unsigned)(mt_d - mt_c); mt_prev = mt_e;
-#endif
     };
     {
-      int s = 0;
-      for (; s + 2 < nk; s++) k_step(s, src, s + 2);
-      for (; s < nk; s++) k_step(s, nxt_src, s + 2 - nk < nk ? s + 2 - nk : 0);
+      // step 0 loads this tile's step 2, or (nk == 2) the next tile's step 0; descriptors picked with scalar selects
+      const bool own = nk > 2;
+      LoadSrc l0;
+#pragma unroll
+      for (int d = 0; d < 4; d++) { l0.ra[d] = own ? src.ra[d] : nxt_src.ra[d]; l0.rb[d] = own ? src.rb[d] : nxt_src.rb[d]; }
+      l0.kstart = own ? src.kstart : nxt_src.kstart;
+      k_step(0, l0, own ? 2 : 0, std::true_type{});
+      int s = 1;
+      for (; s + 2 < nk; s++) k_step(s, src, s + 2, std::false_type{});
+      for (; s < nk; s++) k_step(s, nxt_src, s + 2 - nk, std::false_type{});
     }
     par = (par + nk) & 1;
     mfma_fence();
     LF_TICK(tk2);
 
-    // ------------------------------------------------------------ epilogue: bias, convert, 16-row bands through LDS
-    {
+    // ------------------------------------------------------------ LoRA term: operands; forward: 64 MFMAs per chunk onto the
+    // accumulators (dX: the term is formed per block row inside the epilogue below, from up to two chunks = 32 rank columns)
+    lf_u32x2 rf0[8], lv0[8], rf1[8], lv1[8];
+    lf_u32x4 mw[8];
+    if constexpr (LORA) {
+      int sl = lane;
+      asm volatile("" : "+v"(sl));
+      const int l16 = sl & 15, kg = sl >> 4;
+      const T* rp = rt.rp;
+      const int rank = rt.rank;
+      const __amdgpu_buffer_rsrc_t rsrcRc = __builtin_amdgcn_make_buffer_rsrc((void*)rp, 0, 0x7fffffff, 0x00020000);
+      // chunk t of the operands: 16 rank columns, two registers per 16x16x16 fragment.  FROM_LDS: the A_i fragments of
+      // chunk 0 of the dX product are transposing reads of the rows that landed in the wave's LDS area (within a
+      // 16-lane group, lane 4j+c addresses row j, columns 4c..4c+3 and receives column lane&15, rows 0..3).
+      auto load_chunk = [&](int t, lf_u32x2 (&rf)[8], lf_u32x2 (&lv)[8], auto FROM_LDS) __attribute__((always_inline)) {
+        const int r0 = t * 16 + kg * 4;
+        const int rcc = r0 < rank ? r0 : 0;   // lanes beyond the rank re-read the first columns; zeroed in prep_chunk
+#pragma unroll
+        for (int i = 0; i < 8; i++) lv[i] = *(const lf_u32x2*)(Lp + (int64_t)(wrow0 + i * 16 + l16) * p.R + r0);
+        if constexpr (FROM_LDS.value) {
+          const uint32_t ad = area + (kg * 4 + (l16 >> 2)) * 256 + (l16 & 3) * 8;
+          lf_u32x2 t0, t1, t2, t3, t4, t5, t6, t7;
+          asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(t0) : "v"(ad) : "memory");
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:32" : "=v"(t1) : "v"(ad) : "memory");
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:64" : "=v"(t2) : "v"(ad) : "memory");
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:96" : "=v"(t3) : "v"(ad) : "memory");
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:128" : "=v"(t4) : "v"(ad) : "memory");
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:160" : "=v"(t5) : "v"(ad) : "memory");
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:192" : "=v"(t6) : "v"(ad) : "memory");
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:224" : "=v"(t7) : "v"(ad) : "memory");
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(t0), "+v"(t1), "+v"(t2), "+v"(t3), "+v"(t4), "+v"(t5), "+v"(t6), "+v"(t7) :: "memory");
+          rf[0] = t0; rf[1] = t1; rf[2] = t2; rf[3] = t3; rf[4] = t4; rf[5] = t5; rf[6] = t6; rf[7] = t7;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            const int gn = n0 + wn * 128 + j * 16 + l16;
+            if constexpr (!NN) {
+              rf[j] = *(const lf_u32x2*)(rp + (int64_t)gn * rank + rcc);
+            } else {
+              const uint32_t voff = (uint32_t)((rcc * p.N + gn) * 2);
+              uint32_t e[4];
+#pragma unroll
+              for (int k = 0; k < 4; k++) e[k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcRc, voff, k * p.N * 2, 0);
+              rf[j] = lf_u32x2{e[0] | (e[1] << 16), e[2] | (e[3] << 16)};
+            }
+          }
+        }
+      };
+      // lanes whose rank columns lie beyond the adapter's rank feed zeros; the forward scale goes into the 16-bit L
+      // fragment (fp32 product, one rounding; exact for powers of two)
+      auto prep_chunk = [&](int t, lf_u32x2 (&rf)[8], lf_u32x2 (&lv)[8]) __attribute__((always_inline)) {
+        const bool in_r = t * 16 + kg * 4 < rank;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+          for (int d = 0; d < 2; d++) rf[j][d] = in_r ? rf[j][d] : 0u;
+        if (p.mult_mode == 0 && rt.mult != 1.f) {
+#pragma unroll
+          for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int d = 0; d < 2; d++)
+              lv[i][d] = BigOp<T>::pack2(BigOp<T>::to_float((uint16_t)(lv[i][d] & 0xffffu)) * rt.mult, BigOp<T>::to_float((uint16_t)(lv[i][d] >> 16)) * rt.mult);
+        }
+        // The MFMAs are inline assembly, which the compiler's hazard recogniser does not see: a vector ALU result
+        // needs wait states before an MFMA reads it.  The nop takes the operands as in/outs, so every instruction
+        // that produces them stays in front of it and every MFMA behind.
+        asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
+                                 "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]));
+      };
+      if constexpr (NN) {
+        // dX product: the term is formed in the epilogue, block row by block row, under the keep bits of the wave's
+        // block (one 16-byte row piece per block row, from the LDS area; all ones where no mask applies)
+        const uint32_t ad = area + 4096 + l16 * 16;
+        lf_u32x4 m0_, m1_, m2_, m3_, m4_, m5_, m6_, m7_;
+        asm volatile("ds_read_b128 %0, %1" : "=v"(m0_) : "v"(ad) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:256" : "=v"(m1_) : "v"(ad) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:512" : "=v"(m2_) : "v"(ad) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:768" : "=v"(m3_) : "v"(ad) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(m4_) : "v"(ad) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:1280" : "=v"(m5_) : "v"(ad) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:1536" : "=v"(m6_) : "v"(ad) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:1792" : "=v"(m7_) : "v"(ad) : "memory");
+#ifdef LF_DBG_NOLDS
+        load_chunk(0, rf0, lv0, std::false_type{});
+#else
+        load_chunk(0, rf0, lv0, std::true_type{});
+#endif
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(m0_), "+v"(m1_), "+v"(m2_), "+v"(m3_), "+v"(m4_), "+v"(m5_), "+v"(m6_), "+v"(m7_) :: "memory");
+        const lf_u32x4 ones = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+        mw[0] = sel ? m0_ : ones; mw[1] = sel ? m1_ : ones; mw[2] = sel ? m2_ : ones; mw[3] = sel ? m3_ : ones;
+        mw[4] = sel ? m4_ : ones; mw[5] = sel ? m5_ : ones; mw[6] = sel ? m6_ : ones; mw[7] = sel ? m7_ : ones;
+        prep_chunk(0, rf0, lv0);
+        if (n16 > 1) { load_chunk(1, rf1, lv1, std::false_type{}); prep_chunk(1, rf1, lv1); }
+      } else {
+        load_chunk(0, rf0, lv0, std::false_type{});
+        prep_chunk(0, rf0, lv0);
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+          for (int j = 0; j < 8; j++) BigOp<T>::mfma16(acc[i][j], rf0[j], lv0[i]);
+        for (int t = 1; t < n16; t++) {
+          load_chunk(t, rf1, lv1, std::false_type{});
+          prep_chunk(t, rf1, lv1);
+#pragma unroll
+          for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) BigOp<T>::mfma16(acc[i][j], rf1[j], lv1[i]);
+        }
+        mfma_fence();
+      }
+    }
+
+    // ------------------------------------------------------------ epilogue: (masked LoRA term,) bias, convert, 16-row bands through LDS
+    auto epilogue = [&](auto MASKED) __attribute__((always_inline)) {
       // lane-dependent addresses are derived from an opaque copy of the lane id: computed here, every tile, in a few
       // instructions -- otherwise the compiler hoists a hundred address registers out of the tile loop and spills them
       int ln = lane;
@@ -711,12 +654,54 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       }
       const int orow = ln >> 4, og = ln & 15;  // on the way out: 16 lanes per 256-byte row, 4 rows per instruction
       T* crow = C + (int64_t)(wrow0 + orow) * p.ldc + n0 + wn * 128 + og * 8;
+      // Masked term: the product of block row i (8 blocks, 16x16x16 MFMAs per chunk of 16 rank columns) goes to
+      // ordinary vector registers, P[i & 1]; block row i+1 is multiplied while block row i is converted, which also
+      // covers the wait states between an MFMA and the vector instructions that read its result.  The lane's keep
+      // bits of block (i, j) are bits (j&1)*16 + kg*4 .. +3 of dword j>>1 of the row piece mw[i].
+      lf_f32x4 P[2][8];
+      const float mult = p.mult_mode == 1 ? rt.mult : 1.f;   // (a forward scale is already in the L fragments)
+      const uint32_t bsh = (uint32_t)ekg * 4;
+      auto p_row = [&](auto I) __attribute__((always_inline)) {
+        constexpr int i = I.value;
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
+        for (int j = 0; j < 8; j++) BigOp<T>::mfma16_v0(P[i & 1][j], rf0[j], lv0[i]);
+        if (n16 > 1) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) BigOp<T>::mfma16_v(P[i & 1][j], rf1[j], lv1[i]);
+        }
+      };
+      if constexpr (MASKED.value) p_row(integral_constant<int, 0>{});
+      sfor<8>([&](auto I) {
+        constexpr int i = I.value;
+        uint32_t mws[4] = {0u, 0u, 0u, 0u};
+        if constexpr (MASKED.value) {
+          if constexpr (i + 1 < 8) p_row(integral_constant<int, i + 1>{});
+          lf_f32x4(&tm)[8] = P[i & 1];
+          // wait states between the MFMAs of this block row (a block row of MFMAs ago, except for the last) and the
+          // vector instructions that read their results
+          asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7"
+                       : "+v"(tm[0]), "+v"(tm[1]), "+v"(tm[2]), "+v"(tm[3]), "+v"(tm[4]), "+v"(tm[5]), "+v"(tm[6]), "+v"(tm[7]));
+#pragma unroll
+          for (int q = 0; q < 4; q++) mws[q] = mw[i][q] >> bsh;
+        }
         // band = the 16 rows of accumulator block row i; band row r, granule g (16 bytes = 8 columns) at slot g ^ r
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-          const lf_f32x4 a = acc[i][j];
+          // a definition right in front of the use: the copies out of the accumulation registers cannot rise above it
+          // (without it the masked variant reads all 256 up front, into registers it does not have)
+          if constexpr (MASKED.value) asm volatile("" : "+a"(acc[i][j]));
+          lf_f32x4 a = acc[i][j];
+          if constexpr (MASKED.value) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)mws[j >> 1], (j & 1) * 16 + e, 1);   // 0 or all ones
+              // (the element goes through a scalar first: __builtin_bit_cast applied directly to an element expression of
+              // a vector reads element 0 for every index with this compiler)
+              const float pe = P[i & 1][j][e];
+              const float pm = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pe) & keep);
+              a[e] = __builtin_fmaf(pm, mult, a[e]);   // 1/(1-p) in fp32
+            }
+          }
           const float b0 = BigOp<T>::to_float((uint16_t)(bvp[j][0] & 0xffffu)), b1 = BigOp<T>::to_float((uint16_t)(bvp[j][0] >> 16));
           const float b2 = BigOp<T>::to_float((uint16_t)(bvp[j][1] & 0xffffu)), b3 = BigOp<T>::to_float((uint16_t)(bvp[j][1] >> 16));
           const lf_u32x2 o = {BigOp<T>::pack2(a[0] + b0, a[1] + b1), BigOp<T>::pack2(a[2] + b2, a[3] + b3)};
@@ -732,13 +717,17 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
           asm volatile("ds_read_b128 %0, %1" : "=v"(v[rr]) : "v"(ad) : "memory");
         }
         lgkm0();
+        // Before the first store: the next tile's first two stages have landed (requested in this tile's last two K
+        // steps).  Waiting here, not at the next tile's start, keeps the stores out of the wait.
+        if constexpr (i == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
         // non-temporal: the output is not read again by this kernel; stored this way it leaves the L2 to the operand
-        // panels and its stores are acknowledged sooner (the next tile's first wait for memory is a wait for them)
+        // panels
         for (int rr = 0; rr < 4; rr++) __builtin_nontemporal_store(v[rr], (lf_u32x4*)(crow + (int64_t)(i * 16 + rr * 4) * p.ldc));
         __builtin_amdgcn_sched_barrier(0);  // one band at a time: the scheduler otherwise reads all 256 accumulators up front
-      }
-    }
+      });
+    };
+    epilogue(std::bool_constant<NN && LORA>{});
 #ifdef LF_BIG_TIMING
     if (tid == 0) {
       const long long tk3 = __builtin_readcyclecounter();
@@ -748,11 +737,6 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       atomicAdd(&lf_big_timing[2], (unsigned long long)(tk3 - tk2));
       atomicAdd(&lf_big_timing[3], (unsigned long long)(wall_clock64() - tw0));
       atomicAdd(&lf_big_timing[4], 1ull);
-      atomicAdd(&lf_big_timing[7], (unsigned long long)tm_vm);
-      atomicAdd(&lf_big_timing[8], (unsigned long long)tm_bar);
-      atomicAdd(&lf_big_timing[9], (unsigned long long)tm_lg);
-      atomicAdd(&lf_big_timing[10], (unsigned long long)tm_s0);
-      atomicAdd(&lf_big_timing[11], (unsigned long long)tm_s1);
     }
 #endif
     tile = nxt_tile;
@@ -798,10 +782,12 @@ int lf_cu_count() {
 }
 
 int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, hipStream_t st) {
-  if (p.K % BK != 0 || p.M < BM || p.N < BN || p.N % 8 != 0) return LF_ESHAPE;  // edge tiles are shifted inwards
+  if (p.K % BK != 0 || p.K < 2 * BK || p.M < BM || p.N < BN || p.N % 8 != 0) return LF_ESHAPE;  // edge tiles are shifted inwards
   // a wave's 128 rows lie in one routing block, also in a shifted edge tile
   if (seg.table != nullptr && (seg.block_size_m % 128 != 0 || p.M % 128 != 0)) return LF_ESHAPE;
-  if (p.mask != nullptr && p.N % 16 != 0) return LF_ESHAPE;
+  // the keep-mask comes bit-packed (16 bytes per 128 columns of a row); the dX product forms its term from up to 32 rank columns
+  if (p.mask != nullptr && (!p.mask_bits || p.N % 128 != 0 || p.ldmask % 4 != 0)) return LF_ESHAPE;
+  if (nn && p.L != nullptr && p.R > 32) return LF_ESHAPE;
   const int wgs = lf_cu_count();
   const bool lora = p.L != nullptr;
   if (dtype == LF_BF16) {

@@ -291,7 +291,10 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         mv[ib][ii] = *(const lf_u32x4*)(p.mask + (int64_t)gm * p.ldmask + mcol);
       }
     };
-    if (use_mask && MEARLY) {
+    // (a bit-packed mask is read directly, one dword per accumulator block pair, below: these tiles serve short
+    // row ranges and small shapes, where its few bytes come from L2)
+    const bool bytes_mask = use_mask && !p.mask_bits, bits_mask = use_mask && p.mask_bits;
+    if (bytes_mask && MEARLY) {
 #pragma unroll
       for (int ib = 0; ib < TM32; ib++) load_mask_band(ib);
     }
@@ -342,7 +345,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       const int ib = i >> 1, h = i & 1;  // band of 32 rows, half of the band
-      if (use_mask && h == 0) {
+      if (bytes_mask && h == 0) {
         if constexpr (!MEARLY) load_mask_band(ib);
 #pragma unroll
         for (int ii = 0; ii < MNI; ii++) {
@@ -354,7 +357,15 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         acc[i][j] *= mult;
-        if (use_mask) {
+        if (bits_mask) {
+          // element n of a mask row = bit n & 7 of byte n >> 3: the lane's four columns are four bits of one dword
+          const int gm = min(wrow0 + i * 16 + l16, p.M - 1);
+          const int col0 = min(n0 + wn * WN + j * 16 + kg * 4, p.N - 4);
+          const uint32_t w = *(const uint32_t*)(p.mask + (int64_t)gm * p.ldmask + ((col0 >> 5) << 2));
+          const uint32_t bits = w >> (col0 & 31);
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[i][j][e] = ((bits >> e) & 1u) ? acc[i][j][e] : 0.f;
+        } else if (use_mask) {
           const int dw = j * 4 + kg;  // dword of the 4 columns j*16 + kg*4 ..
           const uint32_t mk = *(const uint32_t*)(mreg + r * WN + (((dw >> 2) ^ ((r / MRW) & (MLPR - 1))) << 4) + (dw & 3) * 4);
 #pragma unroll
@@ -748,12 +759,18 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
   if (p.ldc % 8 != 0 || ((uintptr_t)p.C & 15) != 0) return LF_ESHAPE;
   if (p.L != nullptr && (p.R % 16 != 0 || p.R <= 0 || p.R > LF_MAX_RANK)) return LF_ESHAPE;
   // the keep-mask is read 16 bytes at a time
-  if (p.mask != nullptr && (p.N % 16 != 0 || p.ldmask % 16 != 0 || ((uintptr_t)p.mask & 15) != 0)) return LF_ESHAPE;
+  if (p.mask != nullptr && !p.mask_bits && (p.N % 16 != 0 || p.ldmask % 16 != 0 || ((uintptr_t)p.mask & 15) != 0)) return LF_ESHAPE;
+  // bit-packed: read 4 bytes at a time (the persistent kernel: 16), rows of whole dwords
+  if (p.mask != nullptr && p.mask_bits && (p.N % 32 != 0 || p.ldmask % 4 != 0 || ((uintptr_t)p.mask & 15) != 0)) return LF_ESHAPE;
   // tile loads address a panel of 256 rows (the K-major operand of the NN product: all of it) with 32-bit byte offsets
   if (256 * p.lda * 2 >= 0x7fffffffLL || (int64_t)(nn ? p.K : 256) * p.ldb * 2 >= 0x7fffffffLL) return LF_ESHAPE;
   if (seg.table != nullptr && (seg.block_size_m % 64 != 0)) return LF_ESHAPE;
+  const bool planned = force_cfg < 0;
   auto launch = [&](const LfGemmParams& q, int cfg) {
     if (seg.table != nullptr && seg.block_size_m % 128 != 0 && (cfg == 0 || cfg == 1 || cfg == 7)) cfg = 2;
+    // what the persistent kernel does not take goes to the eight-wave 256x256 tile: a keep-mask with one byte per
+    // element, a dX term of more than 32 rank columns and (when the library chose the tile) a contraction of one K step
+    if (cfg == 7 && ((q.mask != nullptr && (!q.mask_bits || q.N % 128 != 0)) || (nn && q.L != nullptr && q.R > 32) || (planned && q.K < 128))) cfg = 1;
     if (cfg == 7) return lf_launch_gemm_big(q, seg, nn, dtype, st);
     if (dtype == LF_BF16) return nn ? launch_dtype<__bf16, true>(q, seg, cfg, st) : launch_dtype<__bf16, false>(q, seg, cfg, st);
     if (dtype == LF_F16) return nn ? launch_dtype<_Float16, true>(q, seg, cfg, st) : launch_dtype<_Float16, false>(q, seg, cfg, st);

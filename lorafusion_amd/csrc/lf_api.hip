@@ -4,10 +4,12 @@
 
 int lf_launch_nf4_dequant(const uint8_t*, const void*, const float*, const float*, const float*, void*, int64_t,
                           int, int, int, hipStream_t);
-int lf_launch_xa(const void*, const void*, int64_t, void*, const uint8_t*, uint8_t*, uint64_t, void*, int, int, int, const LfSegTable&, int,
+int lf_launch_xa(const void*, const void*, int64_t, void*, const uint8_t*, uint8_t*, int, uint64_t, void*, int, int, int, const LfSegTable&, int,
                  hipStream_t);
+int lf_launch_mask_pack(const uint8_t*, uint8_t*, int64_t, hipStream_t);
+int lf_launch_mask_unpack(const uint8_t*, uint8_t*, int64_t, hipStream_t);
 int lf_launch_dys_dyb(const void*, const void*, void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
-int lf_launch_da(const void*, const uint8_t*, const void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
+int lf_launch_da(const void*, const uint8_t*, int, const void*, void*, size_t, int, int, int, const LfSegTable&, int, hipStream_t);
 int lf_launch_dropout_mask(uint8_t*, int, int, float, const float*, int, uint64_t, hipStream_t);
 size_t lf_xa_workspace(int, int, int, const LfSegTable&);
 size_t lf_dys_dyb_workspace(int, int, int, const LfSegTable&);
@@ -72,6 +74,12 @@ int make_seg(const lf_routing* r, int M, const void* const* ptrs, void* const* o
 }
 
 bool bad_dtype(int d) { return d != LF_BF16 && d != LF_F16; }
+// `dtype` arguments carry the keep-mask format in LF_MASK_BITS: returns that flag and leaves the element type
+int take_mask_bits(int& dtype) {
+  const int bits = (dtype & LF_MASK_BITS) != 0;
+  dtype &= ~LF_MASK_BITS;
+  return bits;
+}
 
 // What the rank-r passes and their planners assume of a dimension they tile (N of dys_dyb, K of xa / da) and of R.
 bool bad_tiled_dim(int v) { return v <= 0 || v % 128 != 0; }
@@ -81,7 +89,7 @@ bool bad_rank_cols(int R) { return R <= 0 || R % 16 != 0 || R > LF_MAX_RANK; }
 
 extern "C" {
 
-int lf_version(void) { return 1; }
+int lf_version(void) { return 2; }
 
 const char* lf_strerror(int code) {
   switch (code) {
@@ -127,35 +135,38 @@ size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* 
 
 int lf_lora_xa(const void* X, const uint8_t* mask, const void* const* a_ptrs, void* S, void* workspace,
                size_t ws_bytes, int M, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  const int mb = take_mask_bits(dtype);
   if (bad_dtype(dtype) || !a_ptrs) return LF_EINVAL;
   LfSegTable t;
   int rc = make_seg(routing, M, a_ptrs, nullptr, t);
   if (rc != LF_OK) return rc;
   for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
   (void)workspace; (void)ws_bytes;  // no partial sums leave the workgroups
-  return lf_launch_xa(X, nullptr, 0, nullptr, mask, nullptr, 0, S, M, K, R, t, dtype, (hipStream_t)stream);
+  return lf_launch_xa(X, nullptr, 0, nullptr, mask, nullptr, mb, 0, S, M, K, R, t, dtype, (hipStream_t)stream);
 }
 
 int lf_lora_xa_seeded(const void* X, uint8_t* mask_out, const void* const* a_ptrs, void* S, int M, int K, int R,
                       const lf_routing* routing, uint64_t seed, int dtype, void* stream) {
+  const int mb = take_mask_bits(dtype);
   if (bad_dtype(dtype) || !a_ptrs || !mask_out) return LF_EINVAL;
   LfSegTable t;
   int rc = make_seg(routing, M, a_ptrs, nullptr, t);
   if (rc != LF_OK) return rc;
   for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
-  return lf_launch_xa(X, nullptr, 0, nullptr, nullptr, mask_out, seed, S, M, K, R, t, dtype, (hipStream_t)stream);
+  return lf_launch_xa(X, nullptr, 0, nullptr, nullptr, mask_out, mb, seed, S, M, K, R, t, dtype, (hipStream_t)stream);
 }
 
 int lf_lora_xa_silu_mul(const void* G, const void* U, int64_t ld, void* X_out, const uint8_t* mask, uint8_t* mask_out,
                         uint64_t seed, const void* const* a_ptrs, void* S, int M, int K, int R, const lf_routing* routing,
                         int dtype, void* stream) {
+  const int mb = take_mask_bits(dtype);
   if (bad_dtype(dtype) || !a_ptrs || !G || !U || !X_out) return LF_EINVAL;
   if (mask && mask_out) return LF_EINVAL;
   LfSegTable t;
   int rc = make_seg(routing, M, a_ptrs, nullptr, t);
   if (rc != LF_OK) return rc;
   for (int s = 0; s < t.n_seg; s++) if (!t.ptr[s]) return LF_EINVAL;
-  return lf_launch_xa(G, U, ld, X_out, mask, mask_out, seed, S, M, K, R, t, dtype, (hipStream_t)stream);
+  return lf_launch_xa(G, U, ld, X_out, mask, mask_out, mb, seed, S, M, K, R, t, dtype, (hipStream_t)stream);
 }
 
 int lf_swiglu_lora_fwd(const void* G, const void* U, int64_t ld, void* X_out, const void* W, const void* bias,
@@ -164,7 +175,7 @@ int lf_swiglu_lora_fwd(const void* G, const void* U, int64_t ld, void* X_out, co
                        const lf_routing* routing, int dtype, void* stream) {
   int rc = lf_lora_xa_silu_mul(G, U, ld, X_out, mask, mask_out, seed, a_ptrs, S_out, M, K, R, routing, dtype, stream);
   if (rc != LF_OK) return rc;
-  return lf_lora_xw_sb(X_out, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype, stream);
+  return lf_lora_xw_sb(X_out, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
 }
 
 int lf_lora_xw_sb(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs,
@@ -197,15 +208,17 @@ int lf_lora_dys_dyb(const void* dY, const void* S, const void* const* b_ptrs, vo
 
 int lf_lora_da(const void* X, const uint8_t* mask, const void* dS, void* const* da_ptrs, void* workspace,
                size_t ws_bytes, int M, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  const int mb = take_mask_bits(dtype);
   if (bad_dtype(dtype) || !da_ptrs) return LF_EINVAL;
   LfSegTable t;
   int rc = make_seg(routing, M, nullptr, da_ptrs, t);
   if (rc != LF_OK) return rc;
-  return lf_launch_da(X, mask, dS, workspace, ws_bytes, M, K, R, t, dtype, (hipStream_t)stream);
+  return lf_launch_da(X, mask, mb, dS, workspace, ws_bytes, M, K, R, t, dtype, (hipStream_t)stream);
 }
 
 int lf_lora_dyw_dsa(const void* dY, const void* W, const void* dS, const void* const* a_ptrs, const uint8_t* mask,
                     void* dX, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  const int mb = take_mask_bits(dtype);
   if (bad_dtype(dtype) || !dY || !W || !dX) return LF_EINVAL;
   LfSegTable t{};
   if (dS) {
@@ -219,7 +232,7 @@ int lf_lora_dyw_dsa(const void* dY, const void* W, const void* dS, const void* c
   LfGemmParams p{};
   p.A = dY; p.B = W; p.C = dX; p.bias = nullptr;
   p.M = M; p.N = K; p.K = N; p.lda = N; p.ldb = K; p.ldc = K;
-  p.L = dS; p.R = R; p.mask = mask; p.ldmask = K; p.mult_mode = 1;
+  p.L = dS; p.R = R; p.mask = mask; p.ldmask = mb ? K / 8 : K; p.mask_bits = mb; p.mult_mode = 1;
   return lf_launch_gemm(p, t, /*nn=*/true, dtype, -1, (hipStream_t)stream);
 }
 
@@ -228,7 +241,7 @@ int lf_lora_fwd(const void* X, const void* W, const void* bias, const uint8_t* m
                 int K, int R, const lf_routing* routing, int dtype, void* stream) {
   int rc = lf_lora_xa(X, mask, a_ptrs, S_out, workspace, ws_bytes, M, K, R, routing, dtype, stream);
   if (rc != LF_OK) return rc;
-  return lf_lora_xw_sb(X, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype, stream);
+  return lf_lora_xw_sb(X, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
 }
 
 int lf_lora_fwd_seeded(const void* X, const void* W, const void* bias, uint8_t* mask_out, const void* const* a_ptrs,
@@ -236,14 +249,14 @@ int lf_lora_fwd_seeded(const void* X, const void* W, const void* bias, uint8_t* 
                        const lf_routing* routing, uint64_t seed, int dtype, void* stream) {
   int rc = lf_lora_xa_seeded(X, mask_out, a_ptrs, S_out, M, K, R, routing, seed, dtype, stream);
   if (rc != LF_OK) return rc;
-  return lf_lora_xw_sb(X, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype, stream);
+  return lf_lora_xw_sb(X, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
 }
 
 int lf_lora_bwd(const void* dY, const void* X, const void* W, const uint8_t* mask, const void* S,
                 const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
                 void* const* db_ptrs, void* dS_out, void* workspace, size_t ws_bytes, int M, int N, int K, int R,
                 const lf_routing* routing, int dtype, void* stream) {
-  int rc = lf_lora_dys_dyb(dY, S, b_ptrs, dS_out, db_ptrs, workspace, ws_bytes, M, N, R, routing, dtype, stream);
+  int rc = lf_lora_dys_dyb(dY, S, b_ptrs, dS_out, db_ptrs, workspace, ws_bytes, M, N, R, routing, dtype & ~LF_MASK_BITS, stream);
   if (rc != LF_OK) return rc;
   rc = lf_lora_da(X, mask, dS_out, da_ptrs, workspace, ws_bytes, M, K, R, routing, dtype, stream);
   if (rc != LF_OK) return rc;
@@ -255,7 +268,7 @@ int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8
                        const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
                        void* const* db_ptrs, void* dS_out, int M, int N, int K, int R, const lf_routing* routing,
                        int dtype, void* stream) {
-  if (bad_dtype(dtype) || !dY || !X || !S || !b_ptrs || !da_ptrs || !db_ptrs || !dS_out) return LF_EINVAL;
+  if (bad_dtype(dtype & ~LF_MASK_BITS) || !dY || !X || !S || !b_ptrs || !da_ptrs || !db_ptrs || !dS_out) return LF_EINVAL;
   if (dX && (!W || !a_ptrs)) return LF_EINVAL;
   if (M <= 0 || N <= 0 || K <= 0 || R <= 0) return LF_EINVAL;
   if (bad_tiled_dim(N) || bad_tiled_dim(K) || bad_rank_cols(R)) return LF_ESHAPE;
@@ -323,10 +336,10 @@ static int nf4_dense(const lf_nf4_weight* W, bool needed, void* workspace, size_
 int lf_nf4_lora_fwd(const void* X, const lf_nf4_weight* W, const void* bias, const uint8_t* mask,
                     const void* const* a_ptrs, const void* const* b_ptrs, void* Y, void* S_out, void* workspace,
                     size_t ws_bytes, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
-  if (bad_dtype(dtype)) return LF_EINVAL;
+  if (bad_dtype(dtype & ~LF_MASK_BITS)) return LF_EINVAL;
   const void* dense;
   size_t head;
-  int rc = nf4_dense(W, true, workspace, ws_bytes, N, K, dtype, (hipStream_t)stream, &dense, &head);
+  int rc = nf4_dense(W, true, workspace, ws_bytes, N, K, dtype & ~LF_MASK_BITS, (hipStream_t)stream, &dense, &head);
   if (rc != LF_OK) return rc;
   return lf_lora_fwd(X, dense, bias, mask, a_ptrs, b_ptrs, Y, S_out, workspace ? (char*)workspace + head : nullptr,
                      ws_bytes - head, M, N, K, R, routing, dtype, stream);
@@ -336,13 +349,25 @@ int lf_nf4_lora_bwd(const void* dY, const void* X, const lf_nf4_weight* W, const
                     const void* const* a_ptrs, const void* const* b_ptrs, void* dX, void* const* da_ptrs,
                     void* const* db_ptrs, void* dS_out, void* workspace, size_t ws_bytes, int M, int N, int K, int R,
                     const lf_routing* routing, int dtype, void* stream) {
-  if (bad_dtype(dtype)) return LF_EINVAL;
+  if (bad_dtype(dtype & ~LF_MASK_BITS)) return LF_EINVAL;
   const void* dense;
   size_t head;
-  int rc = nf4_dense(W, dX != nullptr, workspace, ws_bytes, N, K, dtype, (hipStream_t)stream, &dense, &head);
+  int rc = nf4_dense(W, dX != nullptr, workspace, ws_bytes, N, K, dtype & ~LF_MASK_BITS, (hipStream_t)stream, &dense, &head);
   if (rc != LF_OK) return rc;
   return lf_lora_bwd(dY, X, dense, mask, S, a_ptrs, b_ptrs, dX, da_ptrs, db_ptrs, dS_out,
                      workspace ? (char*)workspace + head : nullptr, ws_bytes - head, M, N, K, R, routing, dtype, stream);
+}
+
+int lf_mask_pack(const uint8_t* mask_bytes, uint8_t* mask_bits, int M, int K, void* stream) {
+  if (!mask_bytes || !mask_bits || M <= 0 || K <= 0) return LF_EINVAL;
+  if (K % 128 != 0 || (((uintptr_t)mask_bytes | (uintptr_t)mask_bits) & 15) != 0) return LF_ESHAPE;
+  return lf_launch_mask_pack(mask_bytes, mask_bits, (int64_t)M * K, (hipStream_t)stream);
+}
+
+int lf_mask_unpack(const uint8_t* mask_bits, uint8_t* mask_bytes, int M, int K, void* stream) {
+  if (!mask_bytes || !mask_bits || M <= 0 || K <= 0) return LF_EINVAL;
+  if (K % 128 != 0 || (((uintptr_t)mask_bytes | (uintptr_t)mask_bits) & 15) != 0) return LF_ESHAPE;
+  return lf_launch_mask_unpack(mask_bits, mask_bytes, (int64_t)M * K, (hipStream_t)stream);
 }
 
 int lf_dropout_mask(uint8_t* mask, int M, int K, float p, const lf_routing* routing, uint64_t seed, void* stream) {

@@ -46,7 +46,8 @@ struct LfGemmParams {
   const void* L;      // [M,R] skinny left operand of the LoRA term (S or dS), or nullptr
   int R;              // columns of L (multiple of 16)
   const uint8_t* mask;  // [M,N] keep-mask applied to the LoRA term (dX path) or nullptr
-  int64_t ldmask;
+  int64_t ldmask;     // bytes between mask rows
+  int mask_bits;      // 0: one byte per element; 1: one bit per element (element n of a row = bit n & 7 of byte n >> 3)
   int mult_mode;      // 0: LoRA term * scale ; 1: LoRA term * 1/(1-p), masked where p > 0
   int grid_m, grid_n;
   int row0;           // global row of local row 0 (routing lookup when a launch covers a row range)

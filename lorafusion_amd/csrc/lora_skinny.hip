@@ -90,6 +90,16 @@ __device__ __forceinline__ lf_u32x4 apply_mask8(lf_u32x4 x, lf_u32x2 m) {
   return r;
 }
 
+// Bit-packed keep-masks: element k of a row = bit k & 7 of byte k >> 3 of the row (K / 8 bytes per row).
+// The eight keep bytes (0/1 each, `lo` = the first four) as eight bits, and back: one multiply gathers / spreads four
+// single bits (no two partial products meet in one bit position, so nothing carries).
+__device__ __forceinline__ uint32_t pack_keep8(uint32_t lo, uint32_t hi) {
+  return ((lo * 0x01020408u) >> 24) | (((hi * 0x01020408u) >> 24) << 4);
+}
+__device__ __forceinline__ lf_u32x2 expand_keep8(uint32_t b) {
+  return lf_u32x2{((b & 0xfu) * 0x00204081u) & 0x01010101u, (((b >> 4) & 0xfu) * 0x00204081u) & 0x01010101u};
+}
+
 __device__ __forceinline__ lf_u32x4 tr_read8(const char* p, int pitch) {
   // 8 contraction elements (rows r..r+3 and r+4..r+7) of this lane's column
   lf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(p));
@@ -121,14 +131,14 @@ struct TileRegs {
 // Coalesced load of the tile whose first element is src[row0*ld + col0]; rows are clamped to max_row-1.
 template <typename T>
 __device__ __forceinline__ void tile_load(TileRegs& r, const T* __restrict__ src, const uint8_t* __restrict__ mask,
-                                          int64_t ld, int row0, int max_row, int col0, int tid, bool use_mask) {
+                                          int64_t ld, int row0, int max_row, int col0, int tid, bool use_mask, bool mask_bits) {
   const int srcg = (tid & 7) ^ tile_key(tid >> 3);   // rows i*32 + (tid>>3) share their key
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int row = min(row0 + i * 32 + (tid >> 3), max_row - 1);
     const int64_t off = (int64_t)row * ld + col0 + srcg * 8;
     r.x[i] = *((const lf_u32x4*)(src + off));
-    if (use_mask) r.m[i] = *((const lf_u32x2*)(mask + off));
+    if (use_mask) r.m[i] = mask_bits ? expand_keep8(mask[off >> 3]) : *((const lf_u32x2*)(mask + off));
   }
 }
 
@@ -188,7 +198,7 @@ constexpr int xa_unroll(int rt) { return rt <= 1 ? 4 : rt <= 2 ? 2 : 1; }
 template <typename T, int RT, bool GEN, bool ACT>
 __global__ void __launch_bounds__(xa_waves(RT) * 64)
 lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T* __restrict__ act_out,
-               const uint8_t* __restrict__ mask, uint8_t* __restrict__ mask_out,
+               const uint8_t* __restrict__ mask, uint8_t* __restrict__ mask_out, int mask_bits,
                uint32_t seed_lo, uint32_t seed_hi, T* __restrict__ S, int M, int K, int R, const LfSegTable seg) {
   constexpr int XA_WAVES = xa_waves(RT), XA_U = xa_unroll(RT), NB = xa_nb(RT, ACT), XA_ROWS = xa_rows(RT, ACT);
   // the partial accumulators of the final sum reuse the patches (a barrier separates the two uses): at
@@ -218,7 +228,7 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
   for (int i = 0; i < 2 * NB; i++) {
     const int r = min(row0 + i * 8 + lrow, Mrows - 1);
     xrow[i] = X + (int64_t)r * ldx + lg * 8;
-    mrow[i] = mask + (int64_t)r * K + lg * 8;
+    mrow[i] = mask_bits ? mask + (((int64_t)r * K + lg * 8) >> 3) : mask + (int64_t)r * K + lg * 8;
     erow[i] = (int64_t)r * K + lg * 8;
     row_real[i] = row0 + i * 8 + lrow < Mrows;
   }
@@ -247,7 +257,7 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
           xv[b][u][i] = *((const lf_u32x4*)(xrow[i] + s * 64));
           if constexpr (ACT) uv[b][u][i] = *((const lf_u32x4*)((const char*)(xrow[i] + s * 64) + u_off));
           if constexpr (!GEN) {
-            if (use_mask) mv[b][u][i] = *((const lf_u32x2*)(mrow[i] + s * 64));
+            if (use_mask) mv[b][u][i] = mask_bits ? expand_keep8(mrow[i][s * 8]) : *((const lf_u32x2*)(mrow[i] + s * 64));
           }
         }
 #pragma unroll
@@ -277,7 +287,16 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
             uint32_t klo, khi;
             lf_keep8((uint64_t)(erow[i] + s * 64) >> 3, thr, seed_lo, seed_hi, klo, khi);
             mv[b][u][i] = lf_u32x2{klo, khi};
-            if (row_real[i]) *(lf_u32x2*)(mask_out + erow[i] + s * 64) = mv[b][u][i];
+            if (mask_bits) {
+              // this lane's eight bits are byte lg of the row's eight bytes of the step: the four lanes of a quad join
+              // theirs (two cross-lane moves) and one of them stores the dword
+              uint32_t w = pack_keep8(klo, khi) << (8 * (lg & 3));
+              w |= (uint32_t)__builtin_amdgcn_mov_dpp((int)w, 0xB1, 0xf, 0xf, true);   // lanes 1 0 3 2
+              w |= (uint32_t)__builtin_amdgcn_mov_dpp((int)w, 0x4E, 0xf, 0xf, true);   // lanes 2 3 0 1
+              if (row_real[i] && (lg & 3) == 0) *(uint32_t*)(mask_out + ((erow[i] + s * 64) >> 3)) = w;
+            } else {
+              if (row_real[i]) *(lf_u32x2*)(mask_out + erow[i] + s * 64) = mv[b][u][i];
+            }
           }
           *(lf_u32x4*)(patch + (i >> 1) * 2048 + wr_off[i & 1]) = use_mask ? apply_mask8(xv[b][u][i], mv[b][u][i]) : xv[b][u][i];
         }
@@ -470,14 +489,14 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
 
   TileRegs tr;
   lf_u32x4 br[NBR], sr[RT];
-  tile_load(tr, dY, (const uint8_t*)nullptr, N, bb0 * ROWS, Mrows, n_begin, tid, false);
+  tile_load(tr, dY, (const uint8_t*)nullptr, N, bb0 * ROWS, Mrows, n_begin, tid, false, false);
   load_b(br, n_begin);
   load_s(sr, bb0);
   store_s(sr);
   tile_store(tr, ys, tid, false);
   store_b(br, bs);
   if (total > 1) {
-    tile_load(tr, dY, (const uint8_t*)nullptr, N, blk_of(1) * ROWS, Mrows, col_of(1), tid, false);
+    tile_load(tr, dY, (const uint8_t*)nullptr, N, blk_of(1) * ROWS, Mrows, col_of(1), tid, false, false);
     load_b(br, col_of(1));
     if (ntiles == 1) load_s(sr, blk_of(1));
   }
@@ -533,7 +552,7 @@ lora_dys_dyb_kernel(const T* __restrict__ dY, const T* __restrict__ S, float* __
           tile_store(tr, ys + ((q + 1) & 1) * TILE_BYTES, tid, false);
           store_b(br, bs + ((q + 1) & 1) * 64 * RP);
           if (q + 2 < total) {
-            tile_load(tr, dY, (const uint8_t*)nullptr, N, blk_of(q + 2) * ROWS, Mrows, col_of(q + 2), tid, false);
+            tile_load(tr, dY, (const uint8_t*)nullptr, N, blk_of(q + 2) * ROWS, Mrows, col_of(q + 2), tid, false, false);
             load_b(br, col_of(q + 2));
             if ((q + 2) % ntiles == 0) load_s(sr, blk_of(q + 2));
           }
@@ -629,7 +648,7 @@ reduce_ds_db_kernel(const float* __restrict__ ds_part, T* __restrict__ dS, int n
 // the transpose path since the contraction index m is the slow dimension of both.
 template <typename T, int RT>
 __global__ void __launch_bounds__(256)
-lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const T* __restrict__ dS,
+lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, int mask_bits, const T* __restrict__ dS,
                float* __restrict__ part, int M, int K, int R, int group, int max_chunks, const LfSegTable seg) {
   constexpr int RP = RT * 32 + 32;
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -668,12 +687,12 @@ lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const 
 
   TileRegs tr;
   lf_u32x4 dr[RT];
-  tile_load(tr, X, mask, K, bb0 * ROWS, Mrows, kt * 64, tid, use_mask);
+  tile_load(tr, X, mask, K, bb0 * ROWS, Mrows, kt * 64, tid, use_mask, mask_bits != 0);
   load_ds(dr, bb0);
   tile_store(tr, xs, tid, use_mask);
   store_ds(dr, dss);
   if (bb0 + 1 < bb1) {
-    tile_load(tr, X, mask, K, (bb0 + 1) * ROWS, Mrows, kt * 64, tid, use_mask);
+    tile_load(tr, X, mask, K, (bb0 + 1) * ROWS, Mrows, kt * 64, tid, use_mask, mask_bits != 0);
     load_ds(dr, bb0 + 1);
   }
   __syncthreads();
@@ -700,7 +719,7 @@ lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const 
       tile_store(tr, xs + ((t + 1) & 1) * TILE_BYTES, tid, use_mask);
       store_ds(dr, dss + ((t + 1) & 1) * ROWS * RP);
       if (b + 2 < bb1) {
-        tile_load(tr, X, mask, K, (b + 2) * ROWS, Mrows, kt * 64, tid, use_mask);
+        tile_load(tr, X, mask, K, (b + 2) * ROWS, Mrows, kt * 64, tid, use_mask, mask_bits != 0);
         load_ds(dr, b + 2);
       }
     }
@@ -738,6 +757,11 @@ __device__ __forceinline__ lf_u32x4 window_rsrc(const void* base, int64_t bytes)
 __device__ __forceinline__ void dma16(const lf_u32x4& rsrc, uint32_t voff, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
+// one wave instruction: lane l fetches 4 bytes at window offset `voff` into LDS byte lds_addr + 4 l
+__device__ __forceinline__ void dma4(const lf_u32x4& rsrc, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+}
+constexpr int da_mask_tile_bytes(int fmt) { return fmt == 1 ? ROWS * 64 : fmt == 2 ? ROWS * 8 : 0; }
 template <int N>
 __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 // at most `groups` groups of G operations each may still be outstanding
@@ -774,6 +798,8 @@ __device__ __forceinline__ void mask_dma(const lf_u32x4& rsrc, const uint32_t (&
   for (int i = 0; i < 2; i++) dma16(rsrc, v[i], lds_mask + i * 4096 + wave * 1024);
 }
 // keep-mask applied in place to a landed tile (any thread mapping; here each thread takes the positions p = i*256 + tid)
+// (BITS: the mask tile holds 8 bytes per row, one bit per element)
+template <bool BITS>
 __device__ __forceinline__ void tile_apply_mask(char* tile, const char* mtile, int tid) {
   lf_u32x4 x[4];
   lf_u32x2 m[4];
@@ -781,7 +807,8 @@ __device__ __forceinline__ void tile_apply_mask(char* tile, const char* mtile, i
   for (int i = 0; i < 4; i++) {   // all reads first: behind a store the compiler would not start the next read
     const int p = i * 256 + tid, row = p >> 3, g = (p & 7) ^ tile_key(row);
     x[i] = *(const lf_u32x4*)(tile + p * 16);
-    m[i] = *(const lf_u32x2*)(mtile + row * 64 + g * 8);
+    if constexpr (BITS) m[i] = expand_keep8(*(const uint8_t*)(mtile + row * 8 + g));
+    else m[i] = *(const lf_u32x2*)(mtile + row * 64 + g * 8);
   }
 #pragma unroll
   for (int i = 0; i < 4; i++) *(lf_u32x4*)(tile + (i * 256 + tid) * 16) = apply_mask8(x[i], m[i]);
@@ -832,13 +859,15 @@ __device__ __forceinline__ lf_u32x4 side_tr8(const char* blk, int row, int c, in
 // of nt tiles keeps at most min(NS, nt + 1) stages of the ring busy, so a third block is never on order).
 //   D_j[r][k] += sum_m dS[m][r] * keep*X[m][k]   per tile j of the slice, in registers over all blocks of the chunk.
 // With a keep-mask the tile is masked in place one iteration before it is consumed.
-template <typename T, int RT, int TPW, int NS, bool MASK>
+template <typename T, int RT, int TPW, int NS, int MASK>
 __global__ void __launch_bounds__(256, 2)
 lora_da_ring_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, const T* __restrict__ dS, float* __restrict__ part,
                     int M, int K, int R, int n_slices, int group, int max_chunks, const LfSegTable seg) {
-  constexpr int STAGE = TILE_BYTES + (MASK ? ROWS * 64 : 0);
+  // MASK: 0 no keep-mask; 1 one byte per element (8 KB per tile, two loads per thread); 2 one bit per element (1 KB per
+  // tile, one 4-byte load per thread)
+  constexpr int STAGE = TILE_BYTES + da_mask_tile_bytes(MASK);
   constexpr int SIDE = ROWS * RT * 32;
-  constexpr int G = 4 + (MASK ? 2 : 0);   // operations per load group and thread, not counting a dS block
+  constexpr int G = 4 + (MASK == 1 ? 2 : MASK == 2 ? 1 : 0);   // operations per load group and thread, not counting a dS block
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   char* ring = lds;
   char* side = lds + NS * STAGE;
@@ -860,7 +889,8 @@ lora_da_ring_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, c
 
   uint32_t xv[4], mv[2], dv[RT];
   tile_voffs(xv, K, tid);
-  mask_voffs(mv, K, tid);
+  if constexpr (MASK == 2) mv[0] = mv[1] = (uint32_t)((tid >> 1) * (K >> 3) + (tid & 1) * 4);   // row tid>>1, half tid&1 of its 8 bytes
+  else mask_voffs(mv, K, tid);
   side_voffs<RT, RT>(dv, R, R, tid);
 
   // Load group of the next pair into stage `ist`; behind the last pair the last tile is ordered again.  The windows
@@ -873,11 +903,17 @@ lora_da_ring_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, c
   const int64_t xnext = (int64_t)ROWS * K * 2 - (int64_t)nt * 128;   // from behind a block's last tile to the next block's first
   auto issue = [&]() {
     tile_dma(window_rsrc(xb, xleft), xv, lds0 + ist * STAGE, wave);
-    if constexpr (MASK) {
+    if constexpr (MASK == 1) {
       // the mask has one byte where X has two: same element offsets, half the byte offsets
       const int64_t eoff = (xb - (const char*)X) >> 1;
       mask_dma(window_rsrc(mask != nullptr ? (const char*)mask + eoff : (const char*)X, mask != nullptr ? (xleft >> 1) : 0), mv,
                lds0 + ist * STAGE + TILE_BYTES, wave);
+    }
+    if constexpr (MASK == 2) {
+      // one bit where X has sixteen: the tile's 128 rows x 8 bytes land row-major (wave w: rows 32w .. 32w+31)
+      const int64_t boff = (xb - (const char*)X) >> 4;
+      dma4(window_rsrc(mask != nullptr ? (const char*)mask + boff : (const char*)X, mask != nullptr ? (xleft >> 4) : 0), mv[0],
+           lds0 + ist * STAGE + TILE_BYTES + wave * 256);
     }
     if (ij == 0 && ib < bb1) side_dma<RT>(window_rsrc(sb, sleft), dv, lds0 + NS * STAGE + ((ib - bb0) & 1) * SIDE, wave);
     ist = ist + 1 == ns ? 0 : ist + 1;
@@ -906,7 +942,7 @@ lora_da_ring_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, c
   if constexpr (MASK) {
     wait_groups<G>(ns - 2);
     ring_barrier();
-    if (use_mask) tile_apply_mask(ring, ring + TILE_BYTES, tid);
+    if (use_mask) tile_apply_mask<MASK == 2>(ring, ring + TILE_BYTES, tid);
   }
   for (int b = bb0; b < bb1; b++) {
     const char* dcur = side + ((b - bb0) & 1) * SIDE;
@@ -920,7 +956,7 @@ lora_da_ring_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, c
         issue();
         if constexpr (MASK) {
           const int nst = cst + 1 == ns ? 0 : cst + 1;
-          if (use_mask) tile_apply_mask(ring + nst * STAGE, ring + nst * STAGE + TILE_BYTES, tid);
+          if (use_mask) tile_apply_mask<MASK == 2>(ring + nst * STAGE, ring + nst * STAGE + TILE_BYTES, tid);
         }
         const char* xcur = ring + cst * STAGE;
         // all fragments of the tile first, then the MFMAs: with one or two waves per SIMD nothing else hides the LDS
@@ -1254,7 +1290,7 @@ static DysRingPlan dysr_plan(int M, int N, int R, const LfSegTable& seg) {
 size_t lf_xa_workspace(int, int, int, const LfSegTable&) { return 0; }
 
 template <typename T, int RT>
-static int xa_launch(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out,
+static int xa_launch(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out, int mask_bits,
                      uint64_t seed, void* S, int M, int K, int R, int64_t rows, const LfSegTable& seg, hipStream_t st) {
   const bool gen = mask_out != nullptr, act = U != nullptr;
   const int wg_rows = xa_rows(RT, act);
@@ -1262,7 +1298,7 @@ static int xa_launch(const void* X, const void* U, int64_t ldx, void* act_out, c
   const uint32_t lo = gen ? (uint32_t)seed : 0u, hi = gen ? (uint32_t)(seed >> 32) : 0u;
 #define LF_XA(GEN, ACT)                                                                                              \
   return lf_launch((lora_xa_kernel<T, RT, GEN, ACT>), dim3(grid), dim3(xa_waves(RT) * 64), 0, st, (const T*)X,       \
-                   (const T*)U, ldx, (T*)act_out, mask, mask_out, lo, hi, (T*)S, M, K, R, seg)
+                   (const T*)U, ldx, (T*)act_out, mask, mask_out, mask_bits, lo, hi, (T*)S, M, K, R, seg)
   if (gen && act) LF_XA(true, true);
   if (gen) LF_XA(true, false);
   if (act) LF_XA(false, true);
@@ -1271,35 +1307,35 @@ static int xa_launch(const void* X, const void* U, int64_t ldx, void* act_out, c
 }
 
 template <typename T>
-static int xa_impl(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out,
+static int xa_impl(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out, int mask_bits,
                    uint64_t seed, void* S, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
   const int nblk = n_row_blocks(M, seg);
   const int64_t rows = seg.table ? (int64_t)nblk * ROWS : M;
   switch (rt_of(R)) {
-    case 1: return xa_launch<T, 1>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, rows, seg, st);
-    case 2: return xa_launch<T, 2>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, rows, seg, st);
-    case 4: return xa_launch<T, 4>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, rows, seg, st);
-    default: return xa_launch<T, 8>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, rows, seg, st);
+    case 1: return xa_launch<T, 1>(X, U, ldx, act_out, mask, mask_out, mask_bits, seed, S, M, K, R, rows, seg, st);
+    case 2: return xa_launch<T, 2>(X, U, ldx, act_out, mask, mask_out, mask_bits, seed, S, M, K, R, rows, seg, st);
+    case 4: return xa_launch<T, 4>(X, U, ldx, act_out, mask, mask_out, mask_bits, seed, S, M, K, R, rows, seg, st);
+    default: return xa_launch<T, 8>(X, U, ldx, act_out, mask, mask_out, mask_bits, seed, S, M, K, R, rows, seg, st);
   }
 }
 
 // mask_out != nullptr: draw the keep-mask from `seed` (written to mask_out [rows, K]) instead of reading `mask`.
 // U != nullptr: X and U are the gate and up halves (rows ldx elements apart) and the pass's input
 // round16(round16(silu(X)) * U) is written to act_out [rows, K]; otherwise X [rows, K] is dense.
-int lf_launch_xa(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out,
+int lf_launch_xa(const void* X, const void* U, int64_t ldx, void* act_out, const uint8_t* mask, uint8_t* mask_out, int mask_bits,
                  uint64_t seed, void* S, int M, int K, int R, const LfSegTable& seg, int dtype, hipStream_t st) {
   if (!X || !S || M <= 0 || K <= 0) return LF_EINVAL;
   if (K % 128 != 0 || R % 16 != 0 || R <= 0 || R > LF_MAX_RANK) return LF_ESHAPE;
   if (seg.table && seg.block_size_m != ROWS) return LF_ESHAPE;
-  if (mask_out != nullptr && ((uintptr_t)mask_out & 7) != 0) return LF_ESHAPE;
+  if (mask_out != nullptr && ((uintptr_t)mask_out & (mask_bits ? 3 : 7)) != 0) return LF_ESHAPE;
   if (U != nullptr) {
     if (!act_out) return LF_EINVAL;
     if (ldx < K || ldx % 8 != 0 || (((uintptr_t)X | (uintptr_t)U | (uintptr_t)act_out) & 15) != 0) return LF_ESHAPE;
   } else {
     ldx = K;
   }
-  if (dtype == LF_BF16) return xa_impl<__bf16>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, seg, st);
-  if (dtype == LF_F16) return xa_impl<_Float16>(X, U, ldx, act_out, mask, mask_out, seed, S, M, K, R, seg, st);
+  if (dtype == LF_BF16) return xa_impl<__bf16>(X, U, ldx, act_out, mask, mask_out, mask_bits, seed, S, M, K, R, seg, st);
+  if (dtype == LF_F16) return xa_impl<_Float16>(X, U, ldx, act_out, mask, mask_out, mask_bits, seed, S, M, K, R, seg, st);
   return LF_EINVAL;
 }
 
@@ -1411,18 +1447,18 @@ static void da_shape(int M, int K, int R, const LfSegTable& seg, int& group, int
 // Ring kernel shapes by rank tiles: tiles per slice (registers: TPW * RT * 4 accumulators) and ring depth (LDS: NS
 // stages of 16 KB, 24 KB with a keep-mask, plus two dS blocks of RT * 4 KB; two workgroups per CU where that fits).
 constexpr int da_tpw(int rt) { return rt >= 4 ? 8 : 16; }
-constexpr int da_ns(int rt, bool masked) { return masked ? (rt == 1 ? 3 : 5) : (rt == 4 ? 3 : 4); }
-static int da_ring_smem(int rt, bool masked) { return da_ns(rt, masked) * (TILE_BYTES + (masked ? ROWS * 64 : 0)) + 2 * ROWS * rt * 32; }
+constexpr int da_ns(int rt, int maskfmt) { return maskfmt ? (rt == 1 ? 3 : 5) : (rt == 4 ? 3 : 4); }
+static int da_ring_smem(int rt, int maskfmt) { return da_ns(rt, maskfmt) * (TILE_BYTES + da_mask_tile_bytes(maskfmt)) + 2 * ROWS * rt * 32; }
 struct DaPlan { int n_slices, group, max_chunks; };
 // Slices of the K axis (balanced, 2 .. TPW tiles each) x chunks of `group` row blocks per segment, by bytes moved: the
 // X stream in whole rounds of resident workgroups, the dS blocks every workgroup fetches, and the fp32 partials
 // (one [R, K] slab per chunk, written here and read by the reduce).
-static DaPlan da_plan(int M, int K, int R, bool masked, const LfSegTable& seg) {
+static DaPlan da_plan(int M, int K, int R, int maskfmt, const LfSegTable& seg) {
   const int rt = rt_of(R), T = K / 64;
   int blocks[LF_MAX_SEG], nseg;
   seg_block_counts(M, seg, blocks, nseg);
-  const int slots = lds_slots(da_ring_smem(rt, masked));
-  const double tile_bytes = TILE_BYTES + (masked ? ROWS * 64 : 0);
+  const int slots = lds_slots(da_ring_smem(rt, maskfmt));
+  const double tile_bytes = TILE_BYTES + da_mask_tile_bytes(maskfmt);
   DaPlan best{1, 1, 1};
   if (T < 2) return best;   // as in dysr_plan
   double best_cost = 1e300;
@@ -1442,9 +1478,10 @@ size_t lf_da_workspace(int M, int K, int R, const LfSegTable& seg) {
   const int nseg = seg.table ? seg.n_seg : 1;
   int max_chunks;
   if (rt_of(R) <= 4) {
-    // the launch plans with or without a keep-mask: room for either
-    const int a = da_plan(M, K, R, true, seg).max_chunks, b = da_plan(M, K, R, false, seg).max_chunks;
+    // the launch plans with or without a keep-mask (one byte or one bit per element): room for any
+    const int a = da_plan(M, K, R, 1, seg).max_chunks, b = da_plan(M, K, R, 0, seg).max_chunks, c = da_plan(M, K, R, 2, seg).max_chunks;
     max_chunks = a > b ? a : b;
+    max_chunks = c > max_chunks ? c : max_chunks;
   } else {
     int group;
     da_shape(M, K, R, seg, group, max_chunks);
@@ -1453,17 +1490,17 @@ size_t lf_da_workspace(int M, int K, int R, const LfSegTable& seg) {
 }
 
 template <typename T, int RT>
-static int da_launch(const void* X, const uint8_t* mask, const void* dS, float* part, int M, int K, int R, int group,
+static int da_launch(const void* X, const uint8_t* mask, int mask_bits, const void* dS, float* part, int M, int K, int R, int group,
                      int max_chunks, dim3 grid, const LfSegTable& seg, hipStream_t st) {
   auto kern = lora_da_kernel<T, RT>;
   constexpr int RP = RT * 32 + 32;
   const int smem = 2 * TILE_BYTES + 2 * ROWS * RP;
   static LfLdsFlags lds_ok;
   if (!lf_allow_lds(kern, smem, lds_ok)) return LF_ELAUNCH;
-  return lf_launch(kern, grid, dim3(256), smem, st, (const T*)X, mask, (const T*)dS, part, M, K, R, group, max_chunks, seg);
+  return lf_launch(kern, grid, dim3(256), smem, st, (const T*)X, mask, mask_bits, (const T*)dS, part, M, K, R, group, max_chunks, seg);
 }
 
-template <typename T, int RT, bool MASK>
+template <typename T, int RT, int MASK>
 static int da_ring_launch(const void* X, const uint8_t* mask, const void* dS, float* part, int M, int K, int R, const DaPlan& pl,
                           int nseg, const LfSegTable& seg, hipStream_t st) {
   auto kern = lora_da_ring_kernel<T, RT, da_tpw(RT), da_ns(RT, MASK), MASK>;
@@ -1475,30 +1512,28 @@ static int da_ring_launch(const void* X, const uint8_t* mask, const void* dS, fl
 }
 
 template <typename T>
-static int da_impl(const void* X, const uint8_t* mask, const void* dS, void* ws, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
+static int da_impl(const void* X, const uint8_t* mask, int mask_bits, const void* dS, void* ws, int M, int K, int R, const LfSegTable& seg, hipStream_t st) {
   const int nseg = seg.table ? seg.n_seg : 1;
   float* part = (float*)ws;
   int group, max_chunks, rc;
   if (rt_of(R) <= 4) {
-    const DaPlan pl = da_plan(M, K, R, mask != nullptr, seg);
+    const int fmt = mask == nullptr ? 0 : mask_bits ? 2 : 1;
+    const DaPlan pl = da_plan(M, K, R, fmt, seg);
     group = pl.group;
     max_chunks = pl.max_chunks;
-    if (mask != nullptr) {
-      switch (rt_of(R)) {
-        case 1: rc = da_ring_launch<T, 1, true>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
-        case 2: rc = da_ring_launch<T, 2, true>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
-        default: rc = da_ring_launch<T, 4, true>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
-      }
-    } else {
-      switch (rt_of(R)) {
-        case 1: rc = da_ring_launch<T, 1, false>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
-        case 2: rc = da_ring_launch<T, 2, false>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
-        default: rc = da_ring_launch<T, 4, false>(X, mask, dS, part, M, K, R, pl, nseg, seg, st); break;
-      }
+#define LF_DA_RING(RTV)                                                                                                   \
+  rc = fmt == 2   ? da_ring_launch<T, RTV, 2>(X, mask, dS, part, M, K, R, pl, nseg, seg, st)                              \
+       : fmt == 1 ? da_ring_launch<T, RTV, 1>(X, mask, dS, part, M, K, R, pl, nseg, seg, st)                              \
+                  : da_ring_launch<T, RTV, 0>(X, mask, dS, part, M, K, R, pl, nseg, seg, st)
+    switch (rt_of(R)) {
+      case 1: LF_DA_RING(1); break;
+      case 2: LF_DA_RING(2); break;
+      default: LF_DA_RING(4); break;
     }
+#undef LF_DA_RING
   } else {
     da_shape(M, K, R, seg, group, max_chunks);
-    rc = da_launch<T, 8>(X, mask, dS, part, M, K, R, group, max_chunks, dim3(K / 64, max_chunks, nseg), seg, st);
+    rc = da_launch<T, 8>(X, mask, mask_bits, dS, part, M, K, R, group, max_chunks, dim3(K / 64, max_chunks, nseg), seg, st);
   }
   if (rc != LF_OK) return rc;
   int maxrank = 0;
@@ -1507,7 +1542,7 @@ static int da_impl(const void* X, const uint8_t* mask, const void* dS, void* ws,
   return lf_launch((reduce_segments_kernel<T>), dim3((unsigned)((nout + 1023) / 1024), nseg), dim3(256), 0, st, (const float*)part, K, R, 1, mask != nullptr ? 1 : 2, M, group, max_chunks, seg);
 }
 
-int lf_launch_da(const void* X, const uint8_t* mask, const void* dS, void* ws, size_t ws_bytes, int M, int K, int R,
+int lf_launch_da(const void* X, const uint8_t* mask, int mask_bits, const void* dS, void* ws, size_t ws_bytes, int M, int K, int R,
                  const LfSegTable& seg, int dtype, hipStream_t st) {
   if (!X || !dS || M <= 0 || K <= 0) return LF_EINVAL;
   if (K % 128 != 0 || R % 16 != 0 || R <= 0 || R > LF_MAX_RANK) return LF_ESHAPE;
@@ -1516,8 +1551,9 @@ int lf_launch_da(const void* X, const uint8_t* mask, const void* dS, void* ws, s
   for (int s = 0; s < nseg; s++) if (!seg.out[s] || seg.rank[s] % 8 != 0 || seg.rank[s] > R) return LF_EINVAL;
   for (int s = 0; s < nseg; s++) if (((uintptr_t)seg.out[s] & 7) != 0) return LF_ESHAPE;  // 8-byte stores of dA
   if (!ws || ws_bytes < lf_da_workspace(M, K, R, seg)) return LF_EWORKSPACE;
-  if (dtype == LF_BF16) return da_impl<__bf16>(X, mask, dS, ws, M, K, R, seg, st);
-  if (dtype == LF_F16) return da_impl<_Float16>(X, mask, dS, ws, M, K, R, seg, st);
+  if (mask != nullptr && mask_bits && ((uintptr_t)mask & 3) != 0) return LF_ESHAPE;   // 4-byte loads of the keep bits
+  if (dtype == LF_BF16) return da_impl<__bf16>(X, mask, mask_bits, dS, ws, M, K, R, seg, st);
+  if (dtype == LF_F16) return da_impl<_Float16>(X, mask, mask_bits, dS, ws, M, K, R, seg, st);
   return LF_EINVAL;
 }
 

@@ -32,15 +32,53 @@ def _check_2d(t: torch.Tensor, name: str, dtype: torch.dtype | None = None) -> N
 
 
 def _check_mask(mask: torch.Tensor | None, shape, name: str = "dropout_mask") -> torch.Tensor | None:
+    """A keep-mask for a ``shape = (M, K)`` input: bool / uint8 ``[M, K]`` (one byte per element, the reference's
+    format) or uint8 ``[M, K // 8]`` (bit-packed: element k of a row = bit k & 7 of byte k >> 3; ``pack_mask``)."""
     if mask is None:
         return None
     if mask.dtype not in (torch.bool, torch.uint8):
         raise ValueError(f"{name} must be a bool (or uint8) tensor, but got {mask.dtype}.")
-    if tuple(mask.shape) != tuple(shape):
+    M, K = tuple(shape)
+    if tuple(mask.shape) != (M, K) and not (mask.dtype == torch.uint8 and tuple(mask.shape) == (M, K // 8)):
         raise ValueError(f"{name} must have shape {tuple(shape)}, but got {tuple(mask.shape)}.")
     if not mask.is_contiguous():
         raise ValueError(f"{name} must be contiguous.")
     L.require_gpu(mask, name)
+    return mask
+
+
+def _dt(t: torch.Tensor, mask: torch.Tensor | None, K: int) -> int:
+    """The C ABI's dtype argument of a call whose keep-mask is ``mask``: the element type, plus the flag that says
+    the mask is bit-packed (told apart by its row length: K // 8 bytes instead of K)."""
+    bits = mask is not None and mask.shape[-1] * 8 == K and mask.dtype == torch.uint8
+    return L.dtype_id(t.dtype) | (L.LF_MASK_BITS if bits else 0)
+
+
+def is_packed_mask(mask: torch.Tensor | None, K: int) -> bool:
+    return mask is not None and mask.dtype == torch.uint8 and mask.shape[-1] * 8 == K
+
+
+def pack_mask(mask: torch.Tensor) -> torch.Tensor:
+    """bool / uint8 ``[M, K]`` keep-mask -> bit-packed uint8 ``[M, K // 8]`` (K % 128 == 0), on the GPU."""
+    if mask.ndim != 2 or mask.dtype not in (torch.bool, torch.uint8) or not mask.is_contiguous():
+        raise ValueError("pack_mask takes a contiguous 2D bool (or uint8) tensor.")
+    L.require_gpu(mask, "mask")
+    M, K = mask.shape
+    _check_dims(M, None, K)
+    bits = torch.empty((M, K // 8), dtype=torch.uint8, device=mask.device)
+    L.check(L.lib().lf_mask_pack(L.ptr(mask), L.ptr(bits), M, K, L.stream_of(mask)), "lf_mask_pack")
+    return bits
+
+
+def unpack_mask(bits: torch.Tensor) -> torch.Tensor:
+    """bit-packed uint8 ``[M, K // 8]`` -> bool ``[M, K]``."""
+    if bits.ndim != 2 or bits.dtype != torch.uint8 or not bits.is_contiguous():
+        raise ValueError("unpack_mask takes a contiguous 2D uint8 tensor.")
+    L.require_gpu(bits, "bits")
+    M, K = bits.shape[0], bits.shape[1] * 8
+    _check_dims(M, None, K)
+    mask = torch.empty((M, K), dtype=torch.bool, device=bits.device)
+    L.check(L.lib().lf_mask_unpack(L.ptr(bits), L.ptr(mask), M, K, L.stream_of(bits)), "lf_mask_unpack")
     return mask
 
 
@@ -122,7 +160,7 @@ def _xa(x, mask, a_list, routing, M, K, R):
     s = torch.empty((M, R), dtype=x.dtype, device=x.device)
     ws, nbytes = _ws(L.LF_OP_XA, M, 0, K, R, routing, x.device)
     rc = L.lib().lf_lora_xa(L.ptr(x), L.ptr(mask), L.ptr_array(a_list), L.ptr(s), L.ptr(ws), nbytes, M, K, R,
-                            routing, L.dtype_id(x.dtype), L.stream_of(x))
+                            routing, _dt(x, mask, K), L.stream_of(x))
     L.check(rc, "lf_lora_xa")
     return s
 
@@ -228,7 +266,8 @@ def fused_dropout_matmul(x: torch.Tensor, a: torch.Tensor, dropout_p: float, see
     s = _xa(x, mask, [a], routing, M, K, L.round_rank(r))
     xs = None
     if store_masked_scaled_x:
-        xs = x if mask is None else torch.where(mask, x * (1.0 / (1.0 - dropout_p)), torch.zeros((), dtype=x.dtype, device=x.device))
+        mb = unpack_mask(mask) if is_packed_mask(mask, K) else mask
+        xs = x if mask is None else torch.where(mb, x * (1.0 / (1.0 - dropout_p)), torch.zeros((), dtype=x.dtype, device=x.device))
     return s, (mask if store_mask else None), xs
 
 
@@ -317,7 +356,7 @@ def fused_lora_da(x: torch.Tensor, ds: torch.Tensor, r: int, dropout_p: float = 
     ws, nbytes = _ws(L.LF_OP_DA, M, 0, K, R, routing, x.device)
     ds_p = _pad_cols(ds, R)
     rc = L.lib().lf_lora_da(L.ptr(x), L.ptr(mask), L.ptr(ds_p), L.ptr_array([da]), L.ptr(ws), nbytes,
-                            M, K, R, routing, L.dtype_id(x.dtype), L.stream_of(x))
+                            M, K, R, routing, _dt(x, mask, K), L.stream_of(x))
     L.check(rc, "lf_lora_da")
     return da
 
@@ -345,7 +384,7 @@ def fused_lora_dyw_dsa(dy: torch.Tensor, w: torch.Tensor, ds: torch.Tensor, a: t
     dx = torch.empty((M, K), dtype=dy.dtype, device=dy.device)
     ds_p = _pad_cols(ds, R)
     rc = L.lib().lf_lora_dyw_dsa(L.ptr(dy), L.ptr(w), L.ptr(ds_p), L.ptr_array([a]), L.ptr(mask), L.ptr(dx),
-                                 M, N, K, R, routing, L.dtype_id(dy.dtype), L.stream_of(dy))
+                                 M, N, K, R, routing, _dt(dy, mask, K), L.stream_of(dy))
     L.check(rc, "lf_lora_dyw_dsa")
     return dx
 
@@ -429,7 +468,7 @@ def fused_multi_lora_da(x, ds, routing: MultiRouting, dropout_mask=None):
     da_list = [torch.empty((r, K), dtype=x.dtype, device=x.device) for r in routing.rank_list]
     ws, nbytes = _ws(L.LF_OP_DA, M, 0, K, routing.R, routing.c, x.device)
     rc = L.lib().lf_lora_da(L.ptr(x), L.ptr(mask), L.ptr(ds), L.ptr_array(da_list), L.ptr(ws), nbytes, M, K,
-                            routing.R, routing.c, L.dtype_id(x.dtype), L.stream_of(x))
+                            routing.R, routing.c, _dt(x, mask, K), L.stream_of(x))
     L.check(rc, "lf_lora_da")
     return da_list
 
@@ -448,7 +487,7 @@ def fused_multi_lora_dyw_dsa(dy, w, ds, a_list, routing: MultiRouting, dropout_m
     mask = _check_mask(dropout_mask, (M, K))
     dx = torch.empty((M, K), dtype=dy.dtype, device=dy.device)
     rc = L.lib().lf_lora_dyw_dsa(L.ptr(dy), L.ptr(w), L.ptr(ds), L.ptr_array(a_list), L.ptr(mask), L.ptr(dx), M, N, K,
-                                 routing.R, routing.c, L.dtype_id(dy.dtype), L.stream_of(dy))
+                                 routing.R, routing.c, _dt(dy, mask, K), L.stream_of(dy))
     L.check(rc, "lf_lora_dyw_dsa")
     return dx
 
@@ -464,23 +503,24 @@ def lora_forward(x, w, a_list, b_list, routing_c, R, mask, bias):
     s = torch.empty((M, R), dtype=x.dtype, device=x.device)
     ws, nbytes = _ws(L.LF_OP_FWD, M, N, K, R, routing_c, x.device)
     rc = L.lib().lf_lora_fwd(L.ptr(x), L.ptr(w), L.ptr(bias), L.ptr(mask), L.ptr_array(a_list), L.ptr_array(b_list),
-                             L.ptr(y), L.ptr(s), L.ptr(ws), nbytes, M, N, K, R, routing_c, L.dtype_id(x.dtype),
+                             L.ptr(y), L.ptr(s), L.ptr(ws), nbytes, M, N, K, R, routing_c, _dt(x, mask, K),
                              L.stream_of(x))
     L.check(rc, "lf_lora_fwd")
     return y, s
 
 
-def lora_forward_seeded(x, w, a_list, b_list, routing_c, R, seed: int, bias):
+def lora_forward_seeded(x, w, a_list, b_list, routing_c, R, seed: int, bias, *, packed: bool = True):
     """As ``lora_forward`` with the keep-mask drawn inside the rank-r kernel from ``seed``.
-    Returns (y, s, mask); the mask equals ``make_dropout_mask`` for the same seed and routing."""
+    Returns (y, s, mask).  The mask comes back bit-packed (uint8 ``[M, K // 8]``, the format the backward kernels read
+    fastest; ``packed=False``: bool ``[M, K]``); unpacked it equals ``make_dropout_mask`` for the same seed and routing."""
     M, K = x.shape
     N = w.shape[0]
     y = torch.empty((M, N), dtype=x.dtype, device=x.device)
     s = torch.empty((M, R), dtype=x.dtype, device=x.device)
-    mask = torch.empty((M, K), dtype=torch.bool, device=x.device)
+    mask = torch.empty((M, K // 8), dtype=torch.uint8, device=x.device) if packed else torch.empty((M, K), dtype=torch.bool, device=x.device)
     rc = L.lib().lf_lora_fwd_seeded(L.ptr(x), L.ptr(w), L.ptr(bias), L.ptr(mask), L.ptr_array(a_list), L.ptr_array(b_list),
                                     L.ptr(y), L.ptr(s), M, N, K, R, routing_c, ctypes.c_uint64(int(seed) & 0xFFFFFFFFFFFFFFFF),
-                                    L.dtype_id(x.dtype), L.stream_of(x))
+                                    _dt(x, mask, K), L.stream_of(x))
     L.check(rc, "lf_lora_fwd_seeded")
     return y, s, mask
 
@@ -496,7 +536,7 @@ def lora_backward(dy, x, w, a_list, b_list, s, routing_c, R, mask, rank_list, re
     ws, nbytes = _ws(L.LF_OP_BWD, M, N, K, R, routing_c, dy.device)
     rc = L.lib().lf_lora_bwd(L.ptr(dy), L.ptr(x), L.ptr(w), L.ptr(mask), L.ptr(s), L.ptr_array(a_list),
                              L.ptr_array(b_list), L.ptr(dx), L.ptr_array(da_list), L.ptr_array(db_list), L.ptr(ds),
-                             L.ptr(ws), nbytes, M, N, K, R, routing_c, L.dtype_id(dy.dtype), L.stream_of(dy))
+                             L.ptr(ws), nbytes, M, N, K, R, routing_c, _dt(dy, mask, K), L.stream_of(dy))
     L.check(rc, "lf_lora_bwd")
     return dx, da_list, db_list
 
@@ -515,7 +555,7 @@ def nf4_lora_forward(x, wref, a_list, b_list, routing_c, R, mask, bias, *, keep_
     ws, nbytes = _ws(L.LF_OP_FWD if keep_dense else L.LF_OP_NF4_FWD, M, N, K, R, routing_c, x.device)
     rc = L.lib().lf_nf4_lora_fwd(L.ptr(x), ctypes.byref(wc), L.ptr(bias), L.ptr(mask), L.ptr_array(a_list),
                                  L.ptr_array(b_list), L.ptr(y), L.ptr(s), L.ptr(ws), nbytes, M, N, K, R, routing_c,
-                                 L.dtype_id(x.dtype), L.stream_of(x))
+                                 _dt(x, mask, K), L.stream_of(x))
     L.check(rc, "lf_nf4_lora_fwd")
     return (y, s, dense) if keep_dense else (y, s)
 
@@ -538,7 +578,7 @@ def nf4_lora_backward(dy, x, wref, a_list, b_list, s, routing_c, R, mask, rank_l
     ws, nbytes = _ws(L.LF_OP_BWD if lean else L.LF_OP_NF4_BWD, M, N, K, R, routing_c, dy.device)
     rc = L.lib().lf_nf4_lora_bwd(L.ptr(dy), L.ptr(x), ctypes.byref(wc), L.ptr(mask), L.ptr(s), L.ptr_array(a_list),
                                  L.ptr_array(b_list), L.ptr(dx), L.ptr_array(da_list), L.ptr_array(db_list), L.ptr(ds),
-                                 L.ptr(ws), nbytes, M, N, K, R, routing_c, L.dtype_id(dy.dtype), L.stream_of(dy))
+                                 L.ptr(ws), nbytes, M, N, K, R, routing_c, _dt(dy, mask, K), L.stream_of(dy))
     L.check(rc, "lf_nf4_lora_bwd")
     return dx, da_list, db_list
 

@@ -82,7 +82,9 @@ class FusedLinearLoRA(torch.autograd.Function):
             y, s, mask = hip_ops.lora_forward_seeded(x2d, linear_w, [lora_a], [lora_b], routing, R, seed, bias)
         else:
             if dropout_p > 0:
-                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+                mask = hip_ops._check_mask(dropout_mask.reshape(M, -1), (M, K))
+                if not hip_ops.is_packed_mask(mask, K):
+                    mask = hip_ops.pack_mask(mask)   # read three times (rank-r forward, dA, dX): an eighth of the bytes each
             routing = L.single_routing(r, alpha, dropout_p if mask is not None else 0.0)
             y, s = hip_ops.lora_forward(x2d, linear_w, [lora_a], [lora_b], routing, R, mask, bias)
 

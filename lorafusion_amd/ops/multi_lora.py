@@ -241,7 +241,9 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
             if routing.enable_dropout:
                 if dropout_mask is None:
                     dropout_mask = hip_ops.make_dropout_mask((M, K), 0.0, seed, x2d.device, routing=routing)
-                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+                mask = hip_ops._check_mask(dropout_mask.reshape(M, -1), (M, K))
+                if not hip_ops.is_packed_mask(mask, K):
+                    mask = hip_ops.pack_mask(mask)   # read three times (rank-r forward, dA, dX): an eighth of the bytes each
             if keep_dequantized:
                 y, s, dense = hip_ops.nf4_lora_forward(x2d, wref, a_list, b_list, routing.c, routing.R, mask, bias,
                                                        keep_dense=True)
@@ -254,7 +256,9 @@ class FusedLinearMultiLoRA(torch.autograd.Function):
             y, s, mask = hip_ops.lora_forward_seeded(x2d, linear_w, a_list, b_list, routing.c, routing.R, seed, bias)
         else:
             if routing.enable_dropout:
-                mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+                mask = hip_ops._check_mask(dropout_mask.reshape(M, -1), (M, K))
+                if not hip_ops.is_packed_mask(mask, K):
+                    mask = hip_ops.pack_mask(mask)   # read three times (rank-r forward, dA, dX): an eighth of the bytes each
             y, s = hip_ops.lora_forward(x2d, linear_w, a_list, b_list, routing.c, routing.R, mask, bias)
 
         ctx.save_for_backward(x2d, linear_w, mask, s, dense, *a_list, *b_list)

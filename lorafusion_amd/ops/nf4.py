@@ -211,7 +211,9 @@ class FusedLinearLoRANF4(torch.autograd.Function):
         if dropout_p > 0:
             if dropout_mask is None:
                 dropout_mask = hip_ops.make_dropout_mask((M, K), dropout_p, seed, x2d.device)
-            mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+            mask = hip_ops._check_mask(dropout_mask.reshape(M, -1), (M, K))
+            if not hip_ops.is_packed_mask(mask, K):
+                mask = hip_ops.pack_mask(mask)   # read three times (rank-r forward, dA, dX): an eighth of the bytes each
         p_eff = dropout_p if mask is not None else 0.0
         routing = L.single_routing(r, alpha, p_eff)
         dense = None

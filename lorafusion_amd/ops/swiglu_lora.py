@@ -31,11 +31,11 @@ def _swiglu_lora_forward(gate, up, ld, w, a_list, b_list, routing_c, R, mask, dr
     s = torch.empty((M, R), dtype=gate.dtype, device=gate.device)
     mask_out = None
     if draw_seed is not None:
-        mask_out = torch.empty((M, K), dtype=torch.bool, device=gate.device)
+        mask_out = torch.empty((M, K // 8), dtype=torch.uint8, device=gate.device)   # drawn masks are kept bit-packed
     rc = L.lib().lf_swiglu_lora_fwd(
         gate.data_ptr(), up.data_ptr(), ld, x.data_ptr(), L.ptr(w), L.ptr(bias), L.ptr(mask), L.ptr(mask_out),
         ctypes.c_uint64(int(draw_seed or 0) & 0xFFFFFFFFFFFFFFFF), L.ptr_array(a_list), L.ptr_array(b_list), y.data_ptr(),
-        s.data_ptr(), M, N, K, R, routing_c, L.dtype_id(gate.dtype), L.stream_of(gate))
+        s.data_ptr(), M, N, K, R, routing_c, hip_ops._dt(gate, mask_out if mask_out is not None else mask, K), L.stream_of(gate))
     L.check(rc, "lf_swiglu_lora_fwd")
     return x, y, s, (mask_out if mask_out is not None else mask)
 
@@ -104,7 +104,9 @@ class FusedSwiGLULinearLoRA(torch.autograd.Function):
         if dropout and dropout_mask is None:
             draw = seed if seed is not None else random.randrange(int(1e6))  # noqa: S311
         elif dropout:
-            mask = hip_ops._check_mask(dropout_mask.reshape(M, K), (M, K))
+            mask = hip_ops._check_mask(dropout_mask.reshape(M, -1), (M, K))
+            if not hip_ops.is_packed_mask(mask, K):
+                mask = hip_ops.pack_mask(mask)   # read three times (rank-r forward, dA, dX): an eighth of the bytes each
         p_used = dropout_p if dropout else 0.0
         routing_c = routing.c if routing is not None else L.single_routing(rank_list[0], alpha, p_used)
         x, y, s, mask = _swiglu_lora_forward(gv, uv, ld, linear_w, a_list, b_list, routing_c, R, mask, draw, bias)

@@ -112,7 +112,11 @@ def test_seeded_forward_draws_the_oracle_mask(ranks):
     M = x.shape[0]
     row_p = np.repeat(info.block_to_dropout_p.float().cpu().numpy(), 128)
     expect = od.keep_mask(M, K, row_p, seed)
-    assert np.array_equal(mask.cpu().numpy().astype(np.uint8), expect)
+    assert mask.dtype == torch.uint8 and tuple(mask.shape) == (M, K // 8)      # drawn masks come back bit-packed
+    assert np.array_equal(mask.cpu().numpy(), np.packbits(expect, axis=1, bitorder="little"))
+    assert np.array_equal(hip_ops.unpack_mask(mask).cpu().numpy().astype(np.uint8), expect)
+    y1, s1, mask1 = hip_ops.lora_forward_seeded(x, w, a_list, b_list, routing.c, routing.R, seed, None, packed=False)
+    assert np.array_equal(mask1.cpu().numpy().astype(np.uint8), expect) and torch.equal(s, s1) and torch.equal(y, y1)
     y2, s2 = hip_ops.lora_forward(x, w, a_list, b_list, routing.c, routing.R, torch.from_numpy(expect).bool().cuda(), None)
     assert torch.equal(s, s2) and torch.equal(y, y2)
 
