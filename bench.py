@@ -2,9 +2,12 @@
 """Benchmark of the fused LoRA-linear hot path on one MI355X.
 
 Headline workload (the configuration the metric names: "8B layer, r=16"): the seven LoRA projections of a
-Llama-3-8B-shaped decoder layer -- hidden 4096, kv 1024, MLP 14336 -- run the way the reference's layer runs
-them, as four LoRA linears (q/k/v merged into one N=6144 linear, gate/up merged into one N=28672 linear,
-lorafusion/patch/patch_transformers.py:50-163): 16384 packed tokens of 4 adapters (rank 16, multipliers
+Llama-3-8B-shaped decoder layer -- hidden 4096, kv 1024, MLP 14336 -- as four LoRA linears: q/k/v merged into one
+N=6144 linear, which is what the reference's layer does (lorafusion/patch/patch_transformers.py:50-163, 278-287), and
+gate/up merged likewise into one N=28672 linear, which the reference does not do (a merged gate/up adapter shares one
+A between the two halves).  The same layer with only q/k/v merged (`workloads.c4_qkv_merged`, the reference's own
+layer: five linears) and as seven separate linears (`workloads.c4_separate`, BASELINE's wording) is measured next to
+it.  16384 packed tokens of 4 adapters (rank 16, multipliers
 {1,2,2,4}, dropout {0,.05,.1,.1}, lognormal segment lengths up to 8192), each adapter padded to 128 rows,
 bf16, training mode (dropout masks drawn in the rank-r pass), forward + backward (dX, dA_i, dB_i).  The
 micro-batch comes in as a scheduler descriptor, goes through the MultiLoRAManager, and every linear is
@@ -50,6 +53,11 @@ WORKLOADS = {
     "c3": (4096, 1, 16, [2.0], [0.0], True, 4096, [("linear", 4096, 14336)]),
     "c4": (16384, 4, 16, [1.0, 2.0, 2.0, 4.0], [0.0, 0.05, 0.1, 0.1], False, 8192,
            [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]),
+    "c4_qkv_merged": (16384, 4, 16, [1.0, 2.0, 2.0, 4.0], [0.0, 0.05, 0.1, 0.1], False, 8192,
+                      [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate", 4096, 14336), ("up", 4096, 14336), ("down", 14336, 4096)]),
+    "c4_separate": (16384, 4, 16, [1.0, 2.0, 2.0, 4.0], [0.0, 0.05, 0.1, 0.1], False, 8192,
+                    [("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024), ("o", 4096, 4096), ("gate", 4096, 14336),
+                     ("up", 4096, 14336), ("down", 14336, 4096)]),
     "c5": (8192, 8, 64, [1.0, 2.0, 2.0, 4.0] * 2, [0.0, 0.05, 0.1, 0.1] * 2, True, 4096,
            [("qkv", 8192, 10240), ("o", 8192, 8192), ("gate_up", 8192, 57344), ("down", 28672, 8192)]),
     "c5_separate": (8192, 8, 64, [1.0, 2.0, 2.0, 4.0] * 2, [0.0, 0.05, 0.1, 0.1] * 2, True, 4096,
@@ -65,6 +73,11 @@ NAMES = {
           "linears of the merged layer (qkv N=6144, o, gate+up N=28672, down), 16384 packed tokens, 4 adapters r=16, "
           "training-mode dropout drawn in the rank-r pass, fwd+bwd, driven by a micro-batch descriptor through the "
           "patched layer; attention, rotary embedding, norms and activation are not part of the path and not run",
+    "c4_qkv_merged": "the same 8B-class layer the way the reference's patched layer runs it: q/k/v merged into one N=6144 "
+                     "linear, o, gate, up and down on their own (five LoRA linears), 16384 packed tokens, 4 adapters r=16, "
+                     "explicit bit-packed masks through the raw ops, fwd+bwd",
+    "c4_separate": "the same 8B-class layer as seven separate LoRA linears (q, k, v, o, gate, up, down), 16384 packed tokens, "
+                   "4 adapters r=16, explicit bit-packed masks through the raw ops, fwd+bwd",
     "c5": "the seven LoRA projections of a 70B-class decoder layer (hidden 8192, kv 1024, MLP 28672) as the four LoRA "
           "linears of the merged layer (qkv N=10240, o, gate+up N=57344, down) with NF4 base weights (dequantised "
           "inside every call), 8192 packed tokens, 8 adapters r=64, explicit masks, fwd+bwd; attention, norms and "
@@ -180,6 +193,7 @@ class Linear:
     """Device tensors of one LoRA linear of a workload and its raw (autograd-free) forward + backward."""
 
     def __init__(self, batch: Batch, name: str, k: int, n: int, g, dev):
+        from lorafusion_amd.ops import hip_ops
         from lorafusion_amd.ops.nf4 import NF4WeightRef, quantize_nf4
 
         b = self.batch = batch
@@ -189,7 +203,8 @@ class Linear:
         w = (torch.randn(n, k, generator=g, device=dev) * 0.02).to(torch.bfloat16)
         self.a = [((torch.rand(b.rank, k, generator=g, device=dev) * 2 - 1) / k ** 0.5).to(torch.bfloat16) for _ in range(b.n_ad)]
         self.b = [(torch.randn(n, b.rank, generator=g, device=dev) * 0.01).to(torch.bfloat16) for _ in range(b.n_ad)]
-        self.mask = (torch.rand(b.Mp, k, generator=g, device=dev) >= b.row_p[:, None]) if b.dropout else None
+        # explicit keep-mask, bit-packed (the library's own format for masks it draws; lf_mask_pack converts a bool tensor)
+        self.mask = hip_ops.pack_mask(torch.rand(b.Mp, k, generator=g, device=dev) >= b.row_p[:, None]) if b.dropout else None
         self.wref = None
         if b.nf4:
             self.packed, self.qs = quantize_nf4(w.float())
@@ -281,6 +296,9 @@ def kernel_breakdown(linears, reps: int):
     }
     t = {k: round(v, 4) for k, v in t.items()}
     overhead = (t["xa"] + t["gemm_fwd"] + t["dys_dyb"] + t["da"] + t["gemm_bwd"]) / (t["plain_gemm_nt"] + t["plain_gemm_nn"]) - 1.0
+    roofline["lora_overhead_vs_plain_gemms"] = round(overhead, 4)
+    roofline["plain_gemm_same_shapes_frac"] = round(
+        sum(2.0 * lin.batch.Mp * lin.k * lin.n for lin in linears) / (t["plain_gemm_nn"] * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4)
     return t, roofline, round(overhead, 4)
 
 
@@ -356,22 +374,81 @@ def raw_workload(name: str, args, dev, breakdown: bool = True) -> dict:
     return res
 
 
-def nf4_dequant_block(dev) -> dict:
-    """Standalone NF4 dequant of W[14336,4096], blocksize 64, double quantised: 2.516 B/element."""
+def nf4_dequant_block(dev, shape=(14336, 4096), fill: bool = False) -> dict:
+    """Standalone NF4 dequant of W[shape], blocksize 64, double quantised: 2.516 B/element.  `fill`: also time a plain
+    fill of the output tensor (torch's fill kernel: stores only), the reference point for what the write stream of
+    this chip reaches at that size."""
     from lorafusion_amd.ops.nf4 import dequantize_nf4_triton, quantize_nf4
 
-    wq = torch.randn(14336, 4096, device=dev) * 0.02
+    rows, cols = shape
+    wq = torch.randn(rows, cols, device=dev) * 0.02
     packed, qs = quantize_nf4(wq)
-    out = torch.empty(14336 * 4096, dtype=torch.bfloat16, device=dev)
+    del wq
+    out = torch.empty(rows * cols, dtype=torch.bfloat16, device=dev)
     t_op = event_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), 20)     # as called from Python
     t_k = graph_time_ms(lambda: dequantize_nf4_triton(packed, qs, out=out), 100)     # the kernel alone
-    n = 14336 * 4096
+    n = rows * cols
     nbytes = n / 2 + n / 64 + 4 * n / 16384 + 1028 + 2 * n
     gbs = nbytes / (t_k * 1e-3) / 1e9
-    return {"GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "launch_ms": round(t_k, 4),
-            "op_ms_from_python": round(t_op, 4), "bytes_per_launch": nbytes, "shape": [14336, 4096],
-            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "nf4_dequant_kernel"}}
+    res = {"GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "launch_ms": round(t_k, 4),
+           "op_ms_from_python": round(t_op, 4), "bytes_per_launch": nbytes, "shape": [rows, cols],
+           "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "nf4_dequant_kernel"}}
+    if fill:
+        t_f = graph_time_ms(lambda: out.fill_(1.0), 100)
+        res["plain_fill_of_the_output"] = {"launch_ms": round(t_f, 4), "GB/s": round(2 * n / (t_f * 1e-3) / 1e9, 1),
+                                           "bytes": 2 * n, "kernel": "torch fill_ (vectorized_elementwise_kernel)"}
+    return res
+
+
+def nf4_block(dev) -> dict:
+    """`--only nf4`: the dequant kernel at the C3 weight and at the four weights of the 70B-class layer, each next to a
+    plain fill of its output."""
+    shapes = {"c3 [14336, 4096]": (14336, 4096), "c5 qkv [10240, 8192]": (10240, 8192), "c5 o [8192, 8192]": (8192, 8192),
+              "c5 gate_up [57344, 8192]": (57344, 8192), "c5 down [8192, 28672]": (8192, 28672)}
+    return {name: nf4_dequant_block(dev, shp, fill=True) for name, shp in shapes.items()}
+
+
+def gemm_ref_block(dev, reps: int = 20) -> dict:
+    """`--only gemm_ref`: the plain GEMMs of the 8B layer's largest shapes through this library (lf_gemm: the persistent
+    kernel without a LoRA term) and through torch.matmul (hipBLASLt), same tensors, same process -- the run the
+    counter comparison in profiles/ is taken from."""
+    from lorafusion_amd.ops import hip_ops
+
+    out = {}
+    for name, (M, N, K, trans_b) in {"16384x4096x4096 NT": (16384, 4096, 4096, True), "16384x4096x28672 NN": (16384, 4096, 28672, False),
+                                     "16384x14336x4096 NT": (16384, 14336, 4096, True)}.items():
+        g = torch.Generator(device=dev).manual_seed(0)
+        a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+        b = (torch.randn(N, K, generator=g, device=dev) if trans_b else torch.randn(K, N, generator=g, device=dev)).to(torch.bfloat16)
+        fl = 2.0 * M * N * K
+        t_lib = event_time_ms(lambda: hip_ops.gemm(a, b, trans_b=trans_b), reps)
+        t_ref = event_time_ms(lambda: torch.matmul(a, b.T if trans_b else b), reps)
+        out[name] = {"lf_gemm_ms": round(t_lib, 4), "lf_gemm_TFLOP/s": round(fl / t_lib / 1e9, 1), "lf_gemm_frac": round(fl / t_lib / 1e9 / BF16_PEAK_TFLOPS, 4),
+                     "torch_matmul_ms": round(t_ref, 4), "torch_matmul_TFLOP/s": round(fl / t_ref / 1e9, 1),
+                     "torch_matmul_frac": round(fl / t_ref / 1e9 / BF16_PEAK_TFLOPS, 4)}
+        del a, b
+        torch.cuda.empty_cache()
+    return out
+
+
+FIG5_M, FIG5_KN = (2048, 4096, 8192), (4096, 5120, 8192)
+
+
+def fig5_block(args, dev) -> dict:
+    """The shape grid of the reference's kernel benchmark (benchmarks_paper/scripts/kernel_perf/1_bench_kernel.sh:3-16,
+    bench_lora_kernels.py:682-685): one LoRA linear, M rows, K = N, r = 16, p = 0.1, forward + backward."""
+    out = {}
+    for m in FIG5_M:
+        for kn in FIG5_KN:
+            name = f"fig5_M{m}_KN{kn}"
+            WORKLOADS[name] = (m, 1, 16, [2.0], [0.1], False, 4096, [("linear", kn, kn)])
+            NAMES[name] = f"single LoRA linear, {m} tokens, K=N={kn}, r=16, p=0.1, explicit bit-packed mask, fwd+bwd"
+            r = raw_workload(name, args, dev)
+            out[f"M={m},K=N={kn}"] = {"ms_per_step": r["ms_per_step"], "TFLOP/s": r["value"], "kernels_ms": r["kernels_ms"],
+                                      "lora_overhead_vs_plain_gemms": r["lora_overhead_vs_plain_gemms"],
+                                      "roofline": {k: r["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "kernel", "launch_ms")}}
+    return out
 
 
 def norm_act_block(dev) -> dict:
@@ -413,7 +490,7 @@ def norm_act_block(dev) -> dict:
     }
     # the down projection's rank-r pass (4 adapters r=16, the layer's segments, keep-mask drawn in the kernel) with the
     # activation as its prologue, next to the activation kernel followed by the plain pass.  Algorithmic bytes per
-    # element: 7 fused (read gate and up, write the product and the mask byte), 6 + 3 separate.
+    # element: 6.125 fused (read gate and up, write the product and the mask bit), 6 + 2.125 separate.
     from lorafusion_amd.ops import multi_lora as ml
 
     seq = segments(16384, 4, seed=0, longest=8192)
@@ -423,13 +500,14 @@ def norm_act_block(dev) -> dict:
     a_list = [torch.randn(16, I, device=dev, generator=g).to(torch.bfloat16) * 0.01 for _ in range(4)]
     a_ptrs = L.ptr_array(a_list)
     s_out = torch.empty(M, 16, device=dev, dtype=torch.bfloat16)
-    mask_out = torch.empty(M, I, device=dev, dtype=torch.bool)
+    mask_out = torch.empty(M, I // 8, device=dev, dtype=torch.uint8)   # bit-packed, as the training path keeps it
     seed = ctypes.c_uint64(1234)
-    calls["down_xa_with_silu_mul_prologue"] = (7 * M * I, "lora_xa_kernel<.., seeded, activation>", lambda: L.check(
+    bits = L.LF_BF16 | L.LF_MASK_BITS
+    calls["down_xa_with_silu_mul_prologue"] = (6 * M * I + M * I // 8, "lora_xa_kernel<.., seeded, activation>", lambda: L.check(
         lib.lf_lora_xa_silu_mul(gu.data_ptr(), gu[:, I:].data_ptr(), 2 * I, c.data_ptr(), None, mask_out.data_ptr(), seed,
-                                a_ptrs, s_out.data_ptr(), M, I, 16, rt.c, 0, st), "lf_lora_xa_silu_mul"))
-    calls["down_xa_seeded_alone"] = (3 * M * I, "lora_xa_kernel<.., seeded>", lambda: L.check(
-        lib.lf_lora_xa_seeded(c.data_ptr(), mask_out.data_ptr(), a_ptrs, s_out.data_ptr(), M, I, 16, rt.c, seed, 0, st),
+                                a_ptrs, s_out.data_ptr(), M, I, 16, rt.c, bits, st), "lf_lora_xa_silu_mul"))
+    calls["down_xa_seeded_alone"] = (2 * M * I + M * I // 8, "lora_xa_kernel<.., seeded>", lambda: L.check(
+        lib.lf_lora_xa_seeded(c.data_ptr(), mask_out.data_ptr(), a_ptrs, s_out.data_ptr(), M, I, 16, rt.c, seed, bits, st),
         "lf_lora_xa_seeded"))
     out = {"rows": M, "hidden": H, "intermediate": I}
     for name, (nbytes, kernel, fn) in calls.items():
@@ -591,7 +669,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload (c4), its roofline and the CPU baseline")
-    ap.add_argument("--only", choices=sorted(WORKLOADS) + ["norm_act"], default=None,
+    ap.add_argument("--only", choices=sorted(WORKLOADS) + ["norm_act", "nf4", "gemm_ref", "fig5"], default=None,
                     help="run one workload through the raw ops and print its entry alone (for profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -612,6 +690,15 @@ def main():
 
     if args.only == "norm_act":
         print(json.dumps({"metric": "norm_act", **norm_act_block(dev)}))
+        return
+    if args.only == "nf4":
+        print(json.dumps({"metric": "nf4_dequant", **nf4_block(dev)}))
+        return
+    if args.only == "gemm_ref":
+        print(json.dumps({"metric": "plain GEMM: lf_gemm vs torch.matmul (hipBLASLt)", **gemm_ref_block(dev)}))
+        return
+    if args.only == "fig5":
+        print(json.dumps({"metric": "fig5 grid", **fig5_block(argparse.Namespace(steps=max(5, args.steps // 2), warmup=2), dev)}))
         return
     if args.only is not None:
         print(json.dumps({"metric": METRIC, **raw_workload(args.only, args, dev, breakdown=not args.no_extras)}))
@@ -634,7 +721,7 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": NAMES["c4"], "tokens": 16384, "rows_launched": Mp, "rank": 16, "adapters": 4,
-                   "seq_len_list": seq, "linears": per},
+                   "seq_len_list": seq, "linears": per, "lora_overhead_vs_plain_gemms": raw["lora_overhead_vs_plain_gemms"]},
         "roofline": raw["roofline"],
         "kernels_ms": raw["kernels_ms"],
         "lora_overhead_vs_plain_gemms": raw["lora_overhead_vs_plain_gemms"],
@@ -644,7 +731,9 @@ def main():
         res["nf4_dequant"] = nf4_dequant_block(dev)
         res["norm_act"] = norm_act_block(dev)
         small = argparse.Namespace(steps=max(5, args.steps // 2), warmup=max(2, args.warmup // 2))
-        res["workloads"] = {name: raw_workload(name, args if name == "c2" else small, dev) for name in ("c1", "c2", "c3", "c5")}
+        res["workloads"] = {name: raw_workload(name, args if name == "c2" else small, dev)
+                            for name in ("c1", "c2", "c3", "c4_qkv_merged", "c4_separate", "c5")}
+        res["workloads"]["fig5"] = fig5_block(small, dev)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline_c4()
     print(json.dumps(res))

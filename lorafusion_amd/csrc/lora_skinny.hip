@@ -350,16 +350,27 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
 }
 
 // S[row][col] = cast( mult * sum_p part[p][row][col] ), zero for padded rows / rank columns.
-// Sum of `n` fp32x4 partials `stride` floats apart, in index order (deterministic), four loads in flight.
+// Sum of `n` fp32x4 partials `stride` floats apart, in index order (deterministic).
 __device__ __forceinline__ lf_f32x4 sum_parts(const float* __restrict__ p, int64_t stride, int n) {
+  // Up to sixteen partials are requested before the first is added: these second stages are short launches whose
+  // time is the chain of memory round trips of one thread, and with four loads in flight a sum of sixteen was four
+  // round trips long (5 us for a few hundred KB).  The order of the additions is the index order either way.
   lf_f32x4 v = {0.f, 0.f, 0.f, 0.f};
   int i = 0;
-  for (; i + 4 <= n; i += 4) {
-    const lf_f32x4 a = *(const lf_f32x4*)(p + (int64_t)i * stride), b = *(const lf_f32x4*)(p + (int64_t)(i + 1) * stride);
-    const lf_f32x4 c = *(const lf_f32x4*)(p + (int64_t)(i + 2) * stride), d = *(const lf_f32x4*)(p + (int64_t)(i + 3) * stride);
-    v += a; v += b; v += c; v += d;
+  for (; i + 16 <= n; i += 16) {
+    lf_f32x4 t[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) t[k] = *(const lf_f32x4*)(p + (int64_t)(i + k) * stride);
+#pragma unroll
+    for (int k = 0; k < 16; k++) v += t[k];
   }
-  for (; i < n; i++) v += *(const lf_f32x4*)(p + (int64_t)i * stride);
+  if (i < n) {
+    lf_f32x4 t[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) t[k] = (i + k < n) ? *(const lf_f32x4*)(p + (int64_t)(i + k) * stride) : lf_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < 16; k++) v += t[k];   // (adding the zeros beyond n changes nothing: x + 0 = x, and -0 cannot arise from a sum that started at +0)
+  }
   return v;
 }
 template <typename T>
