@@ -138,14 +138,20 @@ __device__ __forceinline__ void tile_load(TileRegs& r, const T* __restrict__ src
     const int row = min(row0 + i * 32 + (tid >> 3), max_row - 1);
     const int64_t off = (int64_t)row * ld + col0 + srcg * 8;
     r.x[i] = *((const lf_u32x4*)(src + off));
-    if (use_mask) r.m[i] = mask_bits ? expand_keep8(mask[off >> 3]) : *((const lf_u32x2*)(mask + off));
+    // (bit format: the byte is only requested here; tile_store spreads it into eight bytes)
+    if (use_mask) {
+      if (mask_bits) r.m[i][0] = mask[off >> 3];
+      else r.m[i] = *((const lf_u32x2*)(mask + off));
+    }
   }
 }
 
-__device__ __forceinline__ void tile_store(const TileRegs& r, char* tile, int tid, bool use_mask) {
+__device__ __forceinline__ void tile_store(const TileRegs& r, char* tile, int tid, bool use_mask, bool mask_bits = false) {
 #pragma unroll
-  for (int i = 0; i < 4; i++)
-    *(lf_u32x4*)(tile + (i * 256 + tid) * 16) = use_mask ? apply_mask8(r.x[i], r.m[i]) : r.x[i];
+  for (int i = 0; i < 4; i++) {
+    const lf_u32x2 m = (use_mask && mask_bits) ? expand_keep8(r.m[i][0]) : r.m[i];
+    *(lf_u32x4*)(tile + (i * 256 + tid) * 16) = use_mask ? apply_mask8(r.x[i], m) : r.x[i];
+  }
 }
 
 // Row fragment: 8 consecutive columns (granule g) of `row`.
@@ -257,7 +263,12 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
           xv[b][u][i] = *((const lf_u32x4*)(xrow[i] + s * 64));
           if constexpr (ACT) uv[b][u][i] = *((const lf_u32x4*)((const char*)(xrow[i] + s * 64) + u_off));
           if constexpr (!GEN) {
-            if (use_mask) mv[b][u][i] = mask_bits ? expand_keep8(mrow[i][s * 8]) : *((const lf_u32x2*)(mrow[i] + s * 64));
+            // (bit format: the byte is only requested here and spread into eight bytes where it is used, so that no
+            // wait for it separates the loads of a batch)
+            if (use_mask) {
+              if (mask_bits) mv[b][u][i][0] = mrow[i][s * 8];
+              else mv[b][u][i] = *((const lf_u32x2*)(mrow[i] + s * 64));
+            }
           }
         }
 #pragma unroll
@@ -297,6 +308,9 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
             } else {
               if (row_real[i]) *(lf_u32x2*)(mask_out + erow[i] + s * 64) = mv[b][u][i];
             }
+          }
+          if constexpr (!GEN) {
+            if (use_mask && mask_bits) mv[b][u][i] = expand_keep8(mv[b][u][i][0]);
           }
           *(lf_u32x4*)(patch + (i >> 1) * 2048 + wr_off[i & 1]) = use_mask ? apply_mask8(xv[b][u][i], mv[b][u][i]) : xv[b][u][i];
         }
@@ -700,7 +714,7 @@ lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, int ma
   lf_u32x4 dr[RT];
   tile_load(tr, X, mask, K, bb0 * ROWS, Mrows, kt * 64, tid, use_mask, mask_bits != 0);
   load_ds(dr, bb0);
-  tile_store(tr, xs, tid, use_mask);
+  tile_store(tr, xs, tid, use_mask, mask_bits != 0);
   store_ds(dr, dss);
   if (bb0 + 1 < bb1) {
     tile_load(tr, X, mask, K, (bb0 + 1) * ROWS, Mrows, kt * 64, tid, use_mask, mask_bits != 0);
@@ -727,7 +741,7 @@ lora_da_kernel(const T* __restrict__ X, const uint8_t* __restrict__ mask, int ma
       }
     }
     if (b + 1 < bb1) {
-      tile_store(tr, xs + ((t + 1) & 1) * TILE_BYTES, tid, use_mask);
+      tile_store(tr, xs + ((t + 1) & 1) * TILE_BYTES, tid, use_mask, mask_bits != 0);
       store_ds(dr, dss + ((t + 1) & 1) * ROWS * RP);
       if (b + 2 < bb1) {
         tile_load(tr, X, mask, K, (b + 2) * ROWS, Mrows, kt * 64, tid, use_mask, mask_bits != 0);

@@ -6,11 +6,20 @@
 //   out[2i] = NF4[q[i] >> 4] * absmax ; out[2i+1] = NF4[q[i] & 15] * absmax   (:154-158)
 // with one fp32 rounding per operation and round-to-nearest-even on the final cast.
 //
-// Layout: the weight is one flat run of packed bytes, so the kernel is 1-D.  Each lane takes 4
-// packed bytes (8 elements) per step and writes one 16-byte vector; a wavefront therefore
-// reads 256 contiguous bytes and writes 1 KiB contiguous bytes per step.  The 16 NF4 values
-// and the 256-entry second-level table live in LDS (a wave's lookups hit distinct banks or
-// broadcast).  Each workgroup covers STEPS*2048 elements so several loads are in flight per lane.
+// Layout: the weight is one flat run of packed bytes, so the kernel is 1-D, and every wavefront works alone: no
+// barrier after the set-up of the two tables.  A wave takes chunks of 64*U packed dwords (U steps; each lane 4 packed
+// bytes = 8 elements per step, so a step reads 256 contiguous bytes and writes 1 KiB contiguous bytes); chunk c
+// goes to wave c mod (waves of the grid), so the addresses in flight form one compact window that moves through
+// the weight.  The block scales of a chunk are computed once by its first lanes (one byte load and one table
+// lookup per quantisation block, not per lane and step: the texture addresser's time goes to the data) and handed
+// to the lanes of each step by a cross-lane read.  The loads of a wave's next chunk are issued before the stores
+// of the current one.  The 16 NF4 values and the 256-entry second-level table live in LDS (a wave's lookups hit
+// distinct banks or broadcast).
+//
+// Stores are non-temporal: the output is 4 of every 5 bytes this kernel moves and is written exactly once, and
+// with stores that do not allocate in the caches the [14336, 4096] weight takes 21.5 us instead of 23.5, the
+// [57344, 8192] weight 165 us instead of 220 (7.15 TB/s; a fill of the same output alone: 137 us).  Non-temporal
+// loads of the packed bytes measured slower (26.5 us at [14336, 4096]).
 #include "lf_common.h"
 
 namespace {
@@ -33,73 +42,81 @@ template <> __device__ __forceinline__ uint32_t pack2<_Float16>(float lo, float 
   return __builtin_bit_cast(uint32_t, v);
 }
 
-#ifndef LF_NF4_STEPS
-#define LF_NF4_STEPS 16
-#endif
 constexpr int NF4_THREADS = 256;
-constexpr int NF4_STEPS = LF_NF4_STEPS;
+constexpr int NF4_WAVES = NF4_THREADS / 64;
 
-template <typename T, bool NESTED>
+template <typename T, bool NESTED, int U>
 __global__ void __launch_bounds__(NF4_THREADS)
 nf4_dequant_kernel(const uint32_t* __restrict__ packed, const void* __restrict__ absmax_in,
                    const float* __restrict__ code2, const float* __restrict__ absmax2,
                    const float* __restrict__ offset_p, lf_u32x4* __restrict__ out, int64_t n_words /* packed dwords */,
-                   int shift /* log2(blocksize) - 3: packed dword -> block */, int shift2 /* log2(blocksize2) */) {
+                   int shift /* log2(blocksize) - 3: packed dword -> block */, int shift2 /* log2(blocksize2) */,
+                   int64_t n_chunks /* of 64*U packed dwords */) {
   __shared__ float lut[16];
   __shared__ float lut2[256];
-  __shared__ float am_lds[NF4_THREADS * NF4_STEPS];  // block scales of this workgroup's span (at most one per packed dword)
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63;
   if (tid < 16) lut[tid] = kNf4Code[tid];
   if (NESTED) lut2[tid] = code2[tid];
-  const int64_t wg_base = (int64_t)blockIdx.x * (NF4_THREADS * NF4_STEPS);
-  const int64_t base = wg_base + tid;
-  // packed data first: these are the loads the stores wait for
-  uint32_t w[NF4_STEPS];
-#pragma unroll
-  for (int s = 0; s < NF4_STEPS; s++) {
-    const int64_t i = base + (int64_t)s * NF4_THREADS;
-        w[s] = i < n_words ? packed[i] : 0u;
-  }
-  if (NESTED) __syncthreads();  // lut2 is complete
-  // One scale per quantisation block of the span, computed once (a lane-per-dword lookup would
-  // issue a byte load and a float load per lane and step: twice the vector-memory instructions
-  // of the data itself, and the texture addresser takes 16 cycles for each).
-  const int64_t blk0 = wg_base >> shift;
-  const int nblk = ((NF4_THREADS * NF4_STEPS) >> shift) > 0 ? (NF4_THREADS * NF4_STEPS) >> shift : 1;
+  __syncthreads();
+  const float offset = NESTED ? offset_p[0] : 0.f;
+  const int64_t wave0 = (int64_t)blockIdx.x * NF4_WAVES + (tid >> 6), n_waves = (int64_t)gridDim.x * NF4_WAVES;
+  // quantisation blocks per chunk (a block larger than a chunk holds whole chunks: the launcher picks U so that
+  // there are at most 64), and the lane that holds the scale of this lane's dword in each step
+  const int n_lead = ((64 * U) >> shift) > 0 ? (64 * U) >> shift : 1;
   const int64_t nblk_total = (n_words + ((int64_t)1 << shift) - 1) >> shift;
-  float offset = 0.f;
-  if (NESTED) offset = offset_p[0];
-  for (int j = tid; j < nblk; j += NF4_THREADS) {
-    const int64_t blk = blk0 + j;
-    float a = 0.f;
-    if (blk < nblk_total) {
+  int src[U];
+#pragma unroll
+  for (int s = 0; s < U; s++) src[s] = ((s * 64 + lane) >> shift) * 4;
+
+  uint32_t w_next[U], aq_next = 0;
+  float a2_next = 0.f;
+  auto request = [&](int64_t c) {
+    const int64_t base = c * (64 * U);
+#pragma unroll
+    for (int s = 0; s < U; s++) {
+      const int64_t i = base + s * 64 + lane;
+      w_next[s] = i < n_words ? packed[i] : 0u;
+    }
+    const int64_t blk = (base >> shift) + lane;
+    aq_next = 0;
+    a2_next = 0.f;
+    if (lane < n_lead && blk < nblk_total) {
       if (NESTED) {
-        const uint8_t aq = ((const uint8_t*)absmax_in)[blk];
-        // single-rounding fused multiply-add, as tl.fma in the reference
-        a = __builtin_fmaf(lut2[aq], absmax2[blk >> shift2], offset);
+        aq_next = ((const uint8_t*)absmax_in)[blk];
+        a2_next = absmax2[blk >> shift2];
       } else {
-        a = ((const float*)absmax_in)[blk];
+        a2_next = ((const float*)absmax_in)[blk];
       }
     }
-    am_lds[j] = a;
-  }
-  __syncthreads();
-  float am[NF4_STEPS];
+  };
+  int64_t c = wave0;
+  if (c < n_chunks) request(c);
+  for (; c < n_chunks; c += n_waves) {
+    uint32_t w[U];
 #pragma unroll
-  for (int s = 0; s < NF4_STEPS; s++) am[s] = am_lds[(s * NF4_THREADS + tid) >> shift];
+    for (int s = 0; s < U; s++) w[s] = w_next[s];
+    const uint32_t aq = aq_next;
+    const float a2 = a2_next;
+    if (c + n_waves < n_chunks) request(c + n_waves);
+    // single-rounding fused multiply-add, as tl.fma in the reference
+    const float scale = NESTED ? __builtin_fmaf(lut2[aq], a2, offset) : a2;
+    const int64_t base = c * (64 * U);
 #pragma unroll
-  for (int s = 0; s < NF4_STEPS; s++) {
-    const int64_t i = base + (int64_t)s * NF4_THREADS;
-    if (i < n_words) {
-      lf_u32x4 o;
+    for (int s = 0; s < U; s++) {
+      // (all 64 lanes take part in the cross-lane read: the bounds check comes after it)
+      const float am = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src[s], __builtin_bit_cast(int, scale)));
+      const int64_t i = base + s * 64 + lane;
+      if (i < n_words) {
+        lf_u32x4 o;
 #pragma unroll
-      for (int b = 0; b < 4; b++) {
-        const uint32_t byte = (w[s] >> (8 * b)) & 0xffu;  // memory order: byte b of the dword
-        const float hi = lut[byte >> 4] * am[s];
-        const float lo = lut[byte & 15u] * am[s];
-        o[b] = pack2<T>(hi, lo);
+        for (int b = 0; b < 4; b++) {
+          const uint32_t byte = (w[s] >> (8 * b)) & 0xffu;  // memory order: byte b of the dword
+          const float hi = lut[byte >> 4] * am;
+          const float lo = lut[byte & 15u] * am;
+          o[b] = pack2<T>(hi, lo);
+        }
+        __builtin_nontemporal_store(o, out + i);
       }
-      out[i] = o;  // a plain store: the non-temporal kind fills 117 MB at 5.6 TB/s, this one at 6.45
     }
   }
 }
@@ -119,12 +136,16 @@ int lf_launch_nf4_dequant(const uint8_t* packed, const void* absmax, const float
   shift -= 3;  // 8 elements per packed dword
   while (nested && (1 << shift2) < blocksize2) shift2++;
   const int64_t n_words = n_elems / 8;
-  const int64_t per_wg = (int64_t)NF4_THREADS * NF4_STEPS;
-  const int64_t grid = (n_words + per_wg - 1) / per_wg;
-  if (grid > 0x7fffffffLL) return LF_ESHAPE;
+  // four steps per chunk; one for blocksizes 8 and 16, whose chunk of four steps would hold more than 64 blocks
+  const int u = shift >= 2 ? 4 : 1;
+  const int64_t n_chunks = (n_words + 64 * u - 1) / (64 * u);
+  int64_t grid = (n_chunks + NF4_WAVES - 1) / NF4_WAVES;   // one chunk per wave up to 2^20 workgroups, then several
+  if (grid > (1 << 20)) grid = 1 << 20;
+#define LF_NF4_LAUNCH_U(T, NESTED, U)                                                                    \
+  return lf_launch((nf4_dequant_kernel<T, NESTED, U>), dim3((unsigned)grid), dim3(NF4_THREADS), 0, st,   \
+                   (const uint32_t*)packed, absmax, code2, absmax2, offset, (lf_u32x4*)out, n_words, shift, shift2, n_chunks)
 #define LF_NF4_LAUNCH(T, NESTED)                                                                         \
-  return lf_launch((nf4_dequant_kernel<T, NESTED>), dim3((unsigned)grid), dim3(NF4_THREADS), 0, st,      \
-                     (const uint32_t*)packed, absmax, code2, absmax2, offset, (lf_u32x4*)out, n_words, shift, shift2)
+  do { if (u == 4) LF_NF4_LAUNCH_U(T, NESTED, 4); else LF_NF4_LAUNCH_U(T, NESTED, 1); } while (0)
   if (out_dtype == LF_BF16) {
     if (nested) LF_NF4_LAUNCH(__bf16, true); else LF_NF4_LAUNCH(__bf16, false);
   } else if (out_dtype == LF_F16) {
@@ -133,4 +154,5 @@ int lf_launch_nf4_dequant(const uint8_t* packed, const void* absmax, const float
     return LF_EINVAL;
   }
 #undef LF_NF4_LAUNCH
+#undef LF_NF4_LAUNCH_U
 }

@@ -61,6 +61,34 @@ def test_dequant_all_codes_random_state():
     assert np.array_equal(_bits(dequantize_nf4_triton(packed, qs)), onf4.dequantize(st))
 
 
+@pytest.mark.parametrize("n,bs,nested", [
+    # blocksizes either side of the kernel's chunk of 2048 elements (512 below blocksize 32), lengths that end inside
+    # a chunk and inside a second-level block
+    (240, 8, False), (8 * 1000, 8, True), (560, 16, True), (16 * 4097, 16, False), (32 * 70, 32, True), (64, 64, True),
+    (64 * 33, 64, True), (64 * 629, 64, False), (256 * 10, 256, True), (1024 * 9, 1024, True), (2048 * 3, 2048, True),
+    (4096 * 3, 4096, False), (4096 * 5, 4096, True), (64 * 257, 64, True), (64 * (256 * 3 + 17), 64, True),
+    (1031 * 2112, 64, True),  # 2.2 M elements: a thousand chunks, ragged end
+])
+def test_dequant_random_state_sizes(n, bs, nested):
+    """Random codes and scales (not from the quantiser) at every power-of-two blocksize class."""
+    from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
+
+    rng = np.random.default_rng(n % 9973 + bs)
+    nb = n // bs
+    if nested:
+        st = onf4.NF4State(
+            packed=rng.integers(0, 256, n // 2, dtype=np.uint8), shape=(n,), blocksize=bs,
+            absmax=rng.integers(0, 256, nb, dtype=np.uint8), code2=onf4.dynamic_code_table(),
+            absmax2=(rng.random((nb + 255) // 256) * 0.05 + 1e-3).astype(np.float32),
+            offset=np.asarray([0.0173], dtype=np.float32))
+    else:
+        st = onf4.NF4State(rng.integers(0, 256, n // 2, dtype=np.uint8), (n,), bs,
+                           (rng.random(nb) * 0.1 + 1e-3).astype(np.float32), None, None, None, 256)
+    packed, qs = _to_state(st)
+    got = _bits(dequantize_nf4_triton(packed, qs))
+    assert np.array_equal(got, onf4.dequantize(st))
+
+
 def test_dequant_fp16_output():
     from lorafusion_amd.ops.nf4 import dequantize_nf4_triton
 
