@@ -29,7 +29,7 @@ dropout_mask_kernel(uint8_t* __restrict__ mask, int64_t n16, int K, uint32_t thr
     o[2 * c] = lo;
     o[2 * c + 1] = hi;
   }
-  *(lf_u32x4*)(mask + e0) = o;
+  __builtin_nontemporal_store(o, (lf_u32x4*)(mask + e0));   // a write-only stream: no reason to keep it in the caches
 }
 
 // Keep-mask formats: one byte per element (the reference's bool tensor, lorafusion/ops/triton_ops/dropout.py:79) and
@@ -58,7 +58,7 @@ mask_unpack_kernel(const uint16_t* __restrict__ bits, lf_u32x4* __restrict__ byt
   lf_u32x4 o;
 #pragma unroll
   for (int d = 0; d < 4; d++) o[d] = (((b >> (4 * d)) & 0xfu) * 0x00204081u) & 0x01010101u;
-  bytes[t] = o;
+  __builtin_nontemporal_store(o, bytes + t);
 }
 
 }  // namespace

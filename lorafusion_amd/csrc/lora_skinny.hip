@@ -292,7 +292,7 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
         for (int i = 0; i < 2 * NB; i++) {
           if constexpr (ACT) {
             xv[b][u][i] = silu_mul8<T>(xv[b][u][i], uv[b][u][i]);
-            if (row_real[i]) *(lf_u32x4*)(act_out + erow[i] + s * 64) = xv[b][u][i];
+            if (row_real[i]) __builtin_nontemporal_store(xv[b][u][i], (lf_u32x4*)(act_out + erow[i] + s * 64));
           }
           if constexpr (GEN) {
             uint32_t klo, khi;

@@ -75,7 +75,7 @@ rmsnorm_fwd_kernel(const lf_u32x4* __restrict__ x, const lf_u32x4* __restrict__ 
       unpack8<T>(wv[c], g);
 #pragma unroll
       for (int e = 0; e < 8; e++) f[e] = round16<T>(f[e] * r) * g[e];
-      if (FULL || c * 64 + lane < hc) yr[c * 64 + lane] = pack8<T>(f);
+      if (FULL || c * 64 + lane < hc) __builtin_nontemporal_store(pack8<T>(f), yr + c * 64 + lane);
     }
   }
 }
@@ -160,7 +160,7 @@ rmsnorm_bwd_kernel(const lf_u32x4* dy, const lf_u32x4* __restrict__ x, const lf_
       unpack8<T>(w_piece(c), g);
 #pragma unroll
       for (int e = 0; e < 8; e++) d[e] = r * (d[e] * g[e] - f[e] * coef);
-      if (FULL || c * 64 + lane < hc) dxr[c * 64 + lane] = pack8<T>(d);
+      if (FULL || c * 64 + lane < hc) __builtin_nontemporal_store(pack8<T>(d), dxr + c * 64 + lane);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -249,7 +249,7 @@ silu_mul_fwd_kernel(const lf_u32x4* __restrict__ a, const lf_u32x4* __restrict__
 #pragma unroll
   for (int i = 0; i < ROWS; i++)
     if (row0 + i < M) {
-      c[(int64_t)(row0 + i) * ldc + col] = silu_mul8<T>(av[i], bv[i]);
+      __builtin_nontemporal_store(silu_mul8<T>(av[i], bv[i]), c + (int64_t)(row0 + i) * ldc + col);
     }
 }
 
@@ -284,8 +284,8 @@ silu_mul_bwd_kernel(const lf_u32x4* __restrict__ dc, const lf_u32x4* a, const lf
         gb[e] = fc[e] * silu;
         ga[e] = fc[e] * (silu * (1.0f - sig) + sig) * fb[e];
       }
-      da[(int64_t)(row0 + i) * ldda + col] = pack8<T>(ga);
-      db[(int64_t)(row0 + i) * lddb + col] = pack8<T>(gb);
+      __builtin_nontemporal_store(pack8<T>(ga), da + (int64_t)(row0 + i) * ldda + col);
+      __builtin_nontemporal_store(pack8<T>(gb), db + (int64_t)(row0 + i) * lddb + col);
     }
 }
 
