@@ -131,17 +131,6 @@ __device__ __forceinline__ void sfor(F&& f) {
   [&]<int... I>(std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>{}), ...); }(std::make_integer_sequence<int, N>{});
 }
 
-// Measurement builds only (never defined in the library build): LF_BIG_TIMING adds per-tile cycle counters (seed, K loop,
-// epilogue, waits) summed into lf_big_timing; LF_ABL_NOLOAD / LF_ABL_NOREAD / LF_ABL_NOMASKLOAD / LF_ABL_NOSELECT drop
-// the tile loads, the fragment reads, the keep-mask loads or the keep-mask select (results are then wrong: the
-// builds exist to attribute cycles and clock to the parts of the kernel).
-#ifdef LF_BIG_TIMING
-__device__ unsigned long long lf_big_timing[16];  // cycles: seed, k loop, epilogue, wall (100 MHz), tiles
-#define LF_TICK(var) const long long var = __builtin_readcyclecounter()
-#else
-#define LF_TICK(var)
-#endif
-
 // LORA = false: the instance for calls without a LoRA term (the seed code is compiled out, which also keeps that
 // instance free of register spills: a kernel that needs scratch memory pays for it at every launch).
 template <typename T, bool NN, bool LORA>
@@ -250,11 +239,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     asm volatile("s_add_u32 m0, %0, %1" ::"s"(base), "n"(OFF.value) : "memory", "scc");
   };
   auto issue_load = [&](lf_u32x4 rsrc, uint32_t voff, int soff) __attribute__((always_inline)) {
-#ifndef LF_ABL_NOLOAD
     asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
-#else
-    asm volatile("" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
-#endif
   };
   // all 16 loads of K step k of the tile behind `src` into stage `stage` (prologue only: no MFMAs to hide behind)
   auto load_stage = [&](const LoadSrc& src, int k, int stage) __attribute__((always_inline)) {
@@ -335,19 +320,12 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     const Route rt = route;
     if (has_lora) route = route_of(nxt_tile.m0 + wm * 128);  // in flight during this tile's K loop
 
-    LF_TICK(tk0);
-#ifdef LF_BIG_TIMING
-    const long long tw0 = wall_clock64();
-#endif
     lf_u32x4 fa[2][8], fb[2][8];
     lf_f32x4 acc[8][8];
     uint32_t fa_off[2], fb_off[2];
     // one fragment read of sub-step KS of the stage at LDS byte offset `st`: idx < 8: A fragment idx; else B fragment idx-8
     auto read_one = [&](auto SET, auto KS, uint32_t st, auto IDX) __attribute__((always_inline)) {
       constexpr int idx = IDX.value, set = SET.value, ks = KS.value;
-#ifdef LF_ABL_NOREAD
-      if (st != 0xffffffffu) return;   // (ablation build) never true: the fragments keep their first values
-#endif
       if constexpr (idx < 8) {
         const uint32_t ad = fa_off[ks] + st;
         lf_u32x4 tmp;
@@ -457,14 +435,12 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     }
 
     // ------------------------------------------------------------ K loop
-    LF_TICK(tk1);
     barrier();   // both stages of this tile's first two K steps are in LDS (every wave has waited for its loads)
     {
       const uint32_t st = par * STAGE;
       sfor<16>([&](auto I) { read_one(S0{}, S0{}, st, integral_constant<int, (I.value + 8) & 15>{}); });
     }
     lgkm0();
-    LF_TICK(tk1b);
     // K step s lives in stage (par + s) & 1.  Sub-step 1 of step s refills that stage with step s+2 of this tile; the
     // last two steps prefetch the first two steps of the next tile instead (of this tile again when none follows:
     // loads that nothing consumes keep the step body uniform).  Gap schedule of a step (one MFMA = one gap of three
@@ -523,7 +499,6 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     }
     par = (par + nk) & 1;
     mfma_fence();
-    LF_TICK(tk2);
 
     // ------------------------------------------------------------ LoRA term: operands; forward: 64 MFMAs per chunk onto the
     // accumulators (dX: the term is formed per block row inside the epilogue below, from up to two chunks = 32 rank columns)
@@ -607,11 +582,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         asm volatile("ds_read_b128 %0, %1 offset:1280" : "=v"(m5_) : "v"(ad) : "memory");
         asm volatile("ds_read_b128 %0, %1 offset:1536" : "=v"(m6_) : "v"(ad) : "memory");
         asm volatile("ds_read_b128 %0, %1 offset:1792" : "=v"(m7_) : "v"(ad) : "memory");
-#ifdef LF_DBG_NOLDS
-        load_chunk(0, rf0, lv0, std::false_type{});
-#else
         load_chunk(0, rf0, lv0, std::true_type{});
-#endif
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(m0_), "+v"(m1_), "+v"(m2_), "+v"(m3_), "+v"(m4_), "+v"(m5_), "+v"(m6_), "+v"(m7_) :: "memory");
         const lf_u32x4 ones = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
         mw[0] = sel ? m0_ : ones; mw[1] = sel ? m1_ : ones; mw[2] = sel ? m2_ : ones; mw[3] = sel ? m3_ : ones;
@@ -728,17 +699,6 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       });
     };
     epilogue(std::bool_constant<NN && LORA>{});
-#ifdef LF_BIG_TIMING
-    if (tid == 0) {
-      const long long tk3 = __builtin_readcyclecounter();
-      atomicAdd(&lf_big_timing[0], (unsigned long long)(tk1 - tk0));
-      atomicAdd(&lf_big_timing[it == 0 ? 5 : 6], (unsigned long long)(tk1b - tk1));
-      atomicAdd(&lf_big_timing[1], (unsigned long long)(tk2 - tk1b));
-      atomicAdd(&lf_big_timing[2], (unsigned long long)(tk3 - tk2));
-      atomicAdd(&lf_big_timing[3], (unsigned long long)(wall_clock64() - tw0));
-      atomicAdd(&lf_big_timing[4], 1ull);
-    }
-#endif
     tile = nxt_tile;
     src = nxt_src;
   }
