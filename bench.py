@@ -238,11 +238,11 @@ class Linear:
         return dequantize_nf4_triton(self.packed, self.qs).reshape(self.n, self.k)
 
 
-def gemm_plan(M: int, N: int, routed: bool):
+def gemm_plan(M: int, N: int, K: int, routed: bool):
     from lorafusion_amd import _lib as L
 
     rows, ch, ct = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    L.check(L.lib().lf_gemm_plan(M, N, BLOCK if routed else 0, ctypes.byref(rows), ctypes.byref(ch), ctypes.byref(ct)), "lf_gemm_plan")
+    L.check(L.lib().lf_gemm_plan(M, N, K, BLOCK if routed else 0, ctypes.byref(rows), ctypes.byref(ch), ctypes.byref(ct)), "lf_gemm_plan")
     return rows.value, ch.value, ct.value
 
 
@@ -268,7 +268,7 @@ def kernel_breakdown(linears, reps: int):
         t["dys_dyb"] += graph_time_ms(lambda: hip_ops.fused_multi_lora_dys_dyb(lin.dy, s, lin.b, r), reps)
         t["da"] += graph_time_ms(lambda: hip_ops.fused_multi_lora_da(lin.x, ds, r, lin.mask), reps)
         # the dX GEMM's main launch: output [Mp, K], reduction over N
-        rows, cfg, _ = gemm_plan(b.Mp, lin.k, True)
+        rows, cfg, _ = gemm_plan(b.Mp, lin.k, lin.n, True)
         if rows < b.Mp:
             rh = b.head(rows)
             nseg = len(rh.padded_seq_len_list)

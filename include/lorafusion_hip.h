@@ -70,7 +70,9 @@ extern "C" {
  * One segment per adapter: dA_i / dB_i of a segment are written, not accumulated, so an adapter
  * whose tokens sit in two separate row ranges of one call would keep the second range's gradient
  * only -- pack each adapter's tokens contiguously, as prepare_multi_lora_batch_info's callers do
- * (lorafusion/train/training_utils.py:1304-1334 sorts by adapter), or sum the two outputs. */
+ * (lorafusion/train/training_utils.py:1304-1334 sorts by adapter), or give the two segments their own
+ * outputs and sum them (the Python autograd layer does that by itself when one adapter's tensors are
+ * passed for two segments: each occurrence receives its segment's gradient and autograd adds them). */
 typedef struct lf_routing {
   int32_t n_seg;
   int32_t block_size_m;
@@ -196,12 +198,12 @@ int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int 
  * kernel, needs M, N >= 256).  Returns LF_EINVAL outside -1..7. */
 int lf_set_tile_cfg(int tile_cfg);
 
-/* The launches the library makes for an M x N output (any K) when no configuration is pinned: rows
+/* The launches the library makes for an M x N output contracted over K when no configuration is pinned: rows
  * [0, *rows_head) as one launch of tile configuration *cfg_head and, when *rows_head < M, the rest
  * as a second launch of *cfg_tail (-1 when there is none).  routing_block_size_m: 0 for a
  * single-adapter call, else the routing block size.  For benchmarks that time one kernel of a
  * fused call on its own; no counterpart in the reference (Triton's autotuner picks there). */
-int lf_gemm_plan(int M, int N, int routing_block_size_m, int* rows_head, int* cfg_head, int* cfg_tail);
+int lf_gemm_plan(int M, int N, int K, int routing_block_size_m, int* rows_head, int* cfg_head, int* cfg_tail);
 
 /* NF4 block dequantisation.  Stands in for dequantize_nf4_triton
  * (lorafusion/ops/triton_ops/dequantize_nf4.py:271-346).  packed: uint8 [n/2] (element 2i in the

@@ -96,7 +96,7 @@ def lib() -> ctypes.CDLL:
     l.lf_lora_bwd_static.argtypes = [vp] * 11 + [i, i, i, i, rp, i, vp]
     l.lf_gemm.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, vp]
     l.lf_set_tile_cfg.argtypes = [i]
-    l.lf_gemm_plan.argtypes = [i, i, i, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
+    l.lf_gemm_plan.argtypes = [i, i, i, i, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
     l.lf_nf4_dequant.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, i, i, i, vp]
     l.lf_dropout_mask.argtypes = [vp, i, i, ctypes.c_float, rp, ctypes.c_uint64, vp]
     l.lf_lora_xa_seeded.argtypes = [vp, vp, vp, vp, i, i, i, rp, ctypes.c_uint64, i, vp]

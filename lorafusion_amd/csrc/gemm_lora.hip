@@ -32,6 +32,7 @@
 // fragment as the "a" operand) so each lane ends with four consecutive output columns of one
 // row.
 #include "lf_common.h"
+#include <algorithm>
 #include <type_traits>
 
 namespace {
@@ -137,7 +138,9 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // depends on the tile column only: the tiles of a column, which stream the same B panel and
   // run on one XCD, stay aligned in K and meet each other's lines in the L2 (1.5 % faster at
   // 8192x4096x4096 than an offset by row + column).
-  const int nk = p.K / BK;
+  // (split contraction: this workgroup's share of the K steps is [kbeg, kbeg + nk); an even count, like K / BK)
+  const int kbeg = p.ksplit > 1 ? (int)blockIdx.y * p.ks_steps : 0;
+  const int nk = p.ksplit > 1 ? min(p.ks_steps, p.K / BK - kbeg) : p.K / BK;
   const int kstart = (2 * (pid_n & LF_STAG)) % nk;
 
   // ---- direct-to-LDS buffer loads: per thread one 32-bit byte offset per 16-byte granule (row part,
@@ -189,6 +192,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     char* lb = ldsB + stage * B_STAGE + wave * 1024;
     int kt_pos = kstart + tile;
     if (kt_pos >= nk) kt_pos -= nk;
+    kt_pos += kbeg;
     const int a_soff = kt_pos * (BK * 2);
     const int b_soff = NN ? kt_pos * BK * (int)p.ldb * 2 : a_soff;
 #pragma unroll
@@ -202,6 +206,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   auto issue_load_one = [&](int stage, int tile, int idx) {
     int kt_pos = kstart + tile;
     if (kt_pos >= nk) kt_pos -= nk;
+    kt_pos += kbeg;
     const int a_soff = kt_pos * (BK * 2);
     if (idx < NLA) {
       char* la = ldsA + stage * A_STAGE + wave * 1024;
@@ -246,7 +251,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // one, and behind PAIR0 stages of tile loads in the texture addresser it would start a
   // microsecond late; the seeding MFMAs then run while the tiles land.
   const int wrow0 = m0 + wm * WM;  // first row of this wave's sub-tile
-  if (p.L == nullptr || wrow0 >= p.M) {
+  if (p.L == nullptr || wrow0 >= p.M || kbeg != 0) {   // (split contraction: the first slice carries the term)
     issue_first_tiles();
   } else {
     const T* __restrict__ L = (const T*)p.L;
@@ -595,6 +600,18 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
   // the sub-tile (WN*2 contiguous bytes) instead of 8-byte pieces scattered over 16 rows.
   // Granule g (16 bytes) of band row r sits at slot g ^ ((r / EP_RPW) & EP_KEY): EP_RPW rows span
   // the 64 banks once, so the 16 rows that write together land on different banks.
+  if (p.ksplit > 1) {
+    // split contraction: the fp32 sums of this slice, 16 bytes per lane (row l16 of a block, columns kg*4 .. +3)
+    float* __restrict__ part = p.ks_ws + (int64_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int gm = wrow0 + i * 16 + l16, gn = n0 + wn * WN + j * 16 + kg * 4;
+        if (gm < p.M && gn < p.N) *(lf_f32x4*)(part + (int64_t)gm * p.N + gn) = acc[i][j];
+      }
+    return;
+  }
   T* __restrict__ C = (T*)p.C;
   const uint16_t* bias16 = (const uint16_t*)p.bias;
   constexpr int EP_PITCH = WN * 2;              // bytes per band row
@@ -640,6 +657,40 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
 #endif
 }
 
+// Second stage of a split contraction: C[m][n] = cast(sum over the slices, in index order, + bias[n]).  Eight columns
+// per thread.
+template <typename T>
+__global__ void __launch_bounds__(256)
+ksplit_reduce_kernel(const float* __restrict__ part, int nslices, const uint16_t* __restrict__ bias, T* __restrict__ C,
+                     int M, int N, int64_t ldc) {
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (idx >= (int64_t)M * N) return;
+  const int row = (int)(idx / N), col = (int)(idx % N);
+  lf_f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
+  for (int s = 0; s < nslices; s++) {
+    const float* q = part + (int64_t)s * M * N + idx;
+    lo += *(const lf_f32x4*)q;
+    hi += *(const lf_f32x4*)(q + 4);
+  }
+  if (bias != nullptr) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      lo[e] += MfmaOp<T>::to_float(bias[col + e]);
+      hi[e] += MfmaOp<T>::to_float(bias[col + 4 + e]);
+    }
+  }
+  const lf_u32x4 o = {MfmaOp<T>::pack2(lo[0], lo[1]), MfmaOp<T>::pack2(lo[2], lo[3]), MfmaOp<T>::pack2(hi[0], hi[1]),
+                      MfmaOp<T>::pack2(hi[2], hi[3])};
+  *(lf_u32x4*)((uint16_t*)C + (int64_t)row * ldc + col) = o;
+}
+
+template <typename T>
+int launch_ksplit_reduce(const LfGemmParams& p, hipStream_t st) {
+  const int64_t n8 = (int64_t)p.M * p.N / 8, blocks = (n8 + 255) / 256;
+  return lf_launch(ksplit_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, st, (const float*)p.ks_ws, p.ksplit,
+                   (const uint16_t*)p.bias, (T*)p.C, p.M, p.N, p.ldc);
+}
+
 template <typename T, int BM, int BN, int WM, int WN, bool NN, int NSTAGE>
 int launch_cfg(LfGemmParams p, const LfSegTable& seg, hipStream_t st) {
   constexpr int NTHREADS = (BM / WM) * (BN / WN) * 64;
@@ -649,7 +700,7 @@ int launch_cfg(LfGemmParams p, const LfSegTable& seg, hipStream_t st) {
   auto kern = gemm_lora_kernel<T, BM, BN, WM, WN, NN, NSTAGE>;
   static LfLdsFlags lds_ok;
   if (!lf_allow_lds(kern, SMEM, lds_ok)) return LF_ELAUNCH;
-  return lf_launch(kern, dim3(p.grid_m * p.grid_n), dim3(NTHREADS), SMEM, st, p, seg);
+  return lf_launch(kern, dim3(p.grid_m * p.grid_n, p.ksplit > 1 ? p.ksplit : 1), dim3(NTHREADS), SMEM, st, p, seg);
 }
 
 template <typename T, bool NN>
@@ -670,10 +721,12 @@ int launch_dtype(const LfGemmParams& p, const LfSegTable& seg, int cfg, hipStrea
 }  // namespace
 
 // Tile choice from a measured cost model.  A launch runs in "rounds" of resident workgroups
-// (256 CUs x workgroups per CU).  Costs are microseconds measured at K = 4096 (the choice only
-// compares configurations at equal K): the first round costs lat0 + first_b * fill^2 (a lone
-// tile per CU runs latency bound at boost clock, a full round is power limited), every further
-// round next_a + next_b * fill, where fill is the occupied fraction of the round's slots.
+// (256 CUs x workgroups per CU).  Costs are microseconds measured at K = 4096: the first round
+// costs lat0 + first_b * fill^2 (a lone tile per CU runs latency bound at boost clock, a full round
+// is power limited), every further round next_a + next_b * fill, where fill is the occupied
+// fraction of the round's slots.  For another K every term scales with K / 4096 except kRamp
+// microseconds of lat0 (launch, first loads, epilogue), which a launch pays once whatever its K:
+// a second launch for left-over rows pays off at a long K and does not at a short one.
 struct TileCand { int cfg, bm, bn, slots; double lat0, first_b, next_a, next_b; };
 static const TileCand kCands[] = {
     {7, 256, 256, 256, 70.0, 40.0, 50.0, 30.0},   // persistent, 4 waves of 128x128 (gemm_big.hip): rounds = tiles per workgroup
@@ -683,20 +736,23 @@ static const TileCand kCands[] = {
     {5, 64, 64, 512, 19.0, 17.0, 13.0, 18.0},     // 4 waves, 32x32 per wave: spreads a short row range
     {6, 128, 64, 256, 22.5, 4.5, 13.0, 14.0},     // 4 waves, 64x32 per wave: less operand traffic per flop than 64x64
 };
-static double launch_cost(const TileCand& c, int M, int N) {
+constexpr double kRamp = 6.0;
+static double launch_cost(const TileCand& c, int M, int N, int K) {
   const long tiles = (long)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
   if (tiles <= 0) return 0.0;
   const long full = tiles / c.slots;
   const double fill = (double)(tiles % c.slots) / c.slots;
-  if (full == 0) return c.lat0 + c.first_b * fill * fill;
-  return c.lat0 + c.first_b + (full - 1) * (c.next_a + c.next_b) + (fill > 0 ? c.next_a + c.next_b * fill : 0.0);
+  double at4096;
+  if (full == 0) at4096 = c.lat0 + c.first_b * fill * fill;
+  else at4096 = c.lat0 + c.first_b + (full - 1) * (c.next_a + c.next_b) + (fill > 0 ? c.next_a + c.next_b * fill : 0.0);
+  return kRamp + (at4096 - kRamp) * (K / 4096.0);
 }
-static int choose_cfg(int M, int N, bool allow_big, double* cost_out = nullptr) {
+static int choose_cfg(int M, int N, int K, bool allow_big, double* cost_out = nullptr) {
   int best = 1;
   double best_cost = 1e30;
   for (const TileCand& c : kCands) {
     if (c.cfg == 7 && (!allow_big || M < 256 || N < 256)) continue;
-    const double cost = launch_cost(c, M, N);
+    const double cost = launch_cost(c, M, N, K);
     if (cost < best_cost) { best_cost = cost; best = c.cfg; }
   }
   if (cost_out) *cost_out = best_cost;
@@ -707,23 +763,64 @@ static int choose_cfg(int M, int N, bool allow_big, double* cost_out = nullptr) 
 // with the lowest modelled cost of both launches: usually the one whose tiles fill whole rounds of the chip
 // (32 tile rows of 40 tiles are exactly five rounds; 30 rows of 40 are five rounds too, and leave a longer tail).
 // Returns m_main (0: single launch).
-static int choose_split(int M, int N, bool allow_big, int* cfg_head, int* cfg_tail) {
+static int choose_split(int M, int N, int K, bool allow_big, int* cfg_head, int* cfg_tail) {
   constexpr double kLaunch = 4.0;  // a second launch
   const int grid_n = (N + 255) / 256;
   if (grid_n > 256) return 0;
   const bool big = allow_big && N >= 256;
   const TileCand& head = kCands[big ? 0 : 1];
   double best;
-  choose_cfg(M, N, allow_big, &best);
+  choose_cfg(M, N, K, allow_big, &best);
   int best_m = 0;
   for (int r = 1; r * 256 < M; r++) {
     double tail;
-    const int ct = choose_cfg(M - r * 256, N, allow_big, &tail);
-    const double cost = launch_cost(head, r * 256, N) + tail + kLaunch;
+    const int ct = choose_cfg(M - r * 256, N, K, allow_big, &tail);
+    const double cost = launch_cost(head, r * 256, N, K) + tail + kLaunch;
     if (cost < best) { best = cost; best_m = r * 256; *cfg_tail = ct; }
   }
   *cfg_head = big ? 7 : 1;
   return best_m;
+}
+
+// Split contraction for a launch of few tiles over a long K (left-over rows of a packed batch, short batches): K is
+// cut into slices, workgroup (tile, slice) keeps fp32 sums, a second kernel adds the slices.  Measured on the left-over
+// rows of the 8B and 70B layers (128 and 384 rows; microseconds with the second kernel, unsplit first):
+//   128 x 4096 over 28672 (NN): 64x64 tiles 134 -> 128x64 tiles in 4 slices 52;  over 6144: 31 -> 18
+//   128 x 4096 over 14336 (NT): 54 -> 35;   384 x 8192 over 57344 (NN): 128x128 tiles 580 -> 256x256 tiles in 4 slices 399
+//   384 x 8192 over 28672 (NT): 300 -> 203; 384 x 10240 over 8192: 64 unsplit, 95 in 2 slices of 256x256 tiles
+// So: when the planned tiles fill less than half of the chip's workgroup slots, the launch moves to the 128x64 tile (up
+// to 256 rows) or the eight-wave 256x256 tile (more rows) in as many slices as give every compute unit a workgroup,
+// provided a slice keeps at least 48 K steps on the small tile and 192 on the large one (their fixed cost per
+// workgroup: pipeline fill and an fp32 store of the tile), at most 16 slices and at most kKsplitMaxBytes of partial
+// tiles.  A function of the shape, the planned tile and the routing block alone: a call that is given the workspace
+// lf_workspace_bytes names always makes the same split, so its result does not depend on who calls.
+constexpr size_t kKsplitMaxBytes = (size_t)64 << 20;
+struct KSplit { int cfg, n, steps; };
+static long tiles_of(int M, int N, int cfg, int* slots = nullptr) {
+  int bm = 256, bn = 256, sl = 256;      // configurations 0, 1, 7
+  for (const TileCand& k : kCands) if (k.cfg == cfg) { bm = k.bm; bn = k.bn; sl = k.slots; }
+  if (cfg == 2) { bm = 128; bn = 256; }
+  if (slots != nullptr) *slots = sl;
+  return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+}
+static KSplit ksplit_for(int M, int N, int K, int cfg, int routing_block) {
+  const int nk = K / BK;
+  const KSplit none = {cfg, 1, nk};
+  int slots = 256;
+  if (cfg == 7 || 2 * tiles_of(M, N, cfg, &slots) > slots) return none;   // the planned launch fills half of its slots
+  const bool big_ok = routing_block <= 0 || routing_block % 128 == 0;
+  const int cand = M <= 256 ? 6 : (big_ok ? 1 : 2);
+  const int min_steps = cand == 6 ? 48 : 192;
+  const long tiles = tiles_of(M, N, cand);
+  long n = 256 / tiles;
+  n = std::min(n, (long)16);
+  n = std::min(n, (long)(nk / min_steps));
+  const size_t slice = (size_t)M * N * sizeof(float);
+  n = std::min(n, (long)(kKsplitMaxBytes / slice));
+  if (n < 2) return none;
+  int steps = (int)((nk + n - 1) / n);
+  steps += steps & 1;                                         // an even number of steps per slice (K / BK is even)
+  return {cand, (nk + steps - 1) / steps, steps};             // no empty slice
 }
 
 static std::atomic<int> pinned_cfg{-1};
@@ -733,22 +830,41 @@ int lf_pin_tile_cfg(int cfg) {
   return LF_OK;
 }
 
-// The launches lf_launch_gemm makes for an M x N product when no configuration is pinned: rows [0, *rows_head)
+// The launches lf_launch_gemm makes for an M x N product over K when no configuration is pinned: rows [0, *rows_head)
 // with *cfg_head and, when *rows_head < M, the remaining rows with *cfg_tail (-1 otherwise).
-void lf_plan_gemm(int M, int N, int routing_block, int* rows_head, int* cfg_head, int* cfg_tail) {
+void lf_plan_gemm(int M, int N, int K, int routing_block, int* rows_head, int* cfg_head, int* cfg_tail) {
   const bool allow_big = routing_block <= 0 || (routing_block % 128 == 0 && M % 128 == 0);
   int ch = 1, ct = 1;
-  const int m_main = choose_split(M, N, allow_big, &ch, &ct);
+  const int m_main = choose_split(M, N, K, allow_big, &ch, &ct);
   auto demote = [&](int cfg) { return (routing_block > 0 && routing_block % 128 != 0 && (cfg == 0 || cfg == 1 || cfg == 7)) ? 2 : cfg; };
   if (m_main == 0) {
     *rows_head = M;
-    *cfg_head = demote(choose_cfg(M, N, allow_big));
+    *cfg_head = demote(choose_cfg(M, N, K, allow_big));
     *cfg_tail = -1;
   } else {
     *rows_head = m_main;
     *cfg_head = demote(ch);
     *cfg_tail = demote(ct);
   }
+}
+
+// Bytes of fp32 partial tiles the split contraction of an M x N product over K may write: the largest need over the
+// launches of the plan and over the configurations a launch can be moved to at run time (the eight-wave 256x256 tile
+// and the 128x256 tile stand in for the persistent kernel where it does not apply).
+size_t lf_gemm_ksplit_bytes(int M, int N, int K, int routing_block) {
+  if (M <= 0 || N <= 0 || K < BK) return 0;
+  int rows = 0, ch = 1, ct = -1;
+  lf_plan_gemm(M, N, K, routing_block, &rows, &ch, &ct);
+  size_t need = 0;
+  auto part = [&](int m, int cfg) {
+    for (int c : {cfg, 1, 2}) {
+      const KSplit ks = ksplit_for(m, N, K, c, routing_block);
+      if (ks.n > 1) need = std::max(need, (size_t)ks.n * m * N * sizeof(float));
+    }
+  };
+  part(rows, ch);
+  if (ct >= 0) part(M - rows, ct);
+  return need;
 }
 
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st) {
@@ -772,13 +888,22 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
     // element, a dX term of more than 32 rank columns and (when the library chose the tile) a contraction of one K step
     if (cfg == 7 && ((q.mask != nullptr && (!q.mask_bits || q.N % 128 != 0)) || (nn && q.L != nullptr && q.R > 32) || (planned && q.K < 128))) cfg = 1;
     if (cfg == 7) return lf_launch_gemm_big(q, seg, nn, dtype, st);
-    if (dtype == LF_BF16) return nn ? launch_dtype<__bf16, true>(q, seg, cfg, st) : launch_dtype<__bf16, false>(q, seg, cfg, st);
-    if (dtype == LF_F16) return nn ? launch_dtype<_Float16, true>(q, seg, cfg, st) : launch_dtype<_Float16, false>(q, seg, cfg, st);
-    return (int)LF_EINVAL;
+    if (dtype != LF_BF16 && dtype != LF_F16) return (int)LF_EINVAL;
+    LfGemmParams r = q;
+    r.ksplit = 1;
+    if (planned && r.ks_ws != nullptr && ((uintptr_t)r.ks_ws & 15) == 0) {   // (a pinned tile configuration stays as pinned)
+      const KSplit ks = ksplit_for(r.M, r.N, r.K, cfg, seg.table != nullptr ? seg.block_size_m : 0);
+      if (ks.n > 1 && (size_t)ks.n * r.M * r.N * sizeof(float) <= r.ks_ws_bytes) { cfg = ks.cfg; r.ksplit = ks.n; r.ks_steps = ks.steps; }
+    }
+    int rc;
+    if (dtype == LF_BF16) rc = nn ? launch_dtype<__bf16, true>(r, seg, cfg, st) : launch_dtype<__bf16, false>(r, seg, cfg, st);
+    else rc = nn ? launch_dtype<_Float16, true>(r, seg, cfg, st) : launch_dtype<_Float16, false>(r, seg, cfg, st);
+    if (rc != LF_OK || r.ksplit <= 1) return rc;
+    return dtype == LF_BF16 ? launch_ksplit_reduce<__bf16>(r, st) : launch_ksplit_reduce<_Float16>(r, st);
   };
   if (force_cfg >= 0) return launch(p, force_cfg);
   int m_main = 0, cfg_head = 1, cfg_tail = -1;
-  lf_plan_gemm(p.M, p.N, seg.table != nullptr ? seg.block_size_m : 0, &m_main, &cfg_head, &cfg_tail);
+  lf_plan_gemm(p.M, p.N, p.K, seg.table != nullptr ? seg.block_size_m : 0, &m_main, &cfg_head, &cfg_tail);
   if (cfg_tail < 0) return launch(p, cfg_head);
   LfGemmParams head = p, tail = p;
   head.M = m_main;

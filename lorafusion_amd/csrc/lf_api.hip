@@ -1,6 +1,7 @@
 // extern "C" entry points of liblorafusion_hip.so: argument checks, workspace carving, launches.
 #include "lf_common.h"
 #include <atomic>
+#include <algorithm>
 
 int lf_launch_nf4_dequant(const uint8_t*, const void*, const float*, const float*, const float*, void*, int64_t,
                           int, int, int, hipStream_t);
@@ -114,20 +115,22 @@ size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* 
   const bool reads_k = op == LF_OP_XA || op == LF_OP_DA || op == LF_OP_FWD || op == LF_OP_BWD || op == LF_OP_NF4_FWD ||
                        op == LF_OP_NF4_BWD;
   if ((reads_n && bad_tiled_dim(N)) || (reads_k && bad_tiled_dim(K))) return 0;
+  const int rb = t.table != nullptr ? t.block_size_m : 0;
   switch (op) {
     case LF_OP_XA: return align256(lf_xa_workspace(M, K, R, t));
     case LF_OP_DYS_DYB: return align256(lf_dys_dyb_workspace(M, N, R, t));
     case LF_OP_DA: return align256(lf_da_workspace(M, K, R, t));
-    case LF_OP_FWD: return align256(lf_xa_workspace(M, K, R, t));
+    // (the products of the whole-pass entry points may split their contraction: Y = [M,N] over K, dX = [M,K] over N)
+    case LF_OP_FWD: return align256(std::max(lf_xa_workspace(M, K, R, t), lf_gemm_ksplit_bytes(M, N, K, rb)));
     case LF_OP_BWD: {
       size_t a = lf_dys_dyb_workspace(M, N, R, t), b = lf_da_workspace(M, K, R, t);
-      return align256(a > b ? a : b);
+      return align256(std::max(std::max(a, b), lf_gemm_ksplit_bytes(M, K, N, rb)));
     }
     case LF_OP_NF4_FWD:
-      return align256((size_t)N * K * 2) + align256(lf_xa_workspace(M, K, R, t));
+      return align256((size_t)N * K * 2) + align256(std::max(lf_xa_workspace(M, K, R, t), lf_gemm_ksplit_bytes(M, N, K, rb)));
     case LF_OP_NF4_BWD: {
       size_t a = lf_dys_dyb_workspace(M, N, R, t), b = lf_da_workspace(M, K, R, t);
-      return align256((size_t)N * K * 2) + align256(a > b ? a : b);
+      return align256((size_t)N * K * 2) + align256(std::max(std::max(a, b), lf_gemm_ksplit_bytes(M, K, N, rb)));
     }
     default: return 0;
   }
@@ -178,8 +181,11 @@ int lf_swiglu_lora_fwd(const void* G, const void* U, int64_t ld, void* X_out, co
   return lf_lora_xw_sb(X_out, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
 }
 
-int lf_lora_xw_sb(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs,
-                  void* Y, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+// lf_lora_xw_sb / lf_lora_dyw_dsa with a workspace for the split contraction of under-filled launches (the whole
+// forward / backward entry points pass theirs on; the single-product entry points have none and never split)
+static int xw_sb_ws(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs, void* Y,
+                    void* workspace, size_t ws_bytes, int M, int N, int K, int R, const lf_routing* routing, int dtype,
+                    void* stream) {
   if (bad_dtype(dtype) || !X || !W || !Y) return LF_EINVAL;
   LfSegTable t{};
   if (S) {
@@ -193,7 +199,13 @@ int lf_lora_xw_sb(const void* X, const void* W, const void* bias, const void* S,
   p.A = X; p.B = W; p.C = Y; p.bias = bias;
   p.M = M; p.N = N; p.K = K; p.lda = K; p.ldb = K; p.ldc = N;
   p.L = S; p.R = R; p.mask = nullptr; p.ldmask = 0; p.mult_mode = 0;
+  p.ks_ws = (float*)workspace; p.ks_ws_bytes = workspace ? ws_bytes : 0;
   return lf_launch_gemm(p, t, /*nn=*/false, dtype, -1, (hipStream_t)stream);
+}
+
+int lf_lora_xw_sb(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs,
+                  void* Y, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  return xw_sb_ws(X, W, bias, S, b_ptrs, Y, nullptr, 0, M, N, K, R, routing, dtype, stream);
 }
 
 int lf_lora_dys_dyb(const void* dY, const void* S, const void* const* b_ptrs, void* dS, void* const* db_ptrs,
@@ -216,8 +228,9 @@ int lf_lora_da(const void* X, const uint8_t* mask, const void* dS, void* const* 
   return lf_launch_da(X, mask, mb, dS, workspace, ws_bytes, M, K, R, t, dtype, (hipStream_t)stream);
 }
 
-int lf_lora_dyw_dsa(const void* dY, const void* W, const void* dS, const void* const* a_ptrs, const uint8_t* mask,
-                    void* dX, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+static int dyw_dsa_ws(const void* dY, const void* W, const void* dS, const void* const* a_ptrs, const uint8_t* mask,
+                      void* dX, void* workspace, size_t ws_bytes, int M, int N, int K, int R, const lf_routing* routing,
+                      int dtype, void* stream) {
   const int mb = take_mask_bits(dtype);
   if (bad_dtype(dtype) || !dY || !W || !dX) return LF_EINVAL;
   LfSegTable t{};
@@ -233,7 +246,13 @@ int lf_lora_dyw_dsa(const void* dY, const void* W, const void* dS, const void* c
   p.A = dY; p.B = W; p.C = dX; p.bias = nullptr;
   p.M = M; p.N = K; p.K = N; p.lda = N; p.ldb = K; p.ldc = K;
   p.L = dS; p.R = R; p.mask = mask; p.ldmask = mb ? K / 8 : K; p.mask_bits = mb; p.mult_mode = 1;
+  p.ks_ws = (float*)workspace; p.ks_ws_bytes = workspace ? ws_bytes : 0;
   return lf_launch_gemm(p, t, /*nn=*/true, dtype, -1, (hipStream_t)stream);
+}
+
+int lf_lora_dyw_dsa(const void* dY, const void* W, const void* dS, const void* const* a_ptrs, const uint8_t* mask,
+                    void* dX, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  return dyw_dsa_ws(dY, W, dS, a_ptrs, mask, dX, nullptr, 0, M, N, K, R, routing, dtype, stream);
 }
 
 int lf_lora_fwd(const void* X, const void* W, const void* bias, const uint8_t* mask, const void* const* a_ptrs,
@@ -241,7 +260,8 @@ int lf_lora_fwd(const void* X, const void* W, const void* bias, const uint8_t* m
                 int K, int R, const lf_routing* routing, int dtype, void* stream) {
   int rc = lf_lora_xa(X, mask, a_ptrs, S_out, workspace, ws_bytes, M, K, R, routing, dtype, stream);
   if (rc != LF_OK) return rc;
-  return lf_lora_xw_sb(X, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
+  // (the rank-r pass is done with the workspace: the product's split contraction may have it)
+  return xw_sb_ws(X, W, bias, S_out, b_ptrs, Y, workspace, ws_bytes, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
 }
 
 int lf_lora_fwd_seeded(const void* X, const void* W, const void* bias, uint8_t* mask_out, const void* const* a_ptrs,
@@ -260,7 +280,9 @@ int lf_lora_bwd(const void* dY, const void* X, const void* W, const uint8_t* mas
   if (rc != LF_OK) return rc;
   rc = lf_lora_da(X, mask, dS_out, da_ptrs, workspace, ws_bytes, M, K, R, routing, dtype, stream);
   if (rc != LF_OK) return rc;
-  if (dX) rc = lf_lora_dyw_dsa(dY, W, dS_out, a_ptrs, mask, dX, M, N, K, R, routing, dtype, stream);
+  // (stream order: the partial sums of the two rank-r passes are consumed by now, so the product's split contraction
+  // may reuse the workspace from its start)
+  if (dX) rc = dyw_dsa_ws(dY, W, dS_out, a_ptrs, mask, dX, workspace, ws_bytes, M, N, K, R, routing, dtype, stream);
   return rc;
 }
 
@@ -287,9 +309,9 @@ int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8
 
 int lf_set_tile_cfg(int tile_cfg) { return lf_pin_tile_cfg(tile_cfg); }
 
-int lf_gemm_plan(int M, int N, int routing_block_size_m, int* rows_head, int* cfg_head, int* cfg_tail) {
-  if (M <= 0 || N <= 0 || rows_head == nullptr || cfg_head == nullptr || cfg_tail == nullptr) return LF_EINVAL;
-  lf_plan_gemm(M, N, routing_block_size_m, rows_head, cfg_head, cfg_tail);
+int lf_gemm_plan(int M, int N, int K, int routing_block_size_m, int* rows_head, int* cfg_head, int* cfg_tail) {
+  if (M <= 0 || N <= 0 || K <= 0 || rows_head == nullptr || cfg_head == nullptr || cfg_tail == nullptr) return LF_EINVAL;
+  lf_plan_gemm(M, N, K, routing_block_size_m, rows_head, cfg_head, cfg_tail);
   return LF_OK;
 }
 

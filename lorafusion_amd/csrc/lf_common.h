@@ -52,6 +52,12 @@ struct LfGemmParams {
   int grid_m, grid_n;
   int row0;           // global row of local row 0 (routing lookup when a launch covers a row range)
   int group_m;        // persistent kernel: tile rows per group of its tile order (set by its launcher)
+  // Split contraction (launches with few tiles and a long K; set by lf_launch_gemm): workgroup (x, y) contracts the
+  // K steps [y * ks_steps, (y + 1) * ks_steps) of tile x and writes its fp32 sums to ks_ws[y][M][N]; a second
+  // kernel adds the ksplit slices in index order.  ks_ws / ks_ws_bytes come from the caller (nullptr: never split).
+  float* ks_ws;
+  size_t ks_ws_bytes;
+  int ksplit, ks_steps;
 };
 
 // launchers (one per translation unit)
@@ -59,7 +65,8 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
 int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, hipStream_t st);  // persistent 256x256 tiles
 int lf_cu_count();
 int lf_pin_tile_cfg(int cfg);  // -1: automatic choice
-void lf_plan_gemm(int M, int N, int routing_block, int* rows_head, int* cfg_head, int* cfg_tail);
+void lf_plan_gemm(int M, int N, int K, int routing_block, int* rows_head, int* cfg_head, int* cfg_tail);
+size_t lf_gemm_ksplit_bytes(int M, int N, int K, int routing_block);  // workspace of the split contraction for this product
 
 // Raise a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's copy of
 // the function; one flag array per kernel instantiation; threads that race here repeat the same call).

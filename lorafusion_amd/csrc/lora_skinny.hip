@@ -31,6 +31,7 @@
 #include "lf_common.h"
 #include "act_math.h"
 #include "philox.h"
+#include <type_traits>
 
 namespace {
 
@@ -249,13 +250,21 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
 #pragma unroll
     for (int c = 0; c < RT; c++) acc[nb][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // (a second register set to overlap the next batch's loads costs occupancy and measured slower)
-  lf_u32x4 xv[1][XA_U][2 * NB], av[1][XA_U][RT][2];
-  lf_u32x4 uv[1][XA_U][ACT ? 2 * NB : 1];
-  lf_u32x2 mv[1][XA_U][2 * NB];
-  auto load_batch = [&](int b, int s0) {
+  // The steps in flight form two register sets where there are at least two (ranks up to 32): the loads of one set
+  // are requested before the other set is used, so a wave's memory time and its integer / LDS / MFMA time overlap.
+  // All waves of a launch start together and would otherwise sit in the same phase -- everyone waiting for memory,
+  // then everyone computing.  (Two sets of the full depth cost occupancy and measured slower.)
+#ifndef LF_XA_MODE
+#define LF_XA_MODE 1
+#endif
+  constexpr int NSET = (LF_XA_MODE == 0) ? 1 : (XA_U >= 2 ? 2 : 1), UB = (LF_XA_MODE == 2 && NSET == 2) ? 1 : XA_U / NSET;
+  lf_u32x4 xv[NSET][UB][2 * NB], av[NSET][UB][RT][2];
+  lf_u32x4 uv[NSET][UB][ACT ? 2 * NB : 1];
+  lf_u32x2 mv[NSET][UB][2 * NB];
+  auto load_batch = [&](auto B, int s0) {
+    constexpr int b = B.value;
 #pragma unroll
-    for (int u = 0; u < XA_U; u++) {
+    for (int u = 0; u < UB; u++) {
       const int s = s0 + u * XA_WAVES;
       if (s < nsteps) {
 #pragma unroll
@@ -283,9 +292,10 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
       }
     }
   };
-  auto use_batch = [&](int b, int s0) {
+  auto use_batch = [&](auto B, int s0) {
+    constexpr int b = B.value;
 #pragma unroll
-    for (int u = 0; u < XA_U; u++) {
+    for (int u = 0; u < UB; u++) {
       const int s = s0 + u * XA_WAVES;
       if (s < nsteps) {
 #pragma unroll
@@ -334,9 +344,22 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
       }
     }
   };
-  for (int s0 = wave; s0 < nsteps; s0 += XA_WAVES * XA_U) {
-    load_batch(0, s0);
-    use_batch(0, s0);
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, NSET - 1>;
+  constexpr int STRIDE = XA_WAVES * UB;   // steps between a wave's consecutive batches
+  if constexpr (NSET == 1) {
+    for (int s0 = wave; s0 < nsteps; s0 += STRIDE) {
+      load_batch(Set0{}, s0);
+      use_batch(Set0{}, s0);
+    }
+  } else {
+    load_batch(Set0{}, wave);
+    for (int s0 = wave; s0 < nsteps; s0 += 2 * STRIDE) {
+      load_batch(Set1{}, s0 + STRIDE);      // (steps beyond the row's end are skipped inside)
+      use_batch(Set0{}, s0);
+      load_batch(Set0{}, s0 + 2 * STRIDE);
+      use_batch(Set1{}, s0 + STRIDE);
+    }
   }
   __syncthreads();  // every wave is done with its patches
   // C layout: lane holds column (lane & 15), rows 4*(lane >> 4) + e

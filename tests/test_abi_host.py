@@ -107,6 +107,28 @@ def test_size_query_and_static_backward_refuse_untiled_shapes():
     assert call(256, 256, 256, 16, dy=None) == _lib.LF_EINVAL
 
 
+def test_launch_plan_takes_the_contraction_length():
+    """Host logic of the tile choice: left-over rows get a launch of their own when the contraction is long enough to
+    pay for it, and one launch covers everything when it is short."""
+    import ctypes
+
+    from lorafusion_amd import _lib as L
+
+    def plan(M, N, K, block=128):
+        rows, head, tail = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        assert L.lib().lf_gemm_plan(M, N, K, block, ctypes.byref(rows), ctypes.byref(head), ctypes.byref(tail)) == 0
+        return rows.value, head.value, tail.value
+
+    # 16512 rows = 64 tile rows of 256 and 128 more: the persistent kernel takes the 64, a small tile the rest
+    for N, K in [(6144, 4096), (4096, 6144), (28672, 4096), (4096, 28672), (4096, 14336), (14336, 4096)]:
+        rows, head, tail = plan(16512, N, K)
+        assert (rows, head) == (16384, 7) and tail in (4, 5, 6)
+    for K in (128, 256, 512):
+        assert plan(16512, 4096, K) == (16512, 7, -1)
+    assert plan(2048, 4096, 4096)[0] == 2048        # nothing left over: one launch
+    assert L.lib().lf_gemm_plan(16, 16, 0, 0, None, None, None) == L.LF_EINVAL
+
+
 def test_python_layer_refuses_cpu_tensors():
     from lorafusion_amd.ops.lora_v1 import fused_linear_lora
     from lorafusion_amd.ops.nf4 import QuantState, dequantize_nf4_triton

@@ -134,6 +134,41 @@ def test_one_adapter_equals_single_path():
     assert torch.equal(ym, ys)
 
 
+def test_adapter_in_two_segments_accumulates_through_autograd():
+    """The C ABI writes one dA / dB per segment.  At the autograd layer an adapter whose tokens sit in two separate
+    row ranges is passed once per range: each occurrence gets its segment's gradient and autograd adds them, which
+    is the gradient of the adapter over both ranges (oracle: the two segments' gradients summed)."""
+    from lorafusion_amd.ops.multi_lora import fused_linear_multi_lora, prepare_multi_lora_batch_info
+
+    seq, ranks, p_list, scales = [200, 150, 90], [16, 16, 16], [0.1, 0.0, 0.1], [2.0, 0.5, 2.0]
+    d = multi_inputs(seq, 256, 384, ranks, p_list, seed=11)
+    d["a_list"][2], d["b_list"][2] = d["a_list"][0], d["b_list"][0]      # segment 2 belongs to adapter 0 again
+    info = prepare_multi_lora_batch_info(seq, [0, 1, 0], ranks, p_list, scales, 128, output_dtype=torch.float32)
+    dev = "cuda"
+    x = d["x"].to(dev).requires_grad_(True)
+    a0, a1 = (d["a_list"][i].to(dev).requires_grad_(True) for i in (0, 1))
+    b0, b1 = (d["b_list"][i].to(dev).requires_grad_(True) for i in (0, 1))
+    y = fused_linear_multi_lora(
+        x.unsqueeze(0), d["w"].to(dev), lora_a_list=[a0, a1, a0], lora_b_list=[b0, b1, b0], seq_len_list=seq,
+        padded_seq_len_list=info.padded_seq_len_list, block_to_lookup_table=info.block_to_lookup_table,
+        block_to_dropout_p=info.block_to_dropout_p, block_to_alpha=info.block_to_alpha,
+        enable_dropout=info.enable_dropout, same_dropout_p_value=info.same_dropout_p_value, max_r=info.max_r,
+        dropout_mask=d["mask"].to(dev),
+    )
+    y.backward(d["dy"].to(dev).unsqueeze(0))
+    torch.cuda.synchronize()
+    ye, _ = lora_ref.linear_multi_lora_fwd_fp32(d["x"], d["w"], d["a_list"], d["b_list"], seq, d["padded"], scales, p_list,
+                                                d["mask"], None)
+    dxe, dae, dbe, _ = lora_ref.linear_multi_lora_bwd_fp32(d["dy"], d["x"], d["w"], d["a_list"], d["b_list"], seq,
+                                                           d["padded"], scales, p_list, d["mask"])
+    _close(y[0], ye, "y")
+    _close(x.grad, dxe, "dx")
+    _close(a0.grad, dae[0] + dae[2], "da of the adapter with two segments")
+    _close(b0.grad, dbe[0] + dbe[2], "db of the adapter with two segments")
+    _close(a1.grad, dae[1], "da[1]")
+    _close(b1.grad, dbe[1], "db[1]")
+
+
 def test_multi_errors():
     from lorafusion_amd.ops.multi_lora import fused_linear_multi_lora, prepare_multi_lora_batch_info
 
