@@ -286,7 +286,7 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
     static_assert(NWM == 2 && MNI >= 1, "mask staging: 32 rows x WN bytes per wave fit B_STAGE / NWAVES");
     char* mreg = ldsB + (NSTAGE - 1) * B_STAGE + wave * (B_STAGE / NWAVES);
     const int mrow = lane / MLPR, mg = lane % MLPR;
-    constexpr bool MEARLY = TM32 * MNI <= 8;  // all mask loads up front while they fit in 32 registers
+    constexpr bool MEARLY = TM32 * MNI <= 8 && TM * TN <= 16;  // all mask loads up front while they fit next to the operands of a chunk
     lf_u32x4 mv[TM32][MNI];
     const int mcol = min(n0 + wn * WN + mg * 16, p.N - 16);
     auto load_mask_band = [&](int ib) {
@@ -304,43 +304,70 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
       for (int ib = 0; ib < TM32; ib++) load_mask_band(ib);
     }
     const __amdgpu_buffer_rsrc_t rsrcR = __builtin_amdgcn_make_buffer_rsrc((void*)rp, 0, 0x7fffffff, 0x00020000);
-    // one MFMA k-step covers 32 rank columns; lanes whose 8 columns lie beyond R (or the rank) feed zeros
+    // Bit-packed keep-mask: the dword that holds the lane's four columns of each accumulator block (element n of a
+    // mask row = bit n & 7 of byte n >> 3).  Requested with the operands of the first chunk where the registers allow
+    // (up to 16 blocks per wave), else in one batch behind the MFMAs.
+    constexpr int GI = TM * TN <= 16 ? TM : (16 / TN > 0 ? 16 / TN : 1);   // block rows per batch of mask words
+    constexpr bool BITS_EARLY = GI == TM;
+    static_assert(TM % GI == 0, "whole batches");
+    uint32_t mw[GI][TN];
+    auto load_bits = [&](int i0) {
+#pragma unroll
+      for (int i = 0; i < GI; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const int gm = min(wrow0 + (i0 + i) * 16 + l16, p.M - 1);
+          const int col0 = min(n0 + wn * WN + j * 16 + kg * 4, p.N - 4);
+          mw[i][j] = *(const uint32_t*)(p.mask + (int64_t)gm * p.ldmask + ((col0 >> 5) << 2)) >> (col0 & 31);
+        }
+    };
+    // one MFMA k-step covers 32 rank columns; lanes whose 8 columns lie beyond R (or the rank) feed zeros.
+    // All loads of a chunk are requested before the first is used (the conditions sit outside the loops over the
+    // fragments): the term costs one memory round trip per chunk, not one per fragment -- with a branch and a wait
+    // per fragment the NN seed of a 128x256 tile took 17 us of an 80 us launch.
     for (int t = 0; t < (p.R + 31) / 32; t++) {
       const int r0 = t * 32 + kg * 8;
-      lf_u32x4 rf[TN];
+      lf_u32x4 rf[TN], lf[TM];
+      uint32_t e[NN ? TN : 1][8];
 #pragma unroll
-      for (int j = 0; j < TN; j++) {
-        int gn = min(n0 + wn * WN + j * 16 + l16, p.N - 1);
-        lf_u32x4 v = {0, 0, 0, 0};
-        if (r0 < rank) {
+      for (int j = 0; j < TN; j++) rf[j] = lf_u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < TM; i++) lf[i] = lf_u32x4{0, 0, 0, 0};
+      if (r0 < rank) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const int gn = min(n0 + wn * WN + j * 16 + l16, p.N - 1);
           if constexpr (!NN) {
-            v = *(const lf_u32x4*)(rp + (int64_t)gn * rank + r0);
+            rf[j] = *(const lf_u32x4*)(rp + (int64_t)gn * rank + r0);
           } else {
             // eight rows of one column: buffer loads that share a per-lane offset (row kg*8 of the
             // step, column gn) and take the row as a scalar offset, so the 8 x TN loads in flight
             // need no address registers of their own
             const uint32_t voff = (uint32_t)((kg * 8 * p.N + gn) * 2);
-            uint32_t e[8];
 #pragma unroll
-            for (int k = 0; k < 8; k++) e[k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcR, voff, (t * 32 + k) * p.N * 2, 0);
-            v[0] = e[0] | (e[1] << 16); v[1] = e[2] | (e[3] << 16);
-            v[2] = e[4] | (e[5] << 16); v[3] = e[6] | (e[7] << 16);
+            for (int k = 0; k < 8; k++) e[j][k] = __builtin_amdgcn_raw_buffer_load_b16(rsrcR, voff, (t * 32 + k) * p.N * 2, 0);
           }
         }
-        rf[j] = v;
       }
-      lf_u32x4 lf[TM];
+      if (r0 < p.R) {
 #pragma unroll
-      for (int i = 0; i < TM; i++) {
-        int gm = min(wrow0 + i * 16 + l16, p.M - 1);
-        lf_u32x4 v = {0, 0, 0, 0};
-        if (r0 < p.R) v = *(const lf_u32x4*)(L + (int64_t)gm * p.R + r0);
-        lf[i] = v;
+        for (int i = 0; i < TM; i++) {
+          const int gm = min(wrow0 + i * 16 + l16, p.M - 1);
+          lf[i] = *(const lf_u32x4*)(L + (int64_t)gm * p.R + r0);
+        }
       }
       if (t == 0) {
+        if (bits_mask && BITS_EARLY) load_bits(0);
         __builtin_amdgcn_sched_barrier(0);
         issue_first_tiles();
         __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (NN) {
+        if (r0 < rank) {
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+            rf[j] = lf_u32x4{e[j][0] | (e[j][1] << 16), e[j][2] | (e[j][3] << 16), e[j][4] | (e[j][5] << 16), e[j][6] | (e[j][7] << 16)};
+        }
       }
 #pragma unroll
       for (int i = 0; i < TM; i++)
@@ -359,15 +386,14 @@ gemm_lora_kernel(const LfGemmParams p, const LfSegTable seg) {
         }
       }
       const int r = h * 16 + l16;  // this lane's row of the band
+      if constexpr (!BITS_EARLY) {
+        if (bits_mask && i % GI == 0) load_bits(i);   // the next batch of block rows, all its words at once
+      }
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         acc[i][j] *= mult;
         if (bits_mask) {
-          // element n of a mask row = bit n & 7 of byte n >> 3: the lane's four columns are four bits of one dword
-          const int gm = min(wrow0 + i * 16 + l16, p.M - 1);
-          const int col0 = min(n0 + wn * WN + j * 16 + kg * 4, p.N - 4);
-          const uint32_t w = *(const uint32_t*)(p.mask + (int64_t)gm * p.ldmask + ((col0 >> 5) << 2));
-          const uint32_t bits = w >> (col0 & 31);
+          const uint32_t bits = mw[i % GI][j];
 #pragma unroll
           for (int e = 0; e < 4; e++) acc[i][j][e] = ((bits >> e) & 1u) ? acc[i][j][e] : 0.f;
         } else if (use_mask) {
