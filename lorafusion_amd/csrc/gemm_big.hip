@@ -32,11 +32,14 @@
 //    measured twice as slow), two rows per load instruction with 32 bytes of padding after each pair, and
 //    read with ds_read_b64_tr_b16: the rows that lanes read together sit in different pairs, hence on
 //    different banks.
-//  * The LoRA product seeds the accumulator before a tile's K loop (its operands are requested before
-//    the previous tile's epilogue); the forward scale is folded into the 16-bit L fragments (exact for
-//    powers of two), the backward 1/(1-p) is applied in fp32 together with the keep-mask select.
-//  * Epilogue: 16-row bands of a wave's sub-tile go through 4 KB of LDS per wave (beside the two stages) and
-//    leave as 16-byte stores that cover whole 256-byte rows of the sub-tile.
+//  * The LoRA product is added at the end of a tile: the forward's 64 MFMAs per 16 rank columns go onto the
+//    accumulators right behind the K loop; the dX product's term is formed block row by block row inside the
+//    epilogue, multiplied by 1/(1-p) and masked with the wave's keep bits on the way out.  The operands that
+//    are slow to fetch (keep bits from HBM, A_i rows that need a transposing read) land in the wave's own LDS
+//    area as direct-to-LDS loads during the tile's first K step.  The forward scale is folded into the 16-bit L
+//    fragments (exact for powers of two).
+//  * Epilogue: 16-row bands of a wave's sub-tile go through 4.5 KB of LDS per wave (beside the two stages) and
+//    leave as 16-byte non-temporal stores that cover whole 256-byte rows of the sub-tile.
 #include "lf_common.h"
 #include <type_traits>
 #include <utility>

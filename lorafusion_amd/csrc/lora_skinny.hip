@@ -250,14 +250,12 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
 #pragma unroll
     for (int c = 0; c < RT; c++) acc[nb][c] = lf_f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // The steps in flight form two register sets where there are at least two (ranks up to 32): the loads of one set
-  // are requested before the other set is used, so a wave's memory time and its integer / LDS / MFMA time overlap.
-  // All waves of a launch start together and would otherwise sit in the same phase -- everyone waiting for memory,
-  // then everyone computing.  (Two sets of the full depth cost occupancy and measured slower.)
-#ifndef LF_XA_MODE
-#define LF_XA_MODE 1
-#endif
-  constexpr int NSET = (LF_XA_MODE == 0) ? 1 : (XA_U >= 2 ? 2 : 1), UB = (LF_XA_MODE == 2 && NSET == 2) ? 1 : XA_U / NSET;
+  // Two register sets of one step each at ranks up to 32, one set above: the loads of one set are requested before
+  // the other set is used, so a wave's memory time and its integer / LDS / MFMA time overlap.  All waves of a launch
+  // start together and would otherwise sit in the same phase -- everyone waiting for memory, then everyone
+  // computing.  Measured at 16512 x 4096, rank 16, mask drawn in the kernel: one set of four steps 44.5 us, two sets
+  // of two steps 45.4 (126 registers: half the waves per SIMD), two sets of one step 42.2.
+  constexpr int NSET = XA_U >= 2 ? 2 : 1, UB = 1;
   lf_u32x4 xv[NSET][UB][2 * NB], av[NSET][UB][RT][2];
   lf_u32x4 uv[NSET][UB][ACT ? 2 * NB : 1];
   lf_u32x2 mv[NSET][UB][2 * NB];
