@@ -151,10 +151,11 @@ int lf_lora_fwd(const void* X, const void* W, const void* bias, const uint8_t* m
                 int K, int R, const lf_routing* routing, int dtype, void* stream);
 
 /* Whole forward with the mask drawn from `seed`: lf_lora_xa_seeded then lf_lora_xw_sb
- * (lorafusion/ops/lora_v1.py:87-129 called without a precomputed mask). */
+ * (lorafusion/ops/lora_v1.py:87-129 called without a precomputed mask).  workspace as for lf_lora_fwd
+ * (lf_workspace_bytes(LF_OP_FWD, ...); may be NULL: the product then never splits its contraction). */
 int lf_lora_fwd_seeded(const void* X, const void* W, const void* bias, uint8_t* mask_out, const void* const* a_ptrs,
-                       const void* const* b_ptrs, void* Y, void* S_out, int M, int N, int K, int R,
-                       const lf_routing* routing, uint64_t seed, int dtype, void* stream);
+                       const void* const* b_ptrs, void* Y, void* S_out, void* workspace, size_t ws_bytes, int M, int N,
+                       int K, int R, const lf_routing* routing, uint64_t seed, int dtype, void* stream);
 
 /* Whole backward: lf_lora_dys_dyb, lf_lora_da, and (dX != NULL) lf_lora_dyw_dsa.  Stands in
  * for _fused_linear_lora_backward (lorafusion/ops/lora_v1.py:132-166) and
@@ -296,15 +297,16 @@ int lf_silu_mul_fwd(const void* A, const void* B, void* C, int M, int I, int64_t
  * pass and the rank-r pass's own read of X disappear.  X_out is bit-identical to lf_silu_mul_fwd's output and S to
  * lf_lora_xa's on it.  mask: explicit keep-mask [M,K] or NULL; mask_out != NULL: the mask is drawn from `seed` as
  * lf_lora_xa_seeded draws it and written there (mask and mask_out exclude each other); both NULL: no dropout.
- * lf_swiglu_lora_fwd adds the fused GEMM of lf_lora_xw_sb on X_out: Y = X_out W^T + scale S B^T + bias.
+ * lf_swiglu_lora_fwd adds the fused GEMM of lf_lora_xw_sb on X_out: Y = X_out W^T + scale S B^T + bias
+ * (workspace as for lf_lora_fwd: lf_workspace_bytes(LF_OP_FWD, ...), or NULL).
  * The backward is lf_lora_bwd with X = X_out followed by lf_silu_mul_bwd on its dX. */
 int lf_lora_xa_silu_mul(const void* G, const void* U, int64_t ld, void* X_out, const uint8_t* mask, uint8_t* mask_out,
                         uint64_t seed, const void* const* a_ptrs, void* S, int M, int K, int R, const lf_routing* routing,
                         int dtype, void* stream);
 int lf_swiglu_lora_fwd(const void* G, const void* U, int64_t ld, void* X_out, const void* W, const void* bias,
                        const uint8_t* mask, uint8_t* mask_out, uint64_t seed, const void* const* a_ptrs,
-                       const void* const* b_ptrs, void* Y, void* S_out, int M, int N, int K, int R,
-                       const lf_routing* routing, int dtype, void* stream);
+                       const void* const* b_ptrs, void* Y, void* S_out, void* workspace, size_t ws_bytes, int M, int N,
+                       int K, int R, const lf_routing* routing, int dtype, void* stream);
 int lf_silu_mul_bwd(const void* dC, const void* A, const void* B, void* dA, void* dB, int M, int I, int64_t lddc,
                     int64_t lda, int64_t ldb, int64_t ldda, int64_t lddb, int dtype, void* stream);
 

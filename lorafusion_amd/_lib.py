@@ -100,7 +100,7 @@ def lib() -> ctypes.CDLL:
     l.lf_nf4_dequant.argtypes = [vp, vp, vp, vp, vp, vp, ctypes.c_int64, i, i, i, vp]
     l.lf_dropout_mask.argtypes = [vp, i, i, ctypes.c_float, rp, ctypes.c_uint64, vp]
     l.lf_lora_xa_seeded.argtypes = [vp, vp, vp, vp, i, i, i, rp, ctypes.c_uint64, i, vp]
-    l.lf_lora_fwd_seeded.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, rp, ctypes.c_uint64, i, vp]
+    l.lf_lora_fwd_seeded.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, i, i, i, i, rp, ctypes.c_uint64, i, vp]
     wp = ctypes.POINTER(NF4Weight)
     l.lf_nf4_lora_fwd.argtypes = [vp, wp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, rp, i, vp]
     l.lf_nf4_lora_bwd.argtypes = [vp, vp, wp, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, i, i, i, i, rp, i, vp]
@@ -112,7 +112,7 @@ def lib() -> ctypes.CDLL:
     l.lf_silu_mul_fwd.argtypes = [vp, vp, vp, i, i, i64, i64, i64, i, vp]
     l.lf_silu_mul_bwd.argtypes = [vp, vp, vp, vp, vp, i, i, i64, i64, i64, i64, i64, i, vp]
     l.lf_lora_xa_silu_mul.argtypes = [vp, vp, i64, vp, vp, vp, ctypes.c_uint64, vp, vp, i, i, i, rp, i, vp]
-    l.lf_swiglu_lora_fwd.argtypes = [vp, vp, i64, vp, vp, vp, vp, vp, ctypes.c_uint64, vp, vp, vp, vp, i, i, i, i, rp, i, vp]
+    l.lf_swiglu_lora_fwd.argtypes = [vp, vp, i64, vp, vp, vp, vp, vp, ctypes.c_uint64, vp, vp, vp, vp, vp, ctypes.c_size_t, i, i, i, i, rp, i, vp]
     l.lf_mask_pack.argtypes = [vp, vp, i, i, vp]
     l.lf_mask_unpack.argtypes = [vp, vp, i, i, vp]
     for name in EXPORTS:

@@ -172,15 +172,6 @@ int lf_lora_xa_silu_mul(const void* G, const void* U, int64_t ld, void* X_out, c
   return lf_launch_xa(G, U, ld, X_out, mask, mask_out, mb, seed, S, M, K, R, t, dtype, (hipStream_t)stream);
 }
 
-int lf_swiglu_lora_fwd(const void* G, const void* U, int64_t ld, void* X_out, const void* W, const void* bias,
-                       const uint8_t* mask, uint8_t* mask_out, uint64_t seed, const void* const* a_ptrs,
-                       const void* const* b_ptrs, void* Y, void* S_out, int M, int N, int K, int R,
-                       const lf_routing* routing, int dtype, void* stream) {
-  int rc = lf_lora_xa_silu_mul(G, U, ld, X_out, mask, mask_out, seed, a_ptrs, S_out, M, K, R, routing, dtype, stream);
-  if (rc != LF_OK) return rc;
-  return lf_lora_xw_sb(X_out, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
-}
-
 // lf_lora_xw_sb / lf_lora_dyw_dsa with a workspace for the split contraction of under-filled launches (the whole
 // forward / backward entry points pass theirs on; the single-product entry points have none and never split)
 static int xw_sb_ws(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs, void* Y,
@@ -206,6 +197,15 @@ static int xw_sb_ws(const void* X, const void* W, const void* bias, const void* 
 int lf_lora_xw_sb(const void* X, const void* W, const void* bias, const void* S, const void* const* b_ptrs,
                   void* Y, int M, int N, int K, int R, const lf_routing* routing, int dtype, void* stream) {
   return xw_sb_ws(X, W, bias, S, b_ptrs, Y, nullptr, 0, M, N, K, R, routing, dtype, stream);
+}
+
+int lf_swiglu_lora_fwd(const void* G, const void* U, int64_t ld, void* X_out, const void* W, const void* bias,
+                       const uint8_t* mask, uint8_t* mask_out, uint64_t seed, const void* const* a_ptrs,
+                       const void* const* b_ptrs, void* Y, void* S_out, void* workspace, size_t ws_bytes, int M, int N,
+                       int K, int R, const lf_routing* routing, int dtype, void* stream) {
+  int rc = lf_lora_xa_silu_mul(G, U, ld, X_out, mask, mask_out, seed, a_ptrs, S_out, M, K, R, routing, dtype, stream);
+  if (rc != LF_OK) return rc;
+  return xw_sb_ws(X_out, W, bias, S_out, b_ptrs, Y, workspace, ws_bytes, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
 }
 
 int lf_lora_dys_dyb(const void* dY, const void* S, const void* const* b_ptrs, void* dS, void* const* db_ptrs,
@@ -265,11 +265,11 @@ int lf_lora_fwd(const void* X, const void* W, const void* bias, const uint8_t* m
 }
 
 int lf_lora_fwd_seeded(const void* X, const void* W, const void* bias, uint8_t* mask_out, const void* const* a_ptrs,
-                       const void* const* b_ptrs, void* Y, void* S_out, int M, int N, int K, int R,
-                       const lf_routing* routing, uint64_t seed, int dtype, void* stream) {
+                       const void* const* b_ptrs, void* Y, void* S_out, void* workspace, size_t ws_bytes, int M, int N,
+                       int K, int R, const lf_routing* routing, uint64_t seed, int dtype, void* stream) {
   int rc = lf_lora_xa_seeded(X, mask_out, a_ptrs, S_out, M, K, R, routing, seed, dtype, stream);
   if (rc != LF_OK) return rc;
-  return lf_lora_xw_sb(X, W, bias, S_out, b_ptrs, Y, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
+  return xw_sb_ws(X, W, bias, S_out, b_ptrs, Y, workspace, ws_bytes, M, N, K, R, routing, dtype & ~LF_MASK_BITS, stream);
 }
 
 int lf_lora_bwd(const void* dY, const void* X, const void* W, const uint8_t* mask, const void* S,

@@ -518,9 +518,10 @@ def lora_forward_seeded(x, w, a_list, b_list, routing_c, R, seed: int, bias, *, 
     y = torch.empty((M, N), dtype=x.dtype, device=x.device)
     s = torch.empty((M, R), dtype=x.dtype, device=x.device)
     mask = torch.empty((M, K // 8), dtype=torch.uint8, device=x.device) if packed else torch.empty((M, K), dtype=torch.bool, device=x.device)
+    ws, nbytes = _ws(L.LF_OP_FWD, M, N, K, R, routing_c, x.device)
     rc = L.lib().lf_lora_fwd_seeded(L.ptr(x), L.ptr(w), L.ptr(bias), L.ptr(mask), L.ptr_array(a_list), L.ptr_array(b_list),
-                                    L.ptr(y), L.ptr(s), M, N, K, R, routing_c, ctypes.c_uint64(int(seed) & 0xFFFFFFFFFFFFFFFF),
-                                    _dt(x, mask, K), L.stream_of(x))
+                                    L.ptr(y), L.ptr(s), L.ptr(ws), nbytes, M, N, K, R, routing_c,
+                                    ctypes.c_uint64(int(seed) & 0xFFFFFFFFFFFFFFFF), _dt(x, mask, K), L.stream_of(x))
     L.check(rc, "lf_lora_fwd_seeded")
     return y, s, mask
 

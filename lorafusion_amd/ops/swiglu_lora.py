@@ -32,10 +32,12 @@ def _swiglu_lora_forward(gate, up, ld, w, a_list, b_list, routing_c, R, mask, dr
     mask_out = None
     if draw_seed is not None:
         mask_out = torch.empty((M, K // 8), dtype=torch.uint8, device=gate.device)   # drawn masks are kept bit-packed
+    ws, nbytes = hip_ops._ws(L.LF_OP_FWD, M, N, K, R, routing_c, gate.device)
     rc = L.lib().lf_swiglu_lora_fwd(
         gate.data_ptr(), up.data_ptr(), ld, x.data_ptr(), L.ptr(w), L.ptr(bias), L.ptr(mask), L.ptr(mask_out),
         ctypes.c_uint64(int(draw_seed or 0) & 0xFFFFFFFFFFFFFFFF), L.ptr_array(a_list), L.ptr_array(b_list), y.data_ptr(),
-        s.data_ptr(), M, N, K, R, routing_c, hip_ops._dt(gate, mask_out if mask_out is not None else mask, K), L.stream_of(gate))
+        s.data_ptr(), L.ptr(ws), nbytes, M, N, K, R, routing_c,
+        hip_ops._dt(gate, mask_out if mask_out is not None else mask, K), L.stream_of(gate))
     L.check(rc, "lf_swiglu_lora_fwd")
     return x, y, s, (mask_out if mask_out is not None else mask)
 
