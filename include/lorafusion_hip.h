@@ -97,8 +97,11 @@ typedef struct lf_routing {
 
 int lf_version(void);
 const char* lf_strerror(int code);
-/* Bytes of `workspace` the entry point(s) behind `op` need for this shape.  0 also for a shape or routing
- * the entry point itself would refuse (M <= 0, R not a multiple of 16 in 16..128, a tiled dimension
+/* Bytes of `workspace` the entry point(s) behind `op` use for this shape: the fp32 partial sums of
+ * the rank-r passes, which a call must be given, and for LF_OP_FWD / BWD / NF4_* the fp32 partial
+ * tiles of a split contraction (launches with few tiles and a long K: left-over rows of a packed
+ * batch, short batches), which a call skips when the workspace is smaller or NULL.  0 also for a
+ * shape or routing the entry point itself would refuse (M <= 0, R not a multiple of 16 in 16..128, a tiled dimension
  * -- N for DYS_DYB / BWD / NF4_*, K for XA / DA / FWD / BWD / NF4_* -- that is not a positive multiple
  * of 128, bad routing): the size query never fails harder than the call. */
 size_t lf_workspace_bytes(int op, int M, int N, int K, int R, const lf_routing* routing);
@@ -168,7 +171,8 @@ int lf_lora_bwd(const void* dY, const void* X, const void* W, const uint8_t* mas
 
 /* lf_lora_bwd without a workspace argument, for callers that cannot allocate device memory (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
- * counterpart in the reference.  The fp32 partial sums of the rank-r passes go to a buffer of
+ * counterpart in the reference.  The fp32 partial sums of the rank-r passes (and the partial tiles
+ * of the dX product's split contraction, where it has one) go to a buffer of
  * LF_STATIC_SCRATCH_BYTES that is part of the library's device image (one copy per GPU, held until
  * the process ends); the call allocates and frees nothing.  A call that needs more than the buffer
  * holds (lf_workspace_bytes(LF_OP_BWD, ...) > LF_STATIC_SCRATCH_BYTES) returns LF_ESTATIC and
