@@ -121,6 +121,16 @@ def test_8b_layer_projections(K, N):
     _run_multi(16384, K, N, [16] * 4, [0.0, 0.05, 0.1, 0.1], [1.0, 2.0, 2.0, 4.0])
 
 
+@pytest.mark.parametrize("tokens,K,N,n_adapters,seed", [(2048, 5120, 5120, 2, 1), (4096, 5120, 5120, 4, 0),
+                                                        (8192, 5120, 5120, 4, 0), (2048, 8192, 8192, 2, 1)])
+def test_kernel_grid_shapes(tokens, K, N, n_adapters, seed):
+    """The square shapes of the reference's kernel benchmark grid that no layer above has (hidden 5120: 20 tile
+    columns of 256, a K of 80 steps of 64; 2048 tokens x 8192: one round of 128x256 tiles), adapters of r=16.  (Seeds
+    whose segments all hold several hundred tokens: sums over a handful of rows are covered by the few-term
+    regression list of test_gpu_layer_fullsize.py, with the bound that applies to them.)"""
+    _run_multi(tokens, K, N, [16] * n_adapters, [0.05, 0.1, 0.0, 0.1][:n_adapters], [2.0, 1.0, 2.0, 4.0][:n_adapters], seed=seed)
+
+
 @pytest.mark.parametrize("K,N", [(8192, 8192), (8192, 1024), (8192, 10240), (8192, 28672), (8192, 57344), (28672, 8192)])
 def test_70b_layer_projections_nf4(K, N):
     """8192 tokens, 8 adapters r=64, base weight quantised to NF4 and dequantised on the device; the separate
