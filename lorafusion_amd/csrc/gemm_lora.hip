@@ -817,8 +817,8 @@ static int choose_split(int M, int N, int K, bool allow_big, int* cfg_head, int*
 // So: when the planned tiles fill less than half of the chip's workgroup slots, the launch moves to the 128x64 tile (up
 // to 256 rows) or the eight-wave 256x256 tile (more rows) in as many slices as give every compute unit a workgroup,
 // provided a slice keeps at least 48 K steps on the small tile and 192 on the large one (their fixed cost per
-// workgroup: pipeline fill and an fp32 store of the tile), at most 16 slices and at most kKsplitMaxBytes of partial
-// tiles.  A function of the shape, the planned tile and the routing block alone: a call that is given the workspace
+// workgroup: pipeline fill and an fp32 store of the tile) and the small tile gets at least three slices, at most 16
+// slices and at most kKsplitMaxBytes of partial tiles.  A function of the shape, the planned tile and the routing block alone: a call that is given the workspace
 // lf_workspace_bytes names always makes the same split, so its result does not depend on who calls.
 constexpr size_t kKsplitMaxBytes = (size_t)64 << 20;
 struct KSplit { int cfg, n, steps; };
@@ -843,7 +843,7 @@ static KSplit ksplit_for(int M, int N, int K, int cfg, int routing_block) {
   n = std::min(n, (long)(nk / min_steps));
   const size_t slice = (size_t)M * N * sizeof(float);
   n = std::min(n, (long)(kKsplitMaxBytes / slice));
-  if (n < 2) return none;
+  if (n < (cand == 6 ? 3 : 2)) return none;   // two slices of the small tile only pay for the second kernel (22 -> 24 us at K = 4096)
   int steps = (int)((nk + n - 1) / n);
   steps += steps & 1;                                         // an even number of steps per slice (K / BK is even)
   return {cand, (nk + steps - 1) / steps, steps};             // no empty slice

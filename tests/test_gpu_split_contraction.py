@@ -28,13 +28,13 @@ def _split_bytes(op, M, N, K, R, routing):
 
 
 @pytest.mark.parametrize("M,K,N,r,p,dtype,bias,sized", [
-    (128, 4096, 256, 16, 0.1, torch.bfloat16, False, "fwd"),     # Y over K = 4096 in two slices of 128x64 tiles
-    (128, 4096, 8192, 16, 0.1, torch.bfloat16, False, "both"),   # and dX [128, 4096] over N = 8192 in four
+    (128, 8192, 256, 16, 0.1, torch.bfloat16, False, "fwd"),     # Y over K = 8192 in five slices of 128x64 tiles
+    (128, 4096, 8192, 16, 0.1, torch.bfloat16, False, "bwd"),    # dX [128, 4096] over N = 8192 in four
     (200, 6144, 2048, 32, 0.1, torch.bfloat16, True, "fwd"),     # ragged rows, bias added by the second kernel
     (64, 8192, 384, 16, 0.0, torch.float16, True, "fwd"),        # fp16, no dropout
     (300, 12288, 512, 64, 0.2, torch.bfloat16, False, "fwd"),    # more than 256 rows: eight-wave 256x256 tiles, rank 64
     (384, 512, 12288, 16, 0.1, torch.bfloat16, False, None),     # the same for dX (its slices fit the rank-r passes' bytes)
-    (1, 4096, 128, 16, 0.1, torch.bfloat16, False, "fwd"),       # a single token
+    (1, 8192, 128, 16, 0.1, torch.bfloat16, False, "fwd"),       # a single token
 ])
 def test_single_adapter_split(M, K, N, r, p, dtype, bias, sized):
     from lorafusion_amd import _lib as L
@@ -44,9 +44,9 @@ def test_single_adapter_split(M, K, N, r, p, dtype, bias, sized):
     routing = L.single_routing(r, 2.0, p)
     R = L.round_rank(r)
     # the size query shows the split where its partial tiles are the largest use of the workspace
-    if sized in ("fwd", "both"):
+    if sized == "fwd":
         assert _split_bytes(L.LF_OP_FWD, M, N, K, R, routing) > _split_bytes(L.LF_OP_XA, M, N, K, R, routing)
-    if sized == "both":
+    if sized == "bwd":
         rank_r = max(_split_bytes(L.LF_OP_DYS_DYB, M, N, K, R, routing), _split_bytes(L.LF_OP_DA, M, N, K, R, routing))
         assert _split_bytes(L.LF_OP_BWD, M, N, K, R, routing) > rank_r
     d = single_inputs(M, K, N, r, p=p, seed=3, dtype=dtype, bias=bias)
