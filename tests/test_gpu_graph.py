@@ -55,6 +55,51 @@ def test_forward_backward_replay_matches_eager():
             assert torch.equal(g, e), f"replay {replay}: output {k} differs from the eager call"
 
 
+def test_split_contraction_and_seeded_forward_replay_matches_eager():
+    """A short batch with long contractions: forward (mask drawn in the pass) and backward both split their K range
+    into slices whose fp32 partial tiles live in the call's workspace, which torch allocates inside the capture; the
+    second kernels read what the replay's own first kernels wrote."""
+    from lorafusion_amd import _lib as L
+    from lorafusion_amd.ops import hip_ops
+
+    M, K, N, r = 128, 5120, 5120, 16
+    routing = L.single_routing(r, 2.0, 0.1)
+    assert L.lib().lf_workspace_bytes(L.LF_OP_FWD, M, N, K, r, routing) > 0          # the forward splits
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn((M, K), generator=gen, device="cuda").to(torch.bfloat16)
+    dy = torch.randn((M, N), generator=gen, device="cuda").to(torch.bfloat16)
+    w = (torch.randn((N, K), generator=gen, device="cuda") * 0.02).to(torch.bfloat16)
+    a = (torch.randn((r, K), generator=gen, device="cuda") / 90.0).to(torch.bfloat16)
+    b = (torch.randn((N, r), generator=gen, device="cuda") * 0.01).to(torch.bfloat16)
+
+    def run():
+        y, s, mask = hip_ops.lora_forward_seeded(x, w, [a], [b], routing, r, 1234, None)
+        dx, da, db = hip_ops.lora_backward(dy, x, w, [a], [b], s, routing, r, mask, [r])
+        return [y, dx, *da, *db, mask]
+
+    run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        run()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            outs = run()
+    torch.cuda.synchronize()
+    for replay in range(3):
+        x.copy_(torch.randn(x.shape, generator=gen, device="cuda").to(x.dtype))
+        dy.copy_(torch.randn(dy.shape, generator=gen, device="cuda").to(dy.dtype))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        want = run()
+        torch.cuda.synchronize()
+        for k, (g, e) in enumerate(zip(got, want)):
+            assert torch.equal(g, e), f"replay {replay}: output {k} differs from the eager call"
+
+
 def test_norm_activation_and_prologue_replay_matches_eager():
     """RMSNorm forward / backward (with dw: two kernels and a workspace), SiLU-multiply, and the down projection with
     the activation as its prologue, captured once and replayed on fresh values."""
