@@ -191,7 +191,7 @@ def check_close(actual: torch.Tensor, expected: torch.Tensor, rtol: float = 1e-2
 
     Returns (ok, max_abs_err / max|e|, worst elementwise excess).
     """
-    a, e = actual.double(), expected.double()
+    a, e = actual.detach().double(), expected.detach().double()
     if atol is None:
         atol = 1e-2 * float(e.pow(2).mean().sqrt())
     err = (a - e).abs()
