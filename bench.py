@@ -409,10 +409,13 @@ def nf4_block(dev) -> dict:
     return {name: nf4_dequant_block(dev, shp, fill=True) for name, shp in shapes.items()}
 
 
-def gemm_ref_block(dev, reps: int = 20) -> dict:
+def gemm_ref_block(dev, reps: int = 20, zero: bool = False) -> dict:
     """`--only gemm_ref`: the plain GEMMs of the 8B layer's largest shapes through this library (lf_gemm: the persistent
     kernel without a LoRA term) and through torch.matmul (hipBLASLt), same tensors, same process -- the run the
-    counter comparison in profiles/ is taken from."""
+    counter comparison in profiles/ is taken from.  `--only gemm_ref_zero`: the same launches on all-zero operands:
+    identical instruction streams and memory traffic, no switching in the multipliers.  What the two kernels gain
+    there is what the chip's power management takes from them on real data; it says nothing about throughput on real
+    data and is reported for that comparison only."""
     from lorafusion_amd.ops import hip_ops
 
     out = {}
@@ -421,6 +424,9 @@ def gemm_ref_block(dev, reps: int = 20) -> dict:
         g = torch.Generator(device=dev).manual_seed(0)
         a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
         b = (torch.randn(N, K, generator=g, device=dev) if trans_b else torch.randn(K, N, generator=g, device=dev)).to(torch.bfloat16)
+        if zero:
+            a.zero_()
+            b.zero_()
         fl = 2.0 * M * N * K
         t_lib = event_time_ms(lambda: hip_ops.gemm(a, b, trans_b=trans_b), reps)
         t_ref = event_time_ms(lambda: torch.matmul(a, b.T if trans_b else b), reps)
@@ -669,7 +675,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload (c4), its roofline and the CPU baseline")
-    ap.add_argument("--only", choices=sorted(WORKLOADS) + ["norm_act", "nf4", "gemm_ref", "fig5"], default=None,
+    ap.add_argument("--only", choices=sorted(WORKLOADS) + ["norm_act", "nf4", "gemm_ref", "gemm_ref_zero", "fig5"], default=None,
                     help="run one workload through the raw ops and print its entry alone (for profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -694,8 +700,10 @@ def main():
     if args.only == "nf4":
         print(json.dumps({"metric": "nf4_dequant", **nf4_block(dev)}))
         return
-    if args.only == "gemm_ref":
-        print(json.dumps({"metric": "plain GEMM: lf_gemm vs torch.matmul (hipBLASLt)", **gemm_ref_block(dev)}))
+    if args.only in ("gemm_ref", "gemm_ref_zero"):
+        zero = args.only == "gemm_ref_zero"
+        print(json.dumps({"metric": "plain GEMM: lf_gemm vs torch.matmul (hipBLASLt)" + (", all-zero operands" if zero else ""),
+                          **gemm_ref_block(dev, zero=zero)}))
         return
     if args.only == "fig5":
         print(json.dumps({"metric": "fig5 grid", **fig5_block(argparse.Namespace(steps=max(5, args.steps // 2), warmup=2), dev)}))
@@ -734,6 +742,7 @@ def main():
         res["workloads"] = {name: raw_workload(name, args if name == "c2" else small, dev)
                             for name in ("c1", "c2", "c3", "c4_qkv_merged", "c4_separate", "c5")}
         res["workloads"]["fig5"] = fig5_block(small, dev)
+        res["gemm_ref"] = {"random_operands": gemm_ref_block(dev, reps=10), "all_zero_operands": gemm_ref_block(dev, reps=10, zero=True)}
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline_c4()
     print(json.dumps(res))
