@@ -267,8 +267,13 @@ lora_xa_kernel(const T* __restrict__ X, const T* __restrict__ U, int64_t ldx, T*
       if (s < nsteps) {
 #pragma unroll
         for (int i = 0; i < 2 * NB; i++) {
-          xv[b][u][i] = *((const lf_u32x4*)(xrow[i] + s * 64));
-          if constexpr (ACT) uv[b][u][i] = *((const lf_u32x4*)((const char*)(xrow[i] + s * 64) + u_off));
+          if constexpr (ACT) {
+            // gate and up are read once, here: loads that do not allocate in the caches
+            xv[b][u][i] = __builtin_nontemporal_load((const lf_u32x4*)(xrow[i] + s * 64));
+            uv[b][u][i] = __builtin_nontemporal_load((const lf_u32x4*)((const char*)(xrow[i] + s * 64) + u_off));
+          } else {
+            xv[b][u][i] = *((const lf_u32x4*)(xrow[i] + s * 64));
+          }
           if constexpr (!GEN) {
             // (bit format: the byte is only requested here and spread into eight bytes where it is used, so that no
             // wait for it separates the loads of a batch)

@@ -243,8 +243,9 @@ silu_mul_fwd_kernel(const lf_u32x4* __restrict__ a, const lf_u32x4* __restrict__
 #pragma unroll
   for (int i = 0; i < ROWS; i++)
     if (row0 + i < M) {
-      av[i] = a[(int64_t)(row0 + i) * lda + col];
-      bv[i] = b[(int64_t)(row0 + i) * ldb + col];
+      // (streams read once and written once: neither loads nor stores allocate in the caches)
+      av[i] = __builtin_nontemporal_load(a + (int64_t)(row0 + i) * lda + col);
+      bv[i] = __builtin_nontemporal_load(b + (int64_t)(row0 + i) * ldb + col);
     }
 #pragma unroll
   for (int i = 0; i < ROWS; i++)
@@ -266,9 +267,9 @@ silu_mul_bwd_kernel(const lf_u32x4* __restrict__ dc, const lf_u32x4* a, const lf
 #pragma unroll
   for (int i = 0; i < ROWS; i++)
     if (row0 + i < M) {
-      cv[i] = dc[(int64_t)(row0 + i) * lddc + col];
-      av[i] = a[(int64_t)(row0 + i) * lda + col];
-      bv[i] = b[(int64_t)(row0 + i) * ldb + col];
+      cv[i] = __builtin_nontemporal_load(dc + (int64_t)(row0 + i) * lddc + col);
+      av[i] = __builtin_nontemporal_load(a + (int64_t)(row0 + i) * lda + col);
+      bv[i] = __builtin_nontemporal_load(b + (int64_t)(row0 + i) * ldb + col);
     }
 #pragma unroll
   for (int i = 0; i < ROWS; i++)
@@ -440,7 +441,7 @@ int lf_silu_mul_fwd(const void* A, const void* B, void* C, int M, int I, int64_t
                     int dtype, void* stream) {
   const int rc = act_check(M, I, {A, B, C}, {lda, ldb, ldc});
   if (rc != LF_OK) return rc;
-  constexpr int ROWS = 4;
+  constexpr int ROWS = 2;
   const int ic = I / 8, col_blocks = (ic + ACT_THREADS - 1) / ACT_THREADS;
   const int64_t grid = (int64_t)col_blocks * ((M + ROWS - 1) / ROWS);
   if (grid > 0x7fffffffLL) return LF_ELIMIT;
