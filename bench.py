@@ -145,15 +145,23 @@ def graph_time_ms(fn, reps: int, inner: int = 10) -> float:
     return e0.elapsed_time(e1) / (n * inner)
 
 
-def wall_time_ms(fn, steps: int, warmup: int) -> float:
+def wall_time_ms(fn, steps: int, warmup: int, min_ms: float = 0.0):
+    """Wall clock per step over `steps` back-to-back steps between two synchronisations.  min_ms > 0 (the sub-millisecond
+    workloads beside the headline): when the timed region came out shorter than that, it is timed again over as many
+    steps as fill it -- the closing synchronisation and the first launch cost about half a millisecond, which 20 steps
+    of 0.15 ms do not amortise.  Returns (ms per step, steps timed)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    while True:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        total = (time.perf_counter() - t0) * 1e3
+        if total >= min_ms:
+            return total / steps, steps
+        steps = int(steps * min_ms / max(total, 1e-3) * 1.1) + 1
 
 
 class Batch:
@@ -324,7 +332,7 @@ def raw_workload(name: str, args, dev, breakdown: bool = True) -> dict:
         for lin in linears:
             lin.step()
 
-    ms = wall_time_ms(step, args.steps, args.warmup)
+    ms, steps_timed = wall_time_ms(step, args.steps, args.warmup, min_ms=40.0)
     flops = sum(lin.flops for lin in linears)
     per = {}
     for lin in linears:
@@ -332,7 +340,7 @@ def raw_workload(name: str, args, dev, breakdown: bool = True) -> dict:
         per[lin.name] = {"K": lin.k, "N": lin.n, "ms": round(pm, 4), "TFLOP/s": round(lin.flops / (pm * 1e-3) / 1e12, 1)}
     res = {
         "workload": NAMES[name], "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 4),
-        "tokens": batch.tokens, "rows_launched": batch.Mp, "rank": batch.rank, "adapters": batch.n_ad, "nf4_base": batch.nf4,
+        "steps_timed": steps_timed, "tokens": batch.tokens, "rows_launched": batch.Mp, "rank": batch.rank, "adapters": batch.n_ad, "nf4_base": batch.nf4,
         "seq_len_list": batch.seq, "linears": per,
     }
     if batch.nf4:
@@ -340,7 +348,7 @@ def raw_workload(name: str, args, dev, breakdown: bool = True) -> dict:
             for lin in linears:
                 lin.step(keep_dense=True)
 
-        mk = wall_time_ms(step_keep, args.steps, args.warmup)
+        mk, _ = wall_time_ms(step_keep, args.steps, args.warmup, min_ms=40.0)
         res["reuse_dequantized_weight"] = {
             "ms_per_step": round(mk, 4), "TFLOP/s": round(flops / (mk * 1e-3) / 1e12, 2),
             "note": "the forward's dequantised weight is kept for the backward that follows it: one NF4 dequantisation per "
@@ -366,7 +374,7 @@ def raw_workload(name: str, args, dev, breakdown: bool = True) -> dict:
             with torch.cuda.graph(graph, stream=side):
                 keep = lin.step()
         torch.cuda.synchronize()
-        mg = wall_time_ms(graph.replay, args.steps, args.warmup)
+        mg, _ = wall_time_ms(graph.replay, args.steps, args.warmup, min_ms=40.0)
         del keep
         res["hipgraph_replay"] = {"ms_per_step": round(mg, 4), "TFLOP/s": round(flops / (mg * 1e-3) / 1e12, 2)}
     del linears
@@ -575,7 +583,7 @@ def layer_c4(args, dev):
         for p in params:
             p.grad = None
 
-    ms = wall_time_ms(step, args.steps, args.warmup)
+    ms, _ = wall_time_ms(step, args.steps, args.warmup)
     flops = sum(linear_flops(tokens, k, n, rank) for _, k, n in projs)
     per = {}
     for name, k, n in projs:

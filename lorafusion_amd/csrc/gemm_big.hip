@@ -46,18 +46,24 @@
 
 namespace {
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int STAGE_A = BM * BK * 2;
+// workgroup tile: 32 TI rows x 256 columns (TI = 8: 256x256, a wave owns 128x128; TI = 4: 128x256, a wave owns 64x128)
+constexpr int BN = 256, BK = 64;
 // NN operand B [64 k-rows, 256 columns]: rows of 512 bytes stored in pairs (k-rows r and r+4: the 1024 bytes one wave
 // instruction of the direct load fills), 32 bytes of padding after every pair
 constexpr int PAIR_NN = 1024 + 32;
-template <bool NN> struct Lds {
+template <bool NN, int TI> struct Lds {
+  static constexpr int STAGE_A = TI * 32 * BK * 2;
   static constexpr int STAGE_B = NN ? 32 * PAIR_NN : BN * BK * 2;
   static constexpr int STAGE = STAGE_A + STAGE_B;
-  // per wave behind the stages: the epilogue's band buffer (4.5 KB), before that the landing area of a tile's LoRA
-  // operands (dX product: 4 KB of A_i rows + 2 KB of keep bits)
-  static constexpr int EP_OFF = 2 * STAGE, EP_WAVE = 6144, BYTES = EP_OFF + 4 * EP_WAVE;
-  static_assert(BYTES <= 160 * 1024, "two stages and the epilogue bands fit the LDS of a CU");
+  // 256-row tile: two stages; per wave behind them 6 KB: the epilogue's band buffer (4 KB), before that the landing
+  // area of a tile's LoRA operands (dX product: 4 KB of A_i rows + 2 KB of keep bits).
+  // 128-row tile: three stages (a K step is half as long, so a stage's loads are given two steps to land) and nothing
+  // behind them: a wave's 5 KB (4 KB of A_i rows or the band, 1 KB of keep bits) lie in the stage of the tile's last K
+  // step, in the part that no load writes to between that step's barrier and the next tile's first step.
+  static constexpr int NST = TI == 8 ? 2 : 3;
+  static constexpr int EP_OFF = NST * STAGE, EP_WAVE = TI == 8 ? 6144 : 5120;
+  static constexpr int BYTES = TI == 8 ? EP_OFF + 4 * EP_WAVE : EP_OFF;
+  static_assert(BYTES <= 160 * 1024, "stages, landing area and epilogue bands fit the LDS of a CU");
 };
 
 template <typename T> struct BigOp;
@@ -136,7 +142,7 @@ __device__ __forceinline__ void sfor(F&& f) {
 
 // LORA = false: the instance for calls without a LoRA term (the seed code is compiled out, which also keeps that
 // instance free of register spills: a kernel that needs scratch memory pays for it at every launch).
-template <typename T, bool NN, bool LORA>
+template <typename T, bool NN, bool LORA, int TI>
 __global__ void __launch_bounds__(256, 1)
 gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub (buffer-resource types are device-only)
@@ -145,7 +151,12 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  constexpr int STAGE = Lds<NN>::STAGE, EP_OFF = Lds<NN>::EP_OFF, EP_WAVE = Lds<NN>::EP_WAVE;
+  constexpr int BM = TI * 32, WROWS = TI * 16;   // rows of the workgroup's tile, of a wave's sub-tile
+  constexpr int NL = TI + 8;                     // tile loads per wave and stage (TI of A, 8 of B)
+  constexpr int NM = TI * 8;                     // MFMAs per wave and sub-step
+  constexpr int STAGE_A = Lds<NN, TI>::STAGE_A, STAGE = Lds<NN, TI>::STAGE, EP_OFF = Lds<NN, TI>::EP_OFF, EP_WAVE = Lds<NN, TI>::EP_WAVE;
+  constexpr int NST = Lds<NN, TI>::NST;          // LDS stages
+  constexpr int NH1 = TI + 2;                    // three stages: loads [0, NH1) of a stage (A, the first two of B) are its first half
 
   const int total = p.grid_m * p.grid_n;
   const int G = gridDim.x, wg = blockIdx.x;
@@ -218,19 +229,18 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   const uint32_t m0a = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + wave * 1024));
   const uint32_t m0b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + STAGE_A + wave * (NN ? PAIR_NN : 1024)));
   constexpr int M0B_STEP = NN ? 4 * PAIR_NN : 4096;
-  int istr[16];  // scalar offset of load idx relative to the stage's first byte of its operand
+  int istr[NL];  // scalar offset of load idx (idx < TI: operand A, else B) relative to the stage's first byte of its operand
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    istr[i] = __builtin_amdgcn_readfirstlane(i * a_istride);
-    istr[8 + i] = __builtin_amdgcn_readfirstlane(i * b_istride);
-  }
+  for (int i = 0; i < TI; i++) istr[i] = __builtin_amdgcn_readfirstlane(i * a_istride);
+#pragma unroll
+  for (int i = 0; i < 8; i++) istr[TI + i] = __builtin_amdgcn_readfirstlane(i * b_istride);
   // Scalars the K loop uses come through an empty asm: the compiler then waits for the kernel-argument loads behind
   // them here, once, instead of keeping a "scalar load may be pending" wait inside the loop, where it would also wait
   // for the fragment reads in flight (which it cannot see).
   int nk_s = nk, kb_mul = BK * (int)p.ldb * 2;
   asm volatile("" : "+s"(nk_s), "+s"(kb_mul));
 #pragma unroll
-  for (int i = 0; i < 16; i++) asm volatile("" : "+s"(istr[i]));
+  for (int i = 0; i < NL; i++) asm volatile("" : "+s"(istr[i]));
   // byte offsets (operand A, operand B) of K step k of a tile whose walk starts at kstart
   auto kbase = [&](int kstart, int k, int& ka, int& kb) __attribute__((always_inline)) {
     int kp = kstart + k;
@@ -244,16 +254,16 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   auto issue_load = [&](lf_u32x4 rsrc, uint32_t voff, int soff) __attribute__((always_inline)) {
     asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff) : "memory");
   };
-  // all 16 loads of K step k of the tile behind `src` into stage `stage` (prologue only: no MFMAs to hide behind)
-  auto load_stage = [&](const LoadSrc& src, int k, int stage) __attribute__((always_inline)) {
+  // all loads of K step k of the tile behind `src` into stage `stage` (prologue only: no MFMAs to hide behind)
+  auto load_stage = [&](const LoadSrc& src, int k, int stage, auto COUNT) __attribute__((always_inline)) {
     int ka, kb;
     kbase(src.kstart, k, ka, kb);
-    sfor<16>([&](auto I) {
+    sfor<COUNT.value>([&](auto I) {
       constexpr int idx = I.value;
-      if constexpr (idx < 8) set_m0(m0a + stage * STAGE, std::integral_constant<int, idx * 4096>{});
-      else set_m0(m0b + stage * STAGE, std::integral_constant<int, (idx - 8) * M0B_STEP>{});
+      if constexpr (idx < TI) set_m0(m0a + stage * STAGE, std::integral_constant<int, idx * 4096>{});
+      else set_m0(m0b + stage * STAGE, std::integral_constant<int, (idx - TI) * M0B_STEP>{});
       asm volatile("s_nop 0" ::: "memory");
-      issue_load(idx < 8 ? src.ra : src.rb, idx < 8 ? a_voff : b_voff, (idx < 8 ? ka : kb) + istr[idx]);
+      issue_load(idx < TI ? src.ra : src.rb, idx < TI ? a_voff : b_voff, (idx < TI ? ka : kb) + istr[idx]);
     });
   };
 
@@ -266,19 +276,21 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   };
   using S0 = integral_constant<int, 0>;
   using S1 = integral_constant<int, 1>;
-  constexpr int RDS = 3;   // a fragment read every RDS MFMAs
-  constexpr int LDP = 4;   // a tile load every LDP MFMAs of sub-step 1 (denser issue queues up in the texture addresser: 2 and 3 measured 2-6 % slower)
+  constexpr int RDS = TI == 8 ? 3 : 2;   // a fragment read every RDS MFMAs
+  constexpr int LDP = NM / NL;           // a tile load every LDP MFMAs of sub-step 1 (256x256 tile: 4; denser issue queues up in the texture addresser there: 2 and 3 measured 2-6 % slower)
+  static_assert(RDS * NL <= NM && LDP >= 2, "a sub-step has a gap for every fragment read and two for every tile load");
   const T* __restrict__ Lp = (const T*)p.L;
   T* __restrict__ C = (T*)p.C;
   const uint16_t* bias16 = (const uint16_t*)p.bias;
 
-  // the first two stages of the first tile
+  // the first two stages of the first tile (three stages: and the first half of the third)
   Tile tile = tile_of(0);
   LoadSrc src = src_of(tile);
-  load_stage(src, 0, 0);
-  load_stage(src, 1, 1);
+  load_stage(src, 0, 0, integral_constant<int, NL>{});
+  load_stage(src, 1, 1, integral_constant<int, NL>{});
+  if constexpr (NST == 3) load_stage(src, 2, 2, integral_constant<int, NH1>{});
 
-  // Adapter of a wave's 128 rows: rank, skinny operand, multiplier, whether a keep-mask applies.  With a routing table
+  // Adapter of a wave's rows: rank, skinny operand, multiplier, whether a keep-mask applies.  With a routing table
   // these are two dependent scalar loads (table row, then the segment's pointer), so a tile's lookup is issued while
   // the previous tile computes and costs a latency only for a workgroup's first tile.
   struct Route { int rank; const T* rp; float mult; bool use_mask; };
@@ -309,26 +321,27 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
   };
   constexpr bool has_lora = LORA;   // the launcher picks the LORA instance exactly when there is a term (p.L != nullptr)
   Route route{};
-  if (has_lora) route = route_of(tile.m0 + wm * 128);
+  if (has_lora) route = route_of(tile.m0 + wm * WROWS);
   const int n16 = p.R >> 4;   // chunks of 16 rank columns (one 16x16x16 MFMA step each)
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the first tile's two stages (later tiles: waited for before the epilogue's stores)
-  int par = 0;  // LDS stage of the current tile's K step 0 (tiles follow each other through the two stages without a gap)
+  int par = 0;  // LDS stage of the current tile's K step 0 (tiles follow each other through the stages without a gap)
   for (int it = 0; it < n_my; it++) {
     // everything below is scoped to one tile: fragments, accumulators and LoRA operands do not live across tiles
     const Tile nxt_tile = it + 1 < n_my ? tile_of(it + 1) : tile;
     const LoadSrc nxt_src = src_of(nxt_tile);
     const int m0 = tile.m0, n0 = tile.n0;
-    const int wrow0 = m0 + wm * 128;
+    const int wrow0 = m0 + wm * WROWS;
     const Route rt = route;
-    if (has_lora) route = route_of(nxt_tile.m0 + wm * 128);  // in flight during this tile's K loop
+    if (has_lora) route = route_of(nxt_tile.m0 + wm * WROWS);  // in flight during this tile's K loop
 
-    lf_u32x4 fa[2][8], fb[2][8];
-    lf_f32x4 acc[8][8];
+    lf_u32x4 fa[2][TI], fb[2][8];
+    lf_f32x4 acc[TI][8];
     uint32_t fa_off[2], fb_off[2];
-    // one fragment read of sub-step KS of the stage at LDS byte offset `st`: idx < 8: A fragment idx; else B fragment idx-8
-    auto read_one = [&](auto SET, auto KS, uint32_t st, auto IDX) __attribute__((always_inline)) {
-      constexpr int idx = IDX.value, set = SET.value, ks = KS.value;
+    // one fragment read of sub-step KS of the stage at LDS byte offset `st`, the o-th of its sub-step: first the 8 B
+    // fragments, then the TI A fragments
+    auto read_one = [&](auto SET, auto KS, uint32_t st, auto ORD) __attribute__((always_inline)) {
+      constexpr int idx = ORD.value < 8 ? ORD.value + 8 : ORD.value - 8, set = SET.value, ks = KS.value;   // idx < 8: A fragment idx; else B fragment idx - 8
       if constexpr (idx < 8) {
         const uint32_t ad = fa_off[ks] + st;
         lf_u32x4 tmp;
@@ -360,14 +373,21 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     // requested behind the epilogue's stores: loads and stores share one counter and complete out of order with
     // respect to each other, so a wait for such a load would be a wait for the 128 KB of output stored just before.
     // The dX product (NN) therefore requests, during the tile's first K sub-step (the texture addresser is idle
-    // there), what it cannot fetch quickly afterwards -- the keep-mask bits of the wave's 128x128 block, which come
+    // there), what it cannot fetch quickly afterwards -- the keep-mask bits of the wave's block, which come
     // from HBM, and the first 16 rows of A_i over the wave's columns, which the MFMA needs transposed -- as
     // direct-to-LDS loads into the wave's own 6 KB behind the stages (the epilogue's band buffer, idle until then):
     // no registers are involved, and the data has landed by the vmcnt(0) of the tile's second K step (K >= 128).
     // The L fragments and the forward's B_i fragments are plain 8-byte loads issued right behind the K loop; they come
     // from L2, and their wait coincides with the wait for the next tile's stages that precedes the first store anyway.
     const bool sel = NN && LORA && p.mult_mode == 1 && rt.use_mask;   // keep-mask applies to this wave's rows
-    const uint32_t area = lds0 + EP_OFF + wave * EP_WAVE;               // this wave's 6 KB
+    // This wave's area.  Three stages: in the stage of the tile's last step, behind the first half of a stage's loads
+    // (operand B from its third load on): the last step's own reads of it end at its barrier, and the next load that
+    // writes there is issued in the next tile's first step.  The dX product's operands are requested into it during
+    // the last step's second sub-step and waited for right behind the K loop.
+    const uint32_t last_stage = (uint32_t)((par + nk - 1) % 3) * STAGE;
+    const uint32_t area = NST == 2 ? lds0 + EP_OFF + wave * EP_WAVE : lds0 + last_stage + STAGE_A + 2 * M0B_STEP + wave * EP_WAVE;
+    static_assert(NST == 2 || 4 * EP_WAVE <= 6 * 4096, "the four areas fit the second half of a stage's B part");
+    const uint32_t area_r = area, area_m = area + 4096;   // A_i rows, keep bits
     uint32_t rfl_voff = 0, mk_voff = 0;
     lf_u32x4 rsrcR{}, rsrcM{};
     int rfl_s0 = 0, rfl_step = 0, mk_step = 0;
@@ -382,17 +402,18 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       rfl_voff = (uint32_t)(((sl >> 4) * p.N + (sl & 15) * 8) * 2);
       rfl_s0 = (n0 + wn * 128) * 2;
       rfl_step = 4 * p.N * 2;
-      // keep bits: load q covers rows 64q + lane, 16 bytes (128 columns) each.  Without a mask the two loads read the
+      // keep bits: load q covers rows 64q + lane, 16 bytes (128 columns) each (TI / 4 loads).  Without a mask they read the
       // head of L (an inline-assembly statement under a run-time condition does not compile inside a generic lambda)
       const uint64_t mb = sel ? (uint64_t)(uintptr_t)(p.mask + (int64_t)wrow0 * p.ldmask + ((n0 + wn * 128) >> 3)) : (uint64_t)(uintptr_t)Lp;
       rsrcM = lf_u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)mb), (uint32_t)__builtin_amdgcn_readfirstlane((int)(mb >> 32)) & 0xffffu, 0x7fffffffu, 0x00020000u};
       mk_voff = sel ? (uint32_t)(sl * (int)p.ldmask) : 0u;
       mk_step = sel ? 64 * (int)p.ldmask : 0;
     }
-    constexpr int N_LORA_LOADS = (NN && LORA) ? 6 : 0;
+    constexpr int N_LORA_LOADS = (NN && LORA) ? 4 + TI / 4 : 0;
     // load `q` of the list above, issued in gaps 2q (M0) and 2q+1 of the tile's first sub-step
     auto lora_m0 = [&](auto Q) __attribute__((always_inline)) {
-      set_m0(area, integral_constant<int, Q.value * 1024>{});
+      if constexpr (Q.value < 4) set_m0(area_r, integral_constant<int, Q.value * 1024>{});
+      else set_m0(area_m, integral_constant<int, (Q.value - 4) * 1024>{});
     };
     auto lora_load = [&](auto Q) __attribute__((always_inline)) {
       constexpr int q = Q.value;
@@ -422,7 +443,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       const int l16 = fl & 15, kg = fl >> 4;
       const int key = (l16 >> 1) & 7;
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++) fa_off[ks] = lds0 + (wm * 128 + l16) * 128 + (((ks * 4 + kg) ^ key) << 4);
+      for (int ks = 0; ks < 2; ks++) fa_off[ks] = lds0 + (wm * WROWS + l16) * 128 + (((ks * 4 + kg) ^ key) << 4);
       if constexpr (!NN) {
 #pragma unroll
         for (int ks = 0; ks < 2; ks++) fb_off[ks] = lds0 + STAGE_A + (wn * 128 + l16) * 128 + (((ks * 4 + kg) ^ key) << 4);
@@ -441,7 +462,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
     barrier();   // both stages of this tile's first two K steps are in LDS (every wave has waited for its loads)
     {
       const uint32_t st = par * STAGE;
-      sfor<16>([&](auto I) { read_one(S0{}, S0{}, st, integral_constant<int, (I.value + 8) & 15>{}); });
+      sfor<NL>([&](auto I) { read_one(S0{}, S0{}, st, I); });
     }
     lgkm0();
     // K step s lives in stage (par + s) & 1.  Sub-step 1 of step s refills that stage with step s+2 of this tile; the
@@ -459,11 +480,11 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       int ka, kb;
       kbase(ld.kstart, lk, ka, kb);
       const uint32_t ma = m0a + cur, mb = m0b + cur;
-      int soff[16];
-      sfor<64>([&](auto MM) {
+      int soff[NL];
+      sfor<NM>([&](auto MM) {
         constexpr int m = MM.value;
-        if constexpr (m % RDS == 0 && m / RDS < 16) read_one(S1{}, S1{}, cur, integral_constant<int, (m / RDS + 8) & 15>{});
-        if constexpr (m % 4 == 2) soff[m / 4] = (m / 4 < 8 ? ka : kb) + istr[m / 4];
+        if constexpr (m % RDS == 0 && m / RDS < NL) read_one(S1{}, S1{}, cur, integral_constant<int, m / RDS>{});
+        if constexpr (m % LDP == LDP / 2 && m / LDP < NL) soff[m / LDP] = (m / LDP < TI ? ka : kb) + istr[m / LDP];
         if constexpr (FIRST.value && m < 2 * N_LORA_LOADS) {
           if constexpr (m % 2 == 0) lora_m0(integral_constant<int, m / 2>{});
           else lora_load(integral_constant<int, m / 2>{});
@@ -473,14 +494,14 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       });
       if constexpr (!FIRST.value) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads of step s+1 (issued a sub-step ago) have landed
       barrier();
-      sfor<64>([&](auto MM) {
+      sfor<NM>([&](auto MM) {
         constexpr int m = MM.value;
-        if constexpr (m % RDS == 0 && m / RDS < 16) read_one(S0{}, S0{}, nxt, integral_constant<int, (m / RDS + 8) & 15>{});
-        if constexpr (m % LDP == 0 && m / LDP < 16) {
-          if constexpr (m / LDP < 8) set_m0(ma, integral_constant<int, (m / LDP) * 4096>{});
-          else set_m0(mb, integral_constant<int, (m / LDP - 8) * M0B_STEP>{});
+        if constexpr (m % RDS == 0 && m / RDS < NL) read_one(S0{}, S0{}, nxt, integral_constant<int, m / RDS>{});
+        if constexpr (m % LDP == 0 && m / LDP < NL) {
+          if constexpr (m / LDP < TI) set_m0(ma, integral_constant<int, (m / LDP) * 4096>{});
+          else set_m0(mb, integral_constant<int, (m / LDP - TI) * M0B_STEP>{});
         }
-        if constexpr (m % LDP == 1 && m / LDP < 16) issue_load(m / LDP < 8 ? ld.ra : ld.rb, m / LDP < 8 ? a_voff : b_voff, soff[m / LDP]);
+        if constexpr (m % LDP == 1 && m / LDP < NL) issue_load(m / LDP < TI ? ld.ra : ld.rb, m / LDP < TI ? a_voff : b_voff, soff[m / LDP]);
         mfma_one(1, m, std::false_type{});
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -488,7 +509,71 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       lgkm0();
       __builtin_amdgcn_sched_barrier(0);
     };
-    {
+    // ------------------------------------------------------------ K loop over three stages (128-row tile)
+    // Step s lives in stage (par + s) % 3.  Its sub-step 0 issues the second half of step s+2's loads into the stage
+    // that died at the barrier of step s-1, its sub-step 1 the first half of step s+3's into its own stage, dead since
+    // this step's barrier: a stage's loads are issued over a whole step and have another step to land.  At the barrier
+    // of step s the loads of step s+1 must have landed: all but the 12 issued last.  Steps beyond the tile's last one
+    // are the next tile's first ones.  FIRST (a tile's step 0) waits for nothing: what it needs was waited for before
+    // the previous tile's stores (or the kernel's first loads), and a counted wait here would wait for those stores.
+    uint32_t cst = (uint32_t)par * STAGE;   // byte offset of the current step's stage
+    auto k_step3 = [&](const LoadSrc& l2, int k2, const LoadSrc& l3, int k3, auto FIRST, auto LAST) __attribute__((always_inline)) {
+      const uint32_t cur = cst;
+      const uint32_t nx1 = cur + STAGE >= 3 * STAGE ? cur + STAGE - 3 * STAGE : cur + STAGE;
+      const uint32_t nx2 = nx1 + STAGE >= 3 * STAGE ? nx1 + STAGE - 3 * STAGE : nx1 + STAGE;
+      int ka2, kb2, ka3, kb3;
+      kbase(l2.kstart, k2, ka2, kb2);
+      kbase(l3.kstart, k3, ka3, kb3);
+      const uint32_t mb2 = m0b + nx2, ma3 = m0a + cur, mb3 = m0b + cur;
+      int so = 0;
+      sfor<NM>([&](auto MM) {
+        constexpr int m = MM.value;
+        if constexpr (m % RDS == 0 && m / RDS < NL) read_one(S1{}, S1{}, cur, integral_constant<int, m / RDS>{});
+        // second half of step s+2: loads NH1 .. NL-1 (all of operand B), M0 and the scalar offset in gap 5i+1, the load in gap 5i+2
+        if constexpr (m % 5 == 1 && m / 5 < NL - NH1) {
+          constexpr int idx = NH1 + m / 5;
+          so = kb2 + istr[idx];
+          set_m0(mb2, integral_constant<int, (idx - TI) * M0B_STEP>{});
+        }
+        if constexpr (m % 5 == 2 && m / 5 < NL - NH1) issue_load(l2.rb, b_voff, so);
+        mfma_one(0, m, FIRST);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      if constexpr (!FIRST.value) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+      barrier();
+      sfor<NM>([&](auto MM) {
+        constexpr int m = MM.value;
+        if constexpr (m % RDS == 0 && m / RDS < NL) read_one(S0{}, S0{}, nx1, integral_constant<int, m / RDS>{});
+        // first half of step s+3: loads 0 .. NH1-1
+        if constexpr (m % 5 == 1 && m / 5 < NH1) {
+          constexpr int idx = m / 5;
+          so = (idx < TI ? ka3 : kb3) + istr[idx];
+          if constexpr (idx < TI) set_m0(ma3, integral_constant<int, idx * 4096>{});
+          else set_m0(mb3, integral_constant<int, (idx - TI) * M0B_STEP>{});
+        }
+        if constexpr (m % 5 == 2 && m / 5 < NH1) issue_load(m / 5 < TI ? l3.ra : l3.rb, m / 5 < TI ? a_voff : b_voff, so);
+        // the tile's last step: the dX product's LoRA operands, M0 in gap 5q+3, the load in gap 5q+4
+        if constexpr (LAST.value && m % 5 >= 3 && m / 5 < N_LORA_LOADS) {
+          if constexpr (m % 5 == 3) lora_m0(integral_constant<int, m / 5>{});
+          else lora_load(integral_constant<int, m / 5>{});
+        }
+        mfma_one(1, m, std::false_type{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+      lgkm0();
+      __builtin_amdgcn_sched_barrier(0);
+      cst = nx1;
+    };
+    // K step q of this tile, or, beyond its last, step q - nk of the next: descriptors picked with scalar selects
+    auto pick = [&](int q, LoadSrc& l, int& k) __attribute__((always_inline)) {
+      const bool own = q < nk;
+#pragma unroll
+      for (int d = 0; d < 4; d++) { l.ra[d] = own ? src.ra[d] : nxt_src.ra[d]; l.rb[d] = own ? src.rb[d] : nxt_src.rb[d]; }
+      l.kstart = own ? src.kstart : nxt_src.kstart;
+      k = own ? q : q - nk;
+    };
+    if constexpr (NST == 2) {
       // step 0 loads this tile's step 2, or (nk == 2) the next tile's step 0; descriptors picked with scalar selects
       const bool own = nk > 2;
       LoadSrc l0;
@@ -499,14 +584,30 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       int s = 1;
       for (; s + 2 < nk; s++) k_step(s, src, s + 2, std::false_type{});
       for (; s < nk; s++) k_step(s, nxt_src, s + 2 - nk, std::false_type{});
+      par = (par + nk) & 1;
+    } else {
+      // (nk >= 4: the launcher's condition for this tile)
+      k_step3(src, 2, src, 3, std::true_type{}, std::false_type{});
+      int s = 1;
+      for (; s + 3 < nk; s++) k_step3(src, s + 2, src, s + 3, std::false_type{}, std::false_type{});
+      for (; s + 1 < nk; s++) {
+        LoadSrc l2, l3;
+        int k2, k3;
+        pick(s + 2, l2, k2);
+        pick(s + 3, l3, k3);
+        k_step3(l2, k2, l3, k3, std::false_type{}, std::false_type{});
+      }
+      k_step3(nxt_src, 1, nxt_src, 2, std::false_type{}, std::true_type{});   // step nk-1
+      par = (par + nk) % 3;
+      // the operands requested in the last sub-step (and with them the next tile's first loads)
+      if constexpr (N_LORA_LOADS > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    par = (par + nk) & 1;
     mfma_fence();
 
     // ------------------------------------------------------------ LoRA term: operands; forward: 64 MFMAs per chunk onto the
     // accumulators (dX: the term is formed per block row inside the epilogue below, from up to two chunks = 32 rank columns)
-    lf_u32x2 rf0[8], lv0[8], rf1[8], lv1[8];
-    lf_u32x4 mw[8];
+    lf_u32x2 rf0[8], lv0[TI], rf1[8], lv1[TI];
+    lf_u32x4 mw[TI];
     if constexpr (LORA) {
       int sl = lane;
       asm volatile("" : "+v"(sl));
@@ -517,13 +618,13 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       // chunk t of the operands: 16 rank columns, two registers per 16x16x16 fragment.  FROM_LDS: the A_i fragments of
       // chunk 0 of the dX product are transposing reads of the rows that landed in the wave's LDS area (within a
       // 16-lane group, lane 4j+c addresses row j, columns 4c..4c+3 and receives column lane&15, rows 0..3).
-      auto load_chunk = [&](int t, lf_u32x2 (&rf)[8], lf_u32x2 (&lv)[8], auto FROM_LDS) __attribute__((always_inline)) {
+      auto load_chunk = [&](int t, lf_u32x2 (&rf)[8], lf_u32x2 (&lv)[TI], auto FROM_LDS) __attribute__((always_inline)) {
         const int r0 = t * 16 + kg * 4;
         const int rcc = r0 < rank ? r0 : 0;   // lanes beyond the rank re-read the first columns; zeroed in prep_chunk
 #pragma unroll
-        for (int i = 0; i < 8; i++) lv[i] = *(const lf_u32x2*)(Lp + (int64_t)(wrow0 + i * 16 + l16) * p.R + r0);
+        for (int i = 0; i < TI; i++) lv[i] = *(const lf_u32x2*)(Lp + (int64_t)(wrow0 + i * 16 + l16) * p.R + r0);
         if constexpr (FROM_LDS.value) {
-          const uint32_t ad = area + (kg * 4 + (l16 >> 2)) * 256 + (l16 & 3) * 8;
+          const uint32_t ad = area_r + (kg * 4 + (l16 >> 2)) * 256 + (l16 & 3) * 8;
           lf_u32x2 t0, t1, t2, t3, t4, t5, t6, t7;
           asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(t0) : "v"(ad) : "memory");
           asm volatile("ds_read_b64_tr_b16 %0, %1 offset:32" : "=v"(t1) : "v"(ad) : "memory");
@@ -553,7 +654,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       };
       // lanes whose rank columns lie beyond the adapter's rank feed zeros; the forward scale goes into the 16-bit L
       // fragment (fp32 product, one rounding; exact for powers of two)
-      auto prep_chunk = [&](int t, lf_u32x2 (&rf)[8], lf_u32x2 (&lv)[8]) __attribute__((always_inline)) {
+      auto prep_chunk = [&](int t, lf_u32x2 (&rf)[8], lf_u32x2 (&lv)[TI]) __attribute__((always_inline)) {
         const bool in_r = t * 16 + kg * 4 < rank;
 #pragma unroll
         for (int j = 0; j < 8; j++)
@@ -561,7 +662,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
           for (int d = 0; d < 2; d++) rf[j][d] = in_r ? rf[j][d] : 0u;
         if (p.mult_mode == 0 && rt.mult != 1.f) {
 #pragma unroll
-          for (int i = 0; i < 8; i++)
+          for (int i = 0; i < TI; i++)
 #pragma unroll
             for (int d = 0; d < 2; d++)
               lv[i][d] = BigOp<T>::pack2(BigOp<T>::to_float((uint16_t)(lv[i][d] & 0xffffu)) * rt.mult, BigOp<T>::to_float((uint16_t)(lv[i][d] >> 16)) * rt.mult);
@@ -569,41 +670,49 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         // The MFMAs are inline assembly, which the compiler's hazard recogniser does not see: a vector ALU result
         // needs wait states before an MFMA reads it.  The nop takes the operands as in/outs, so every instruction
         // that produces them stays in front of it and every MFMA behind.
-        asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
-                                 "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]));
+        if constexpr (TI == 8) {
+          asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
+                                   "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]));
+        } else {
+          asm volatile("s_nop 3" : "+v"(rf[0]), "+v"(rf[1]), "+v"(rf[2]), "+v"(rf[3]), "+v"(rf[4]), "+v"(rf[5]), "+v"(rf[6]), "+v"(rf[7]),
+                                   "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]));
+        }
       };
       if constexpr (NN) {
         // dX product: the term is formed in the epilogue, block row by block row, under the keep bits of the wave's
         // block (one 16-byte row piece per block row, from the LDS area; all ones where no mask applies)
-        const uint32_t ad = area + 4096 + l16 * 16;
-        lf_u32x4 m0_, m1_, m2_, m3_, m4_, m5_, m6_, m7_;
+        const uint32_t ad = area_m + l16 * 16;
+        lf_u32x4 m0_, m1_, m2_, m3_, m4_{}, m5_{}, m6_{}, m7_{};
         asm volatile("ds_read_b128 %0, %1" : "=v"(m0_) : "v"(ad) : "memory");
         asm volatile("ds_read_b128 %0, %1 offset:256" : "=v"(m1_) : "v"(ad) : "memory");
         asm volatile("ds_read_b128 %0, %1 offset:512" : "=v"(m2_) : "v"(ad) : "memory");
         asm volatile("ds_read_b128 %0, %1 offset:768" : "=v"(m3_) : "v"(ad) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(m4_) : "v"(ad) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:1280" : "=v"(m5_) : "v"(ad) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:1536" : "=v"(m6_) : "v"(ad) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:1792" : "=v"(m7_) : "v"(ad) : "memory");
+        if constexpr (TI == 8) {
+          asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(m4_) : "v"(ad) : "memory");
+          asm volatile("ds_read_b128 %0, %1 offset:1280" : "=v"(m5_) : "v"(ad) : "memory");
+          asm volatile("ds_read_b128 %0, %1 offset:1536" : "=v"(m6_) : "v"(ad) : "memory");
+          asm volatile("ds_read_b128 %0, %1 offset:1792" : "=v"(m7_) : "v"(ad) : "memory");
+        }
         load_chunk(0, rf0, lv0, std::true_type{});
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(m0_), "+v"(m1_), "+v"(m2_), "+v"(m3_), "+v"(m4_), "+v"(m5_), "+v"(m6_), "+v"(m7_) :: "memory");
+        if constexpr (TI == 8) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(m0_), "+v"(m1_), "+v"(m2_), "+v"(m3_), "+v"(m4_), "+v"(m5_), "+v"(m6_), "+v"(m7_) :: "memory");
+        else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(m0_), "+v"(m1_), "+v"(m2_), "+v"(m3_) :: "memory");
         const lf_u32x4 ones = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
         mw[0] = sel ? m0_ : ones; mw[1] = sel ? m1_ : ones; mw[2] = sel ? m2_ : ones; mw[3] = sel ? m3_ : ones;
-        mw[4] = sel ? m4_ : ones; mw[5] = sel ? m5_ : ones; mw[6] = sel ? m6_ : ones; mw[7] = sel ? m7_ : ones;
+        if constexpr (TI == 8) { mw[4] = sel ? m4_ : ones; mw[5] = sel ? m5_ : ones; mw[6] = sel ? m6_ : ones; mw[7] = sel ? m7_ : ones; }
         prep_chunk(0, rf0, lv0);
         if (n16 > 1) { load_chunk(1, rf1, lv1, std::false_type{}); prep_chunk(1, rf1, lv1); }
       } else {
         load_chunk(0, rf0, lv0, std::false_type{});
         prep_chunk(0, rf0, lv0);
 #pragma unroll
-        for (int i = 0; i < 8; i++)
+        for (int i = 0; i < TI; i++)
 #pragma unroll
           for (int j = 0; j < 8; j++) BigOp<T>::mfma16(acc[i][j], rf0[j], lv0[i]);
         for (int t = 1; t < n16; t++) {
           load_chunk(t, rf1, lv1, std::false_type{});
           prep_chunk(t, rf1, lv1);
 #pragma unroll
-          for (int i = 0; i < 8; i++)
+          for (int i = 0; i < TI; i++)
 #pragma unroll
             for (int j = 0; j < 8; j++) BigOp<T>::mfma16(acc[i][j], rf1[j], lv1[i]);
         }
@@ -618,7 +727,7 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
       int ln = lane;
       asm volatile("" : "+v"(ln));
       const int e16 = ln & 15, ekg = ln >> 4;
-      const uint32_t ep_lds = lds0 + EP_OFF + wave * EP_WAVE;
+      const uint32_t ep_lds = area;
       lf_u32x2 bvp[8];
 #pragma unroll
       for (int j = 0; j < 8; j++) bvp[j] = lf_u32x2{0u, 0u};
@@ -645,11 +754,11 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
         }
       };
       if constexpr (MASKED.value) p_row(integral_constant<int, 0>{});
-      sfor<8>([&](auto I) {
+      sfor<TI>([&](auto I) {
         constexpr int i = I.value;
         uint32_t mws[4] = {0u, 0u, 0u, 0u};
         if constexpr (MASKED.value) {
-          if constexpr (i + 1 < 8) p_row(integral_constant<int, i + 1>{});
+          if constexpr (i + 1 < TI) p_row(integral_constant<int, i + 1>{});
           lf_f32x4(&tm)[8] = P[i & 1];
           // wait states between the MFMAs of this block row (a block row of MFMAs ago, except for the last) and the
           // vector instructions that read their results
@@ -709,13 +818,14 @@ gemm_big_kernel(const LfGemmParams p, const LfSegTable seg) {
 #endif
 }
 
-template <typename T, bool NN, bool LORA>
+template <typename T, bool NN, bool LORA, int TI>
 int launch_big(LfGemmParams p, const LfSegTable& seg, int max_wgs, hipStream_t st) {
+  constexpr int BM = TI * 32;
   p.grid_m = (p.M + BM - 1) / BM;
   p.grid_n = (p.N + BN - 1) / BN;
-  auto kern = gemm_big_kernel<T, NN, LORA>;
+  auto kern = gemm_big_kernel<T, NN, LORA, TI>;
   static LfLdsFlags lds_ok;
-  constexpr int SMEM_BYTES = Lds<NN>::BYTES;
+  constexpr int SMEM_BYTES = Lds<NN, TI>::BYTES;
   if (!lf_allow_lds(kern, SMEM_BYTES, lds_ok)) return LF_ELAUNCH;
   // Tile order: an XCD's 32 concurrent tiles form a block of group_m tile rows x 32 / group_m columns.  8 x 4 fetches
   // the fewest operand panels (8 + 4).  With a long K and at most 16 tile columns the left operand does not fit the
@@ -744,22 +854,24 @@ int lf_cu_count() {
   return n;
 }
 
-int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, hipStream_t st) {
-  if (p.K % BK != 0 || p.K < 2 * BK || p.M < BM || p.N < BN || p.N % 8 != 0) return LF_ESHAPE;  // edge tiles are shifted inwards
-  // a wave's 128 rows lie in one routing block, also in a shifted edge tile
-  if (seg.table != nullptr && (seg.block_size_m % 128 != 0 || p.M % 128 != 0)) return LF_ESHAPE;
+template <typename T, int TI>
+int launch_big_ti(const LfGemmParams& p, const LfSegTable& seg, bool nn, int wgs, hipStream_t st) {
+  if (p.L != nullptr) return nn ? launch_big<T, true, true, TI>(p, seg, wgs, st) : launch_big<T, false, true, TI>(p, seg, wgs, st);
+  return nn ? launch_big<T, true, false, TI>(p, seg, wgs, st) : launch_big<T, false, false, TI>(p, seg, wgs, st);
+}
+
+int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int tile_rows, hipStream_t st) {
+  if (tile_rows != 256 && tile_rows != 128) return LF_EINVAL;
+  // edge tiles are shifted inwards; the K loop runs over two stages (256 rows) or three (128 rows: at least four K steps)
+  if (p.K % BK != 0 || p.K < (tile_rows == 256 ? 2 : 4) * BK || p.M < tile_rows || p.N < BN || p.N % 8 != 0) return LF_ESHAPE;
+  // the rows of a wave (half a tile's) lie in one routing block, also in a shifted edge tile
+  const int wrows = tile_rows / 2;
+  if (seg.table != nullptr && (seg.block_size_m % wrows != 0 || p.M % wrows != 0)) return LF_ESHAPE;
   // the keep-mask comes bit-packed (16 bytes per 128 columns of a row); the dX product forms its term from up to 32 rank columns
   if (p.mask != nullptr && (!p.mask_bits || p.N % 128 != 0 || p.ldmask % 4 != 0)) return LF_ESHAPE;
   if (nn && p.L != nullptr && p.R > 32) return LF_ESHAPE;
   const int wgs = lf_cu_count();
-  const bool lora = p.L != nullptr;
-  if (dtype == LF_BF16) {
-    if (lora) return nn ? launch_big<__bf16, true, true>(p, seg, wgs, st) : launch_big<__bf16, false, true>(p, seg, wgs, st);
-    return nn ? launch_big<__bf16, true, false>(p, seg, wgs, st) : launch_big<__bf16, false, false>(p, seg, wgs, st);
-  }
-  if (dtype == LF_F16) {
-    if (lora) return nn ? launch_big<_Float16, true, true>(p, seg, wgs, st) : launch_big<_Float16, false, true>(p, seg, wgs, st);
-    return nn ? launch_big<_Float16, true, false>(p, seg, wgs, st) : launch_big<_Float16, false, false>(p, seg, wgs, st);
-  }
+  if (dtype == LF_BF16) return tile_rows == 256 ? launch_big_ti<__bf16, 8>(p, seg, nn, wgs, st) : launch_big_ti<__bf16, 4>(p, seg, nn, wgs, st);
+  if (dtype == LF_F16) return tile_rows == 256 ? launch_big_ti<_Float16, 8>(p, seg, nn, wgs, st) : launch_big_ti<_Float16, 4>(p, seg, nn, wgs, st);
   return LF_EINVAL;
 }

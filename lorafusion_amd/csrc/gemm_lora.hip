@@ -761,6 +761,7 @@ static const TileCand kCands[] = {
     {4, 128, 128, 512, 38.0, 47.0, 5.0, 70.0},    // 4 waves, two workgroups per CU
     {5, 64, 64, 512, 19.0, 17.0, 13.0, 18.0},     // 4 waves, 32x32 per wave: spreads a short row range
     {6, 128, 64, 256, 22.5, 4.5, 13.0, 14.0},     // 4 waves, 64x32 per wave: less operand traffic per flop than 64x64
+    {8, 128, 256, 256, 41.5, 15.0, 45.0, 30.0},   // persistent, 4 waves of 64x128 (gemm_big.hip): 2048 x 4096 outputs are one round of it
 };
 constexpr double kRamp = 6.0;
 static double launch_cost(const TileCand& c, int M, int N, int K) {
@@ -773,11 +774,14 @@ static double launch_cost(const TileCand& c, int M, int N, int K) {
   else at4096 = c.lat0 + c.first_b + (full - 1) * (c.next_a + c.next_b) + (fill > 0 ? c.next_a + c.next_b * fill : 0.0);
   return kRamp + (at4096 - kRamp) * (K / 4096.0);
 }
-static int choose_cfg(int M, int N, int K, bool allow_big, double* cost_out = nullptr) {
+static int choose_cfg(int M, int N, int K, bool allow_big, double* cost_out = nullptr, bool allow_mid = true) {
   int best = 1;
   double best_cost = 1e30;
   for (const TileCand& c : kCands) {
     if (c.cfg == 7 && (!allow_big || M < 256 || N < 256)) continue;
+    // (a lone 128x256 tile per CU takes 41 us whatever the fill, the same for both operand layouts: below half a round
+    // the smaller tiles are faster)
+    if (c.cfg == 8 && (!allow_big || !allow_mid || M < 128 || N < 256 || K < 256 || 2 * (long)((M + 127) / 128) * ((N + 255) / 256) <= c.slots)) continue;
     const double cost = launch_cost(c, M, N, K);
     if (cost < best_cost) { best_cost = cost; best = c.cfg; }
   }
@@ -800,7 +804,8 @@ static int choose_split(int M, int N, int K, bool allow_big, int* cfg_head, int*
   int best_m = 0;
   for (int r = 1; r * 256 < M; r++) {
     double tail;
-    const int ct = choose_cfg(M - r * 256, N, K, allow_big, &tail);
+    // (left-over rows behind whole rounds of 256x256 tiles: small tiles or a split contraction, not the 128-row persistent tile)
+    const int ct = choose_cfg(M - r * 256, N, K, allow_big, &tail, false);
     const double cost = launch_cost(head, r * 256, N, K) + tail + kLaunch;
     if (cost < best) { best = cost; best_m = r * 256; *cfg_tail = ct; }
   }
@@ -851,7 +856,7 @@ static KSplit ksplit_for(int M, int N, int K, int cfg, int routing_block) {
 
 static std::atomic<int> pinned_cfg{-1};
 int lf_pin_tile_cfg(int cfg) {
-  if (cfg < -1 || cfg > 7) return LF_EINVAL;
+  if (cfg < -1 || cfg > 8) return LF_EINVAL;
   pinned_cfg.store(cfg, std::memory_order_relaxed);
   return LF_OK;
 }
@@ -883,7 +888,7 @@ size_t lf_gemm_ksplit_bytes(int M, int N, int K, int routing_block) {
   lf_plan_gemm(M, N, K, routing_block, &rows, &ch, &ct);
   size_t need = 0;
   auto part = [&](int m, int cfg) {
-    for (int c : {cfg, 1, 2}) {
+    for (int c : {cfg, 1, 2, choose_cfg(m, N, K, false)}) {
       const KSplit ks = ksplit_for(m, N, K, c, routing_block);
       if (ks.n > 1) need = std::max(need, (size_t)ks.n * m * N * sizeof(float));
     }
@@ -913,7 +918,12 @@ int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dt
     // what the persistent kernel does not take goes to the eight-wave 256x256 tile: a keep-mask with one byte per
     // element, a dX term of more than 32 rank columns and (when the library chose the tile) a contraction of one K step
     if (cfg == 7 && ((q.mask != nullptr && (!q.mask_bits || q.N % 128 != 0)) || (nn && q.L != nullptr && q.R > 32) || (planned && q.K < 128))) cfg = 1;
-    if (cfg == 7) return lf_launch_gemm_big(q, seg, nn, dtype, st);
+    // the 128-row persistent tile has the same limits; a product it was planned for then runs on the small tile the
+    // cost model likes best (pinned: on the four-wave 128x256 tile)
+    if (cfg == 8 && ((q.mask != nullptr && (!q.mask_bits || q.N % 128 != 0)) || (nn && q.L != nullptr && q.R > 32)))
+      cfg = planned ? choose_cfg(q.M, q.N, q.K, false) : 2;
+    if (cfg == 7) return lf_launch_gemm_big(q, seg, nn, dtype, 256, st);
+    if (cfg == 8) return lf_launch_gemm_big(q, seg, nn, dtype, 128, st);
     if (dtype != LF_BF16 && dtype != LF_F16) return (int)LF_EINVAL;
     LfGemmParams r = q;
     r.ksplit = 1;

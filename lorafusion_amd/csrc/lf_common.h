@@ -62,7 +62,7 @@ struct LfGemmParams {
 
 // launchers (one per translation unit)
 int lf_launch_gemm(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int force_cfg, hipStream_t st);
-int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, hipStream_t st);  // persistent 256x256 tiles
+int lf_launch_gemm_big(const LfGemmParams& p, const LfSegTable& seg, bool nn, int dtype, int tile_rows, hipStream_t st);  // persistent tiles of 256 or 128 rows x 256 columns
 int lf_cu_count();
 int lf_pin_tile_cfg(int cfg);  // -1: automatic choice
 void lf_plan_gemm(int M, int N, int K, int routing_block, int* rows_head, int* cfg_head, int* cfg_tail);

@@ -1,7 +1,8 @@
-"""GPU parity of the persistent 256x256 GEMM kernel's fused paths at small sizes.
+"""GPU parity of the persistent GEMM kernel's fused paths at small sizes, for both of its tiles (256x256 over two
+LDS stages, 128x256 over three).
 
 The library picks that kernel by itself only for large products; here it is pinned
-(lf_set_tile_cfg(7)) so that its LoRA seeding (rank chunks, per-wave routing lookups, the scale
+(lf_set_tile_cfg(7) / (8)) so that its LoRA seeding (rank chunks, per-wave routing lookups, the scale
 folded into the skinny operand), its keep-mask select on the dX path, bias, fp16, edge tiles that
 are shifted inwards and tiles that span two adapters all run against the CPU oracle at sizes the
 oracle restates in full.  Tolerances as in test_gpu_lora_single.py / test_gpu_lora_multi.py.
@@ -16,12 +17,12 @@ from tests.test_gpu_lora_single import _run_case as run_single
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture
-def big_tiles():
+@pytest.fixture(params=[7, 8], ids=["256x256", "128x256"])
+def big_tiles(request):
     from lorafusion_amd import _lib
 
-    assert _lib.lib().lf_set_tile_cfg(7) == 0
-    yield
+    assert _lib.lib().lf_set_tile_cfg(request.param) == 0
+    yield request.param
     assert _lib.lib().lf_set_tile_cfg(-1) == 0
 
 
@@ -84,5 +85,22 @@ def test_pinned_tile_rejects_small_products():
             hip_ops.gemm(a, b)
     finally:
         assert _lib.lib().lf_set_tile_cfg(-1) == 0
-    assert _lib.lib().lf_set_tile_cfg(8) != 0
+    assert _lib.lib().lf_set_tile_cfg(9) != 0
     hip_ops.gemm(a, b)
+
+
+def test_pinned_128_row_tile_rejects_a_short_contraction():
+    """The 128-row tile runs its K loop over three stages: fewer than four K steps (K < 256) is a shape error when pinned
+    (the library's own choice never lands there)."""
+    from lorafusion_amd import _lib
+    from lorafusion_amd.ops import hip_ops
+
+    a = torch.randn(256, 192, device="cuda").bfloat16()
+    b = torch.randn(256, 192, device="cuda").bfloat16()
+    assert _lib.lib().lf_set_tile_cfg(8) == 0
+    try:
+        with pytest.raises(RuntimeError):
+            hip_ops.gemm(a, b)
+    finally:
+        assert _lib.lib().lf_set_tile_cfg(-1) == 0
+    assert torch.allclose(hip_ops.gemm(a, b).float(), a.float() @ b.float().T, rtol=2e-2, atol=0.5)

@@ -15,7 +15,7 @@ def _close(actual, expected, what, rtol=1e-2):
     assert ok, f"{what}: max|err|/max|e| = {rel:.3e}, worst excess {excess:.3e}"
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("trans_b", [True, False])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (520, 640, 384), (1024, 1280, 1024), (77, 136, 64), (130, 72, 704),
                                    (256, 264, 64), (300, 256, 192), (2100, 4360, 320)])
@@ -24,6 +24,8 @@ def test_gemm_all_tiles(cfg, trans_b, M, N, K):
 
     if cfg == 7 and (M < 256 or N < 256 or K < 128):
         pytest.skip("the persistent 256x256 kernel shifts edge tiles inwards (M, N >= 256) and pipelines two K steps (K >= 128)")
+    if cfg == 8 and (M < 128 or N < 256 or K < 256):
+        pytest.skip("the persistent 128x256 kernel shifts edge tiles inwards (M >= 128, N >= 256) and pipelines three K steps (K >= 256)")
 
     g = torch.Generator().manual_seed(M + N + K)
     a = torch.randn(M, K, generator=g).bfloat16()
