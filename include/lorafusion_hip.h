@@ -195,12 +195,13 @@ int lf_gemm(const void* A, const void* B, const void* bias, void* C, int M, int 
             int tile_cfg, void* stream);
 
 /* Tile configuration of every later MFMA GEMM launch of this process that does not name one itself
- * (the fused entry points, lf_gemm with tile_cfg = -1): 0..7 pins it, -1 (the initial state)
+ * (the fused entry points, lf_gemm with tile_cfg = -1): 0..8 pins it, -1 (the initial state)
  * returns to the library's own choice.  A process-wide setting meant for tests and tuning runs --
  * parity of every tile shape at small sizes; the reference has the same kind of knob in the
  * Triton autotune configs of its kernels (lorafusion/ops/triton_ops/config.py).  A launch whose
- * shape the pinned configuration cannot take fails with LF_ESHAPE (7, the persistent 256x256
- * kernel, needs M, N >= 256).  Returns LF_EINVAL outside -1..7. */
+ * shape the pinned configuration cannot take fails with LF_ESHAPE (7, the persistent kernel's
+ * 256x256 tile, needs M, N >= 256 and K >= 128; 8, its 128x256 tile, M >= 128, N >= 256 and
+ * K >= 256).  Returns LF_EINVAL outside -1..8. */
 int lf_set_tile_cfg(int tile_cfg);
 
 /* The launches the library makes for an M x N output contracted over K when no configuration is pinned: rows

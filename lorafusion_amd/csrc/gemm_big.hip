@@ -1,4 +1,4 @@
-// Persistent 256x256-tile MFMA GEMM with the LoRA term seeded into the accumulator, for gfx950 (MI355X).
+// Persistent MFMA GEMM in tiles of 256x256 or 128x256 with the LoRA term added to the accumulator, for gfx950 (MI355X).
 //
 //   C[M,N] = A[M,K] * op(B) + mult * (L[M,R] * Rop) (+ bias)        (operands as in gemm_lora.hip)
 //
@@ -7,7 +7,7 @@
 // persistent forward is fused_lora_xw_sb_tma.py:314,351-357) and fused_lora_dyw_dsa / fused_multi_lora_dyw_dsa
 // (fused_lora_dyw_dsa.py:69-181, fused_multi_lora_dyw_dsa.py:60-185).
 //
-// Structure
+// Structure (of the 256x256 tile, TI = 8; what the 128x256 tile, TI = 4, does differently comes last)
 //  * One workgroup per CU (at most), four 64-lane waves, each owning a 128x128 sub-tile (8x8 blocks of
 //    16x16x32 MFMA, 256 accumulator registers).  One wave per SIMD: a K step of 32 costs 16 LDS fragment
 //    reads per wave for 64 MFMAs, a third less LDS traffic than eight waves of 128x64.
@@ -38,8 +38,14 @@
 //    are slow to fetch (keep bits from HBM, A_i rows that need a transposing read) land in the wave's own LDS
 //    area as direct-to-LDS loads during the tile's first K step.  The forward scale is folded into the 16-bit L
 //    fragments (exact for powers of two).
-//  * Epilogue: 16-row bands of a wave's sub-tile go through 4.5 KB of LDS per wave (beside the two stages) and
+//  * Epilogue: 16-row bands of a wave's sub-tile go through 4 KB of LDS per wave (beside the two stages) and
 //    leave as 16-byte non-temporal stores that cover whole 256-byte rows of the sub-tile.
+//  * TI = 4: four waves of 64x128 (one round of 128x256 tiles is what 2048 x 4096 outputs give 256 CUs).  A K step
+//    is half as long but loads three quarters as much, so the stages are three: step s issues the second half of
+//    step s+2's loads in its first sub-step and the first half of step s+3's in its second, one load per five MFMAs,
+//    and waits with vmcnt(12) before its barrier (see k_step3).  Nothing fits behind three stages: a wave's band /
+//    landing area lies inside the stage of the tile's last K step, and the dX product's operands are requested in
+//    that step's second sub-step.
 #include "lf_common.h"
 #include <type_traits>
 #include <utility>
