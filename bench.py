@@ -428,7 +428,9 @@ def gemm_ref_block(dev, reps: int = 20, zero: bool = False) -> dict:
 
     out = {}
     for name, (M, N, K, trans_b) in {"16384x4096x4096 NT": (16384, 4096, 4096, True), "16384x4096x28672 NN": (16384, 4096, 28672, False),
-                                     "16384x14336x4096 NT": (16384, 14336, 4096, True)}.items():
+                                     "16384x14336x4096 NT": (16384, 14336, 4096, True),
+                                     # the single linear of workload c1 (one round of the persistent kernel's 128x256 tiles)
+                                     "2048x4096x4096 NT": (2048, 4096, 4096, True), "2048x4096x4096 NN": (2048, 4096, 4096, False)}.items():
         g = torch.Generator(device=dev).manual_seed(0)
         a = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
         b = (torch.randn(N, K, generator=g, device=dev) if trans_b else torch.randn(K, N, generator=g, device=dev)).to(torch.bfloat16)

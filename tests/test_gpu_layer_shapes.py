@@ -131,6 +131,24 @@ def test_kernel_grid_shapes(tokens, K, N, n_adapters, seed):
     _run_multi(tokens, K, N, [16] * n_adapters, [0.05, 0.1, 0.0, 0.1][:n_adapters], [2.0, 1.0, 2.0, 4.0][:n_adapters], seed=seed)
 
 
+def test_one_round_of_128_row_persistent_tiles():
+    """1800 tokens of two adapters over a 4096 x 4096 weight: the padded batch is between half a round and one round of
+    128x256 tiles, which the library runs on the persistent kernel's three-stage instance in both products (asserted
+    from the launch plan, so the case keeps its meaning if the plan changes)."""
+    import ctypes
+
+    from lorafusion_amd import _lib as L
+    from lorafusion_amd.ops.multi_lora import prepare_multi_lora_batch_info
+
+    seq = lognormal_segments(1800, 2, seed=1)
+    info = prepare_multi_lora_batch_info(seq, [0, 1], [16, 16], [0.05, 0.1], [2.0, 1.0], 128, output_dtype=torch.float32)
+    Mp = sum(info.padded_seq_len_list)
+    rows, ch, ct = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    L.check(L.lib().lf_gemm_plan(Mp, 4096, 4096, 128, ctypes.byref(rows), ctypes.byref(ch), ctypes.byref(ct)), "lf_gemm_plan")
+    assert (rows.value, ch.value, ct.value) == (Mp, 8, -1)
+    _run_multi(1800, 4096, 4096, [16, 16], [0.05, 0.1], [2.0, 1.0], seed=1)
+
+
 @pytest.mark.parametrize("K,N", [(8192, 8192), (8192, 1024), (8192, 10240), (8192, 28672), (8192, 57344), (28672, 8192)])
 def test_70b_layer_projections_nf4(K, N):
     """8192 tokens, 8 adapters r=64, base weight quantised to NF4 and dequantised on the device; the separate
