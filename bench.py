@@ -277,6 +277,8 @@ def kernel_breakdown(linears, reps: int):
         t["da"] += graph_time_ms(lambda: hip_ops.fused_multi_lora_da(lin.x, ds, r, lin.mask), reps)
         # the dX GEMM's main launch: output [Mp, K], reduction over N
         rows, cfg, _ = gemm_plan(b.Mp, lin.k, lin.n, True)
+        if cfg == 7 and r.R > 32:
+            cfg = 1   # the persistent kernel forms the dX term from at most 32 rank columns: the library runs this launch on the eight-wave 256x256 tile
         if rows < b.Mp:
             rh = b.head(rows)
             nseg = len(rh.padded_seq_len_list)
