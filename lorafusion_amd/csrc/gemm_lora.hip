@@ -867,7 +867,15 @@ void lf_plan_gemm(int M, int N, int K, int routing_block, int* rows_head, int* c
   const bool allow_big = routing_block <= 0 || (routing_block % 128 == 0 && M % 128 == 0);
   int ch = 1, ct = 1;
   const int m_main = choose_split(M, N, K, allow_big, &ch, &ct);
-  auto demote = [&](int cfg) { return (routing_block > 0 && routing_block % 128 != 0 && (cfg == 0 || cfg == 1 || cfg == 7)) ? 2 : cfg; };
+  // A long contraction under a wide output runs faster on the eight-wave 256x256 tile than on the persistent kernel
+  // (8192 x 8192 over 28672: 3.08 against 3.24 ms, over 57344: 5.74 against 5.85; at 4096 columns the two are level, and
+  // at shorter contractions the persistent kernel is 3-8 % ahead): its long K loops let the tiles of an XCD drift apart
+  // and lose the L2 hits on the panels they share.
+  auto long_k = [&](int cfg) { return (cfg == 7 && K >= 16384 && N >= 8192) ? 1 : cfg; };
+  auto demote = [&](int cfg0) {
+    const int cfg = long_k(cfg0);
+    return (routing_block > 0 && routing_block % 128 != 0 && (cfg == 0 || cfg == 1 || cfg == 7)) ? 2 : cfg;
+  };
   if (m_main == 0) {
     *rows_head = M;
     *cfg_head = demote(choose_cfg(M, N, K, allow_big));
