@@ -127,6 +127,18 @@ def test_launch_plan_takes_the_contraction_length():
         assert plan(16512, 4096, K) == (16512, 7, -1)
     assert plan(2048, 4096, 4096)[0] == 2048        # nothing left over: one launch
     assert L.lib().lf_gemm_plan(16, 16, 0, 0, None, None, None) == L.LF_EINVAL
+    # The persistent kernel's 128x256 tile (8) takes single launches between half a round and one round of its tiles
+    # on 256 compute units; fewer rows go to small tiles, more to its 256x256 tile (7), left-over rows never to 8.
+    assert plan(2048, 4096, 4096) == (2048, 8, -1) and plan(1536, 4096, 6144) == (1536, 8, -1)
+    assert plan(1024, 4096, 4096)[1] not in (7, 8)
+    assert plan(4096, 4096, 4096) == (4096, 7, -1) and plan(2048, 8192, 8192) == (2048, 7, -1)
+    assert plan(2048, 4096, 128)[1] != 8            # its K loop needs four steps of 64
+    for M in (8448, 8576, 16512, 16640):
+        for N, K in [(4096, 4096), (8192, 8192), (57344, 8192), (10240, 8192)]:
+            assert plan(M, N, K)[2] != 8
+    # a long contraction under a wide output: the eight-wave 256x256 tile (1), not the persistent kernel
+    assert plan(8192, 8192, 28672) == (8192, 1, -1) and plan(8576, 8192, 28672)[:2] == (8192, 1)
+    assert plan(8192, 8192, 8192)[1] == 7 and plan(16384, 4096, 28672)[1] == 7
 
 
 def test_python_layer_refuses_cpu_tensors():
