@@ -297,8 +297,10 @@ int lf_lora_bwd_static(const void* dY, const void* X, const void* W, const uint8
   LfSegTable t;
   int rc = make_seg(routing, M, nullptr, nullptr, t);
   if (rc != LF_OK) return rc;
+  // what lf_workspace_bytes(LF_OP_BWD, ...) names: the rank-r passes' partial sums or the dX product's partial tiles,
+  // whichever is larger (with less, the product would not split its contraction and its sums would differ in order)
   const size_t a = lf_dys_dyb_workspace(M, N, R, t), b = lf_da_workspace(M, K, R, t);
-  const size_t need = align256(a > b ? a : b);
+  const size_t need = align256(std::max(std::max(a, b), lf_gemm_ksplit_bytes(M, K, N, t.table != nullptr ? t.block_size_m : 0)));
   if (need > (size_t)LF_STATIC_SCRATCH_BYTES) return LF_ESTATIC;
   void* ws = nullptr;
   rc = static_scratch(&ws);
