@@ -384,7 +384,26 @@ def raw_workload(name: str, args, dev, breakdown: bool = True) -> dict:
     return res
 
 
-def nf4_dequant_block(dev, shape=(14336, 4096), fill: bool = False) -> dict:
+def nf4_cpu_baseline(packed, qs, shape, nbytes: float) -> dict:
+    """The C restatement of the dequantisation (oracle/nf4_oracle.c, one thread) on the same packed weight, host
+    memory to host memory: best of three runs of the whole weight, in the kernel's own unit."""
+    import numpy as np
+
+    from oracle import nf4 as onf4
+
+    st = onf4.NF4State(packed=packed.cpu().numpy().reshape(-1), absmax=qs.absmax.cpu().numpy(), shape=tuple(shape),
+                       blocksize=qs.blocksize, code2=qs.state2.code.cpu().numpy(), absmax2=qs.state2.absmax.cpu().numpy(),
+                       offset=qs.offset.cpu().numpy().reshape(1).astype(np.float32), blocksize2=qs.state2.blocksize)
+    best = float("inf")
+    for _ in range(3):
+        t0 = time.perf_counter()
+        onf4.dequantize(st)
+        best = min(best, time.perf_counter() - t0)
+    return {"value": round(nbytes / best / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"the whole {list(shape)} weight, oracle/nf4_oracle.c on one host core, best of 3 runs, {best * 1e3:.0f} ms/run"}
+
+
+def nf4_dequant_block(dev, shape=(14336, 4096), fill: bool = False, cpu: bool = False) -> dict:
     """Standalone NF4 dequant of W[shape], blocksize 64, double quantised: 2.516 B/element.  `fill`: also time a plain
     fill of the output tensor (torch's fill kernel: stores only), the reference point for what the write stream of
     this chip reaches at that size."""
@@ -404,6 +423,8 @@ def nf4_dequant_block(dev, shape=(14336, 4096), fill: bool = False) -> dict:
            "op_ms_from_python": round(t_op, 4), "bytes_per_launch": nbytes, "shape": [rows, cols],
            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "nf4_dequant_kernel"}}
+    if cpu:
+        res["cpu_baseline"] = nf4_cpu_baseline(packed, qs, (rows, cols), nbytes)
     if fill:
         t_f = graph_time_ms(lambda: out.fill_(1.0), 100)
         res["plain_fill_of_the_output"] = {"launch_ms": round(t_f, 4), "GB/s": round(2 * n / (t_f * 1e-3) / 1e9, 1),
@@ -748,7 +769,7 @@ def main():
         "raw_ops_explicit_mask": {"ms_per_step": raw["ms_per_step"], "TFLOP/s": raw["value"], "linears": raw["linears"]},
     }
     if not args.no_extras:
-        res["nf4_dequant"] = nf4_dequant_block(dev)
+        res["nf4_dequant"] = nf4_dequant_block(dev, cpu=not args.no_cpu_baseline)
         res["norm_act"] = norm_act_block(dev)
         small = argparse.Namespace(steps=max(5, args.steps // 2), warmup=max(2, args.warmup // 2))
         res["workloads"] = {name: raw_workload(name, args if name == "c2" else small, dev)
